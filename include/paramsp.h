@@ -1,0 +1,148 @@
+/*
+ * libparamsp_hip.so -- C ABI of the MI355X (gfx950, wave64) ParamSpMM / ParamSDDMM hot path.
+ *
+ * Plain pointers and sizes only: no torch types, no C++ in the signatures.  Every `const float*` /
+ * `const int*` marked DEVICE must point to GPU memory valid on the stream's device; HOST pointers are
+ * ordinary CPU memory.  `stream` is a hipStream_t passed as void* (NULL = the default stream).  Device
+ * entry points only enqueue work; they never synchronise and never allocate.
+ *
+ * Every function returns 0 on success or a negative psp_status; psp_last_error() gives the text of the
+ * last failure on the calling thread.  Nothing here calls exit() (the reference's launchers do on a launch
+ * error, SpMM/SpMM_kernel.cu:189-194).
+ *
+ * Each declaration cites the interface of zzzlxhhh/ParamSpMM_AE it stands in for.  The three PyTorch
+ * extension modules ParamSpMM / ParamSDDMM / ParamSpCONV (pybind, same names and argument order as the
+ * reference's bindings) are thin glue over this header.
+ */
+#ifndef PARAMSP_H
+#define PARAMSP_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *psp_stream_t; /* hipStream_t */
+
+enum psp_status {
+    PSP_OK = 0,
+    PSP_ERR_ARG = -1,    /* bad argument (null pointer, negative size, CF / blkWarpNum out of range) */
+    PSP_ERR_LAUNCH = -2, /* hipGetLastError() after the launch was not hipSuccess */
+    PSP_ERR_RANGE = -3   /* sizes exceed what the 32-bit index arithmetic of the kernels can address */
+};
+
+const char *psp_last_error(void);
+int psp_version(void);
+
+/* How a (N, CF, blkWarpNum) request of the Python layer maps onto the wave64 kernels.
+ * CF keeps its meaning "column coarsening": the number of `vec`-wide column vectors one lane owns;
+ * blkWarpNum keeps its meaning "wavefronts per workgroup" (4 or 8, SpMM/SpMM.cpp:77-141). */
+typedef struct psp_spmm_plan {
+    int vec;            /* floats per feature load: 4 (N%4==0), 2 (N%2==0) or 1 */
+    int coarsen;        /* column vectors per lane (the request's CF, 1..8) */
+    int lanes_per_row;  /* power of two, 1..64: lanes that share one sparse row */
+    int rows_per_wave;  /* 64 / lanes_per_row */
+    int unroll;         /* non-zeros whose feature loads are in flight together per lane */
+    int col_tiles;      /* grid.y: ceil(N / (lanes_per_row*coarsen*vec)) */
+    int waves_per_block;
+} psp_spmm_plan;
+int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan);
+
+/* ---------------------------------------------------------------------------------------------
+ * HOST: PCSR index construction
+ * ------------------------------------------------------------------------------------------- */
+
+/* Row splitting, SpMM/SpMM.cpp:15-40 (`split_csr`).  Row i with [lb,hb) becomes ceil((hb-lb)/g) segments
+ * of at most g non-zeros.  psp_split_csr_count returns S; psp_split_csr fills rowPtr_split[S+1] and
+ * target_row[S] and returns S. */
+int psp_split_csr_count(const int *rowPtr, int nrows, int g);
+int psp_split_csr(const int *rowPtr, int nrows, int g, int *rowPtr_split, int *target_row);
+
+/* SpMM/SpMM.cpp:42-75 (`split_csr_par`): same output; the caller supplies the exclusive prefix sum of the
+ * per-row segment counts (graph_input.py:135-136); rows are processed by several host threads.
+ * Returns S = row_split_offset[nrows]. */
+int psp_split_csr_par(const int *rowPtr, const int *row_split_offset, int nrows, int g,
+                      int *rowPtr_split, int *target_row);
+
+/* BCSR with 2x1 blocks in SciPy `tobsr` order (graph_input.py:243-266 calls csr.tobsr(blocksize=(2,1))):
+ * inside block-row t the blocks appear in first-encounter order, row 2t's columns first, then the columns
+ * only row 2t+1 has.  nrows may be odd (the missing row is empty, graph_input.py:248-255).
+ * psp_bcsr_count returns nblk; psp_bcsr_build fills rowPtr_b[(nrows+1)/2+1], colIdx_b[nblk],
+ * val_b[nblk*2] and returns nblk. */
+int psp_bcsr_count(const int *rowPtr, const int *colIdx, int nrows, int ncols);
+int psp_bcsr_build(const int *rowPtr, const int *colIdx, const float *val, int nrows, int ncols,
+                   int *rowPtr_b, int *colIdx_b, float *val_b);
+
+/* ---------------------------------------------------------------------------------------------
+ * DEVICE: genmask, SDDMM/sddmm.cpp:663-673 -> sddmm_kernel.cu:78-141.
+ * mask[nnz] (int32) is fully written: CSR slot -> flat index into val_b of the same non-zero.
+ * rowPtr must hold at least 2*nblkrows entries (+1 when the row count is even).
+ * ------------------------------------------------------------------------------------------- */
+int psp_genmask(const int *rowPtr_b, const int *rowPtr, const float *val_b, int nblkrows, int nnz,
+                int *mask, psp_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * DEVICE: SpMM  Y = A * X, fp32.  X is [*, N] row-major with leading dimension N; Y is
+ * [rows_out, N] and is completely defined on return (rows the matrix does not cover are zero), so the
+ * caller passes uninitialised memory -- the reference allocates zeros and then launches
+ * (SpMM/SpMM_kernel.cu:136, 281-282).
+ * ------------------------------------------------------------------------------------------- */
+
+/* ParamSpMM.csr_spmm, SpMM/SpMM.cpp:77-141 -> SpMM_kernel.cu:129-197, 1157-1243.  M = rows of A. */
+int psp_spmm_csr_f32(const int *rowPtr, const int *colIdx, const float *val, const float *X, float *Y,
+                     int M, int N, int rows_out, int CF, int blkWarpNum, psp_stream_t stream);
+
+/* ParamSpMM.csr_split_spmm, SpMM/SpMM.cpp:143-207 -> SpMM_kernel.cu:199-268, 1245-1360.
+ * S = number of segments.  Rows made of one segment are stored, rows made of several are accumulated
+ * with fp32 atomics (order not fixed, as in the reference). */
+int psp_spmm_csr_split_f32(const int *rowPtr_split, const int *colIdx, const float *val,
+                           const int *target_row, const float *X, float *Y, int S, int N, int rows_out,
+                           int CF, int blkWarpNum, psp_stream_t stream);
+
+/* ParamSpMM.bcsr_spmm, SpMM/SpMM.cpp:209-271 -> SpMM_kernel.cu:273-343, 1362-1493.
+ * Mb block-rows; val_b is [nblk,2]; rows_out >= 2*Mb.  A zero block entry contributes nothing. */
+int psp_spmm_bcsr_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *X,
+                      float *Y, int Mb, int N, int rows_out, int CF, int blkWarpNum, psp_stream_t stream);
+
+/* ParamSpMM.bcsr_split_spmm, SpMM/SpMM.cpp:273-337 -> SpMM_kernel.cu:345-420, 1495-1651.
+ * target_row holds block-row indices. */
+int psp_spmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b,
+                            const int *target_row, const float *X, float *Y, int Sb, int N, int rows_out,
+                            int CF, int blkWarpNum, psp_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * DEVICE: SDDMM  out[p] = <A[row(p),:], B[col(p),:]>, fp32, NOT scaled by the stored values (the reference
+ * kernels never multiply them in, SDDMM/sddmm_kernel.cu:917-983).  A and B are [*, K] row-major.
+ * `scale` may be NULL; when given (an extension of this library used by the attention benchmark) the result
+ * is multiplied by scale[p] (csr) -- pass NULL for the reference semantics.
+ * ------------------------------------------------------------------------------------------- */
+
+/* ParamSDDMM.csr_sddmm, SDDMM/sddmm.cpp:15-65 -> sddmm_kernel.cu:143-192, 917-983.  out[nnz]. */
+int psp_sddmm_csr_f32(const int *rowPtr, const int *colIdx, const float *A, const float *B,
+                      const float *scale, float *out, int M, int K, int blkWarpNum, psp_stream_t stream);
+
+/* ParamSDDMM.csr_split_sddmm, SDDMM/sddmm.cpp:67-120 -> sddmm_kernel.cu:194-246, 986-1057. */
+int psp_sddmm_csr_split_f32(const int *rowPtr_split, const int *colIdx, const int *target_row,
+                            const float *A, const float *B, const float *scale, float *out, int S, int K,
+                            int blkWarpNum, psp_stream_t stream);
+
+/* ParamSDDMM.bcsr_sddmm, SDDMM/sddmm.cpp:122-172 -> sddmm_kernel.cu:248-300, 1059-1176.
+ * out is [nblk,2]; entries whose block value is zero are written as zero.  A needs 2*Mb rows. */
+int psp_sddmm_bcsr_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *A,
+                       const float *B, float *out, int Mb, int K, int blkWarpNum, psp_stream_t stream);
+
+/* ParamSDDMM.bcsr_split_sddmm, SDDMM/sddmm.cpp:174-228 -> sddmm_kernel.cu:302-352, 1178-1287. */
+int psp_sddmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b,
+                             const int *target_row, const float *A, const float *B, float *out, int Sb,
+                             int K, int blkWarpNum, psp_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * DEVICE: softmax over the stored entries of every CSR row (out[p] = exp(e[p]-max_r) / sum_r).
+ * No counterpart in the reference (its AGNN layer applies no softmax, gnn_conv.py:136-142); it exists for
+ * the SDDMM -> softmax -> SpMM attention pipeline.  in and out may alias.
+ * ------------------------------------------------------------------------------------------- */
+int psp_segment_softmax_f32(const int *rowPtr, const float *in, float *out, int M, psp_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PARAMSP_H */

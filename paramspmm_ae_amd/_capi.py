@@ -1,0 +1,91 @@
+"""ctypes view of libparamsp_hip.so (the C ABI declared in include/paramsp.h).
+
+Used by the host-side format builder (row split, BCSR) and by tests / benchmarks that want to drive the
+kernels without the PyTorch extension modules.  There is no fallback: if the library has not been built
+the import of this module raises.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libparamsp_hip.so")
+
+if not os.path.exists(LIB_PATH):
+    raise ImportError(
+        "libparamsp_hip.so is not built: run `make -C %s` (or script/build_param.sh) first" % os.path.join(_HERE, "csrc")
+    )
+
+lib = ctypes.CDLL(LIB_PATH)
+
+_vp = ctypes.c_void_p
+_i = ctypes.c_int
+
+
+class SpmmPlan(ctypes.Structure):
+    _fields_ = [
+        ("vec", _i),
+        ("coarsen", _i),
+        ("lanes_per_row", _i),
+        ("rows_per_wave", _i),
+        ("unroll", _i),
+        ("col_tiles", _i),
+        ("waves_per_block", _i),
+    ]
+
+    def as_dict(self):
+        return {k: getattr(self, k) for k, _ in self._fields_}
+
+
+# name -> argtypes; every entry returns int.  Keep in step with include/paramsp.h.
+SIGNATURES = {
+    "psp_version": [],
+    "psp_spmm_plan_for": [_i, _i, _i, ctypes.POINTER(SpmmPlan)],
+    "psp_split_csr_count": [_vp, _i, _i],
+    "psp_split_csr": [_vp, _i, _i, _vp, _vp],
+    "psp_split_csr_par": [_vp, _vp, _i, _i, _vp, _vp],
+    "psp_bcsr_count": [_vp, _vp, _i, _i],
+    "psp_bcsr_build": [_vp, _vp, _vp, _i, _i, _vp, _vp, _vp],
+    "psp_genmask": [_vp, _vp, _vp, _i, _i, _vp, _vp],
+    "psp_spmm_csr_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "psp_spmm_csr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "psp_spmm_bcsr_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "psp_spmm_bcsr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "psp_sddmm_csr_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "psp_sddmm_csr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "psp_sddmm_bcsr_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "psp_sddmm_bcsr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "psp_segment_softmax_f32": [_vp, _vp, _vp, _i, _vp],
+}
+
+for _name, _args in SIGNATURES.items():
+    _fn = getattr(lib, _name)
+    _fn.argtypes = _args
+    _fn.restype = _i
+lib.psp_last_error.argtypes = []
+lib.psp_last_error.restype = ctypes.c_char_p
+
+
+class ParamSpError(RuntimeError):
+    pass
+
+
+def check(rc):
+    """Raise on a negative status; pass counts through."""
+    if rc < 0:
+        raise ParamSpError("libparamsp_hip: %s (status %d)" % (lib.psp_last_error().decode(), rc))
+    return rc
+
+
+def spmm_plan(N, CF, blkWarpNum):
+    p = SpmmPlan()
+    check(lib.psp_spmm_plan_for(N, CF, blkWarpNum, ctypes.byref(p)))
+    return p.as_dict()
+
+
+def ptr(t):
+    """Address of a torch tensor's / numpy array's first element (None -> NULL)."""
+    if t is None:
+        return None
+    if hasattr(t, "data_ptr"):
+        return t.data_ptr()
+    return t.ctypes.data

@@ -1,0 +1,352 @@
+// extern "C" surface of libparamsp_hip.so (declared in include/paramsp.h), the small utility kernels
+// (zero fill, genmask, segment softmax) and the host-side PCSR index construction.
+#include <algorithm>
+#include <thread>
+#include <vector>
+#include <string.h>
+#include "psp_common.h"
+#include "spmm_kernel.h"
+#include "sddmm_kernel.h"
+
+// ------------------------------------------------------------------------------------------------
+// errors
+// ------------------------------------------------------------------------------------------------
+static thread_local char g_err[512] = "";
+
+int psp_fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+PSP_EXPORT const char *psp_last_error(void) { return g_err; }
+PSP_EXPORT int psp_version(void) { return 100; }
+
+// ------------------------------------------------------------------------------------------------
+// (N, CF, blkWarpNum) -> wave64 launch plan
+// ------------------------------------------------------------------------------------------------
+PSP_EXPORT int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan)
+{
+    PSP_REQUIRE(plan != nullptr, "plan is null");
+    PSP_REQUIRE(N >= 1, "feature dimension must be positive (got %d)", N);
+    PSP_REQUIRE(CF >= 1 && CF <= 8, "CF must be 1..8 (got %d)", CF);
+    PSP_REQUIRE(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8 (got %d)", blkWarpNum);
+    const int V = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
+    const int nvec = N / V;
+    int C = std::min(CF, nvec);
+    int L = 1;
+    while (L < PSP_WAVE && L * C < nvec) L <<= 1;
+    // in-flight budget: about 8 feature vectors per lane
+    int U = C == 1 ? 8 : C == 2 ? 4 : C <= 4 ? 2 : 1;
+    while (U > L) U >>= 1;
+    plan->vec = V;
+    plan->coarsen = C;
+    plan->lanes_per_row = L;
+    plan->rows_per_wave = PSP_WAVE / L;
+    plan->unroll = U;
+    plan->col_tiles = psp_ceil_div(nvec, L * C);
+    plan->waves_per_block = blkWarpNum;
+    return PSP_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// zero fill
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) psp_zero_kernel(float *__restrict__ p, size_t n)
+{
+    // n4 float4 stores from a 16-byte aligned start, scalar head and tail
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * blockDim.x;
+    const size_t head = std::min<size_t>(n, (size_t)((16 - ((uintptr_t)p & 15)) & 15) / 4);
+    float *q = p + head;
+    const size_t n4 = (n - head) / 4;
+    psp_f32x4 z = {0.f, 0.f, 0.f, 0.f};
+    for (size_t i = tid; i < n4; i += stride) ((psp_f32x4 *)q)[i] = z;
+    if (tid < head) p[tid] = 0.f;
+    const size_t tail0 = head + n4 * 4;
+    if (tid < n - tail0) p[tail0 + tid] = 0.f;
+}
+
+int psp_zero_f32(float *p, size_t n, hipStream_t stream)
+{
+    if (n == 0) return PSP_OK;
+    const size_t want = (n / 4 + 255) / 256 + 1;
+    const int blocks = (int)std::min<size_t>(want, 256 * 32);
+    hipLaunchKernelGGL(psp_zero_kernel, dim3(blocks), dim3(256), 0, stream, p, n);
+    return psp_check_launch("zero fill");
+}
+
+// ------------------------------------------------------------------------------------------------
+// genmask (SDDMM/sddmm_kernel.cu:78-141): one lane per block-row walks its blocks in storage order
+// ------------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+psp_genmask_kernel(const int *__restrict__ rowPtr_b, const int *__restrict__ rowPtr,
+                   const float *__restrict__ val_b, int *__restrict__ mask, int nblkrows)
+{
+    const int t = blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= nblkrows) return;
+    const int lb = rowPtr_b[t], hb = rowPtr_b[t + 1];
+    if (lb == hb) return;
+    int cnt0 = rowPtr[2 * t], cnt1 = rowPtr[2 * t + 1];
+    for (int i = lb; i < hb; i++) {
+        const psp_f32x2 v = ((const psp_f32x2 *)val_b)[i];
+        if (v[0] != 0.0f) mask[cnt0++] = 2 * i;
+        if (v[1] != 0.0f) mask[cnt1++] = 2 * i + 1;
+    }
+}
+
+PSP_EXPORT int psp_genmask(const int *rowPtr_b, const int *rowPtr, const float *val_b, int nblkrows, int nnz,
+                           int *mask, psp_stream_t stream)
+{
+    PSP_REQUIRE(nblkrows >= 0 && nnz >= 0, "genmask: negative size");
+    if (nnz == 0 || nblkrows == 0) return PSP_OK;
+    PSP_REQUIRE(rowPtr_b && rowPtr && val_b && mask, "genmask: null pointer");
+    // slots no non-zero block entry maps to stay zero, as in the reference (mask = zeros, sddmm_kernel.cu:126)
+    int rc = psp_zero_f32((float *)mask, (size_t)nnz, (hipStream_t)stream);
+    if (rc != PSP_OK) return rc;
+    hipLaunchKernelGGL(psp_genmask_kernel, dim3(psp_ceil_div(nblkrows, 256)), dim3(256), 0, (hipStream_t)stream,
+                       rowPtr_b, rowPtr, val_b, mask, nblkrows);
+    return psp_check_launch("genmask kernel");
+}
+
+// ------------------------------------------------------------------------------------------------
+// segment softmax: 16 lanes per row, three sweeps over the row (max, sum, write); rows of up to 16
+// entries never re-read memory
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ float psp_max16(float v)
+{
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), 0xB1, 0xF, 0xF, false)));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), 0x4E, 0xF, 0xF, false)));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), 0x141, 0xF, 0xF, false)));
+    v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), 0x140, 0xF, 0xF, false)));
+    return v;
+}
+
+__global__ void __launch_bounds__(256)
+psp_segment_softmax_kernel(const int *__restrict__ rowPtr, const float *in, float *out, int M)
+{
+    const int row = (blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+    const int sub = threadIdx.x & 15;
+    int lb = 0, hb = 0;
+    if (row < M) {
+        lb = rowPtr[row];
+        hb = rowPtr[row + 1];
+    }
+    if (lb == hb) return;  // whole 16-lane group leaves together
+    const float NEG = -3.402823466e+38f;
+    const float first = (lb + sub < hb) ? in[lb + sub] : NEG;
+    float mx = first;
+    for (int p = lb + 16 + sub; p < hb; p += 16) mx = fmaxf(mx, in[p]);
+    mx = psp_max16(mx);
+    float s = (lb + sub < hb) ? __expf(first - mx) : 0.0f;
+    for (int p = lb + 16 + sub; p < hb; p += 16) s += __expf(in[p] - mx);
+    s = psp_group_sum<4>(s);
+    const float inv = 1.0f / s;
+    // all reads of a chunk happen before its writes, so in == out is fine
+    float e0 = __expf(first - mx) * inv;
+    for (int p = lb + 16 + sub; p < hb; p += 16) out[p] = __expf(in[p] - mx) * inv;
+    if (lb + sub < hb) out[lb + sub] = e0;
+}
+
+PSP_EXPORT int psp_segment_softmax_f32(const int *rowPtr, const float *in, float *out, int M, psp_stream_t stream)
+{
+    PSP_REQUIRE(M >= 0, "segment_softmax: negative row count");
+    if (M == 0) return PSP_OK;
+    PSP_REQUIRE(rowPtr && in && out, "segment_softmax: null pointer");
+    hipLaunchKernelGGL(psp_segment_softmax_kernel, dim3(psp_ceil_div((long long)M * 16, 256)), dim3(256), 0,
+                       (hipStream_t)stream, rowPtr, in, out, M);
+    return psp_check_launch("segment softmax kernel");
+}
+
+// ------------------------------------------------------------------------------------------------
+// host: row split (SpMM/SpMM.cpp:15-75)
+// ------------------------------------------------------------------------------------------------
+PSP_EXPORT int psp_split_csr_count(const int *rowPtr, int nrows, int g)
+{
+    PSP_REQUIRE(rowPtr && nrows >= 0, "split_csr: bad rowPtr / nrows");
+    PSP_REQUIRE(g >= 1, "split_csr: granularity must be positive (got %d)", g);
+    long long S = 0;
+    for (int i = 0; i < nrows; i++) {
+        const int k = rowPtr[i + 1] - rowPtr[i];
+        PSP_REQUIRE(k >= 0, "split_csr: rowPtr decreases at row %d", i);
+        S += (k + g - 1) / g;
+    }
+    if (S > 0x7fffffffLL) return psp_fail(PSP_ERR_RANGE, "split_csr: %lld segments do not fit int32", S);
+    return (int)S;
+}
+
+static void split_rows(const int *rowPtr, int r0, int r1, int g, int off, int *rowPtr_split, int *target_row)
+{
+    for (int i = r0; i < r1; i++) {
+        const int hb = rowPtr[i + 1];
+        for (int lb = rowPtr[i]; lb < hb; lb += g) {
+            target_row[off] = i;
+            rowPtr_split[off + 1] = std::min(lb + g, hb);
+            off++;
+        }
+    }
+}
+
+PSP_EXPORT int psp_split_csr(const int *rowPtr, int nrows, int g, int *rowPtr_split, int *target_row)
+{
+    const int S = psp_split_csr_count(rowPtr, nrows, g);
+    if (S < 0) return S;
+    PSP_REQUIRE(rowPtr_split && (target_row || S == 0), "split_csr: null output");
+    rowPtr_split[0] = 0;
+    split_rows(rowPtr, 0, nrows, g, 0, rowPtr_split, target_row);
+    return S;
+}
+
+PSP_EXPORT int psp_split_csr_par(const int *rowPtr, const int *row_split_offset, int nrows, int g,
+                                 int *rowPtr_split, int *target_row)
+{
+    PSP_REQUIRE(rowPtr && row_split_offset && nrows >= 0, "split_csr_par: bad input");
+    PSP_REQUIRE(g >= 1, "split_csr_par: granularity must be positive (got %d)", g);
+    const int S = row_split_offset[nrows];
+    PSP_REQUIRE(S >= 0 && rowPtr_split && (target_row || S == 0), "split_csr_par: bad output");
+    // the offsets must be the exclusive prefix of ceil(nnz_i / g): rows write disjoint ranges only then
+    for (int i = 0; i < nrows; i++) {
+        const int k = rowPtr[i + 1] - rowPtr[i];
+        PSP_REQUIRE(k >= 0 && row_split_offset[i + 1] - row_split_offset[i] == (k + g - 1) / g,
+                    "split_csr_par: row_split_offset is not the prefix sum of ceil(nnz/g) at row %d", i);
+    }
+    rowPtr_split[0] = 0;
+    unsigned hw = std::thread::hardware_concurrency();
+    int nthreads = (int)std::min<unsigned>(hw ? hw : 1, 16);
+    if (nrows < (1 << 16)) nthreads = 1;
+    if (nthreads <= 1) {
+        split_rows(rowPtr, 0, nrows, g, 0, rowPtr_split, target_row);
+        return S;
+    }
+    std::vector<std::thread> pool;
+    const int per = (nrows + nthreads - 1) / nthreads;
+    for (int t = 0; t < nthreads; t++) {
+        const int r0 = std::min(nrows, t * per), r1 = std::min(nrows, r0 + per);
+        if (r0 == r1) continue;
+        pool.emplace_back(split_rows, rowPtr, r0, r1, g, row_split_offset[r0], rowPtr_split, target_row);
+    }
+    for (auto &th : pool) th.join();
+    return S;
+}
+
+// ------------------------------------------------------------------------------------------------
+// host: BCSR 2x1 in first-encounter block order (what SciPy's tobsr produces, graph_input.py:245-256)
+// ------------------------------------------------------------------------------------------------
+static int bcsr_walk(const int *rowPtr, const int *colIdx, const float *val, int nrows, int ncols,
+                     int *rowPtr_b, int *colIdx_b, float *val_b)
+{
+    const int nbr = (nrows + 1) / 2;
+    std::vector<int> slot((size_t)std::max(ncols, 1), -1);
+    long long nblk = 0;
+    if (rowPtr_b) rowPtr_b[0] = 0;
+    for (int t = 0; t < nbr; t++) {
+        const long long first = nblk;
+        for (int k = 0; k < 2; k++) {
+            const int r = 2 * t + k;
+            if (r >= nrows) break;
+            for (int p = rowPtr[r]; p < rowPtr[r + 1]; p++) {
+                const int c = colIdx[p];
+                if (c < 0 || c >= ncols) return psp_fail(PSP_ERR_ARG, "bcsr: column %d out of range at entry %d", c, p);
+                if (slot[c] < first) {
+                    if (nblk >= 0x7fffffffLL) return psp_fail(PSP_ERR_RANGE, "bcsr: block count overflows int32");
+                    slot[c] = (int)nblk;
+                    if (colIdx_b) {
+                        colIdx_b[nblk] = c;
+                        val_b[2 * nblk] = 0.0f;
+                        val_b[2 * nblk + 1] = 0.0f;
+                    }
+                    nblk++;
+                }
+                if (colIdx_b) val_b[2 * (size_t)slot[c] + k] += val[p];
+            }
+        }
+        if (rowPtr_b) rowPtr_b[t + 1] = (int)nblk;
+    }
+    return (int)nblk;
+}
+
+PSP_EXPORT int psp_bcsr_count(const int *rowPtr, const int *colIdx, int nrows, int ncols)
+{
+    PSP_REQUIRE(rowPtr && nrows >= 0 && ncols >= 0, "bcsr_count: bad input");
+    PSP_REQUIRE(colIdx || rowPtr[nrows] == 0, "bcsr_count: colIdx is null");
+    return bcsr_walk(rowPtr, colIdx, nullptr, nrows, ncols, nullptr, nullptr, nullptr);
+}
+
+PSP_EXPORT int psp_bcsr_build(const int *rowPtr, const int *colIdx, const float *val, int nrows, int ncols,
+                              int *rowPtr_b, int *colIdx_b, float *val_b)
+{
+    PSP_REQUIRE(rowPtr && nrows >= 0 && ncols >= 0 && rowPtr_b, "bcsr_build: bad input");
+    const bool empty = rowPtr[nrows] == 0;
+    PSP_REQUIRE(empty || (colIdx && val && colIdx_b && val_b), "bcsr_build: null pointer");
+    if (empty) {
+        for (int t = 0; t <= (nrows + 1) / 2; t++) rowPtr_b[t] = 0;
+        return 0;
+    }
+    return bcsr_walk(rowPtr, colIdx, val, nrows, ncols, rowPtr_b, colIdx_b, val_b);
+}
+
+// ------------------------------------------------------------------------------------------------
+// device entry points
+// ------------------------------------------------------------------------------------------------
+PSP_EXPORT int psp_spmm_csr_f32(const int *rowPtr, const int *colIdx, const float *val, const float *X, float *Y,
+                                int M, int N, int rows_out, int CF, int blkWarpNum, psp_stream_t stream)
+{
+    return psp_spmm_launch<false, false>(rowPtr, colIdx, val, nullptr, X, Y, M, N, rows_out, CF, blkWarpNum,
+                                         (hipStream_t)stream);
+}
+
+PSP_EXPORT int psp_spmm_csr_split_f32(const int *rowPtr_split, const int *colIdx, const float *val,
+                                      const int *target_row, const float *X, float *Y, int S, int N, int rows_out,
+                                      int CF, int blkWarpNum, psp_stream_t stream)
+{
+    return psp_spmm_launch<false, true>(rowPtr_split, colIdx, val, target_row, X, Y, S, N, rows_out, CF, blkWarpNum,
+                                        (hipStream_t)stream);
+}
+
+PSP_EXPORT int psp_spmm_bcsr_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *X,
+                                 float *Y, int Mb, int N, int rows_out, int CF, int blkWarpNum, psp_stream_t stream)
+{
+    return psp_spmm_launch<true, false>(rowPtr_b, colIdx_b, val_b, nullptr, X, Y, Mb, N, rows_out, CF, blkWarpNum,
+                                        (hipStream_t)stream);
+}
+
+PSP_EXPORT int psp_spmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b,
+                                       const int *target_row, const float *X, float *Y, int Sb, int N,
+                                       int rows_out, int CF, int blkWarpNum, psp_stream_t stream)
+{
+    return psp_spmm_launch<true, true>(rowPtr_bs, colIdx_b, val_b, target_row, X, Y, Sb, N, rows_out, CF, blkWarpNum,
+                                       (hipStream_t)stream);
+}
+
+PSP_EXPORT int psp_sddmm_csr_f32(const int *rowPtr, const int *colIdx, const float *A, const float *B,
+                                 const float *scale, float *out, int M, int K, int blkWarpNum, psp_stream_t stream)
+{
+    return psp_sddmm_launch<false, false>(rowPtr, colIdx, nullptr, nullptr, A, B, scale, out, M, K, blkWarpNum,
+                                          (hipStream_t)stream);
+}
+
+PSP_EXPORT int psp_sddmm_csr_split_f32(const int *rowPtr_split, const int *colIdx, const int *target_row,
+                                       const float *A, const float *B, const float *scale, float *out, int S,
+                                       int K, int blkWarpNum, psp_stream_t stream)
+{
+    return psp_sddmm_launch<false, true>(rowPtr_split, colIdx, nullptr, target_row, A, B, scale, out, S, K,
+                                         blkWarpNum, (hipStream_t)stream);
+}
+
+PSP_EXPORT int psp_sddmm_bcsr_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *A,
+                                  const float *B, float *out, int Mb, int K, int blkWarpNum, psp_stream_t stream)
+{
+    return psp_sddmm_launch<true, false>(rowPtr_b, colIdx_b, val_b, nullptr, A, B, nullptr, out, Mb, K, blkWarpNum,
+                                         (hipStream_t)stream);
+}
+
+PSP_EXPORT int psp_sddmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b,
+                                        const int *target_row, const float *A, const float *B, float *out, int Sb,
+                                        int K, int blkWarpNum, psp_stream_t stream)
+{
+    return psp_sddmm_launch<true, true>(rowPtr_bs, colIdx_b, val_b, target_row, A, B, nullptr, out, Sb, K,
+                                        blkWarpNum, (hipStream_t)stream);
+}

@@ -1,0 +1,170 @@
+// Parameterised SDDMM kernel for gfx950 (wave64): out[p] = <A[row(p),:], B[col(p),:]> for every stored
+// entry p.  Semantics follow SDDMM/sddmm_kernel.cu:917-1287 (the stored values never scale the result; for
+// 2x1 blocks they only decide which of the two entries is computed).
+//
+// A sparse row is owned by L = 2^LOGL lanes; each lane keeps C vectors of V floats of the A row in
+// registers and loads the matching part of the B row, so a group reads L*V*4 contiguous bytes per load.
+// The per-lane partial dot products are summed across the group with DPP / ds_swizzle butterflies.  The L
+// results of one chunk of L non-zeros are parked one per lane and written with a single coalesced store
+// (the reference stores one float per warp per non-zero).
+#pragma once
+#include "psp_common.h"
+#include "spmm_kernel.h"  // psp_vec
+
+// Sum over aligned groups of 2^LOGL lanes; every lane of the group receives the total.
+template <int LOGL> __device__ __forceinline__ float psp_group_sum(float v)
+{
+    if constexpr (LOGL >= 1)  // lane ^ 1
+        v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));
+    if constexpr (LOGL >= 2)  // lane ^ 2
+        v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));
+    if constexpr (LOGL >= 3)  // mirror inside 8 lanes: the partner sits in the other quad
+        v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));
+    if constexpr (LOGL >= 4)  // mirror inside 16 lanes
+        v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));
+    if constexpr (LOGL >= 5)  // lane ^ 16 inside 32 lanes
+        v += __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F));
+    if constexpr (LOGL >= 6)  // lane ^ 32
+        v += __int_as_float(__builtin_amdgcn_ds_bpermute((int)((threadIdx.x ^ 32) & 63) << 2, __float_as_int(v)));
+    return v;
+}
+
+// val: bcsr -> [nblk,2] block values (gate); csr -> optional per-entry scale (may be null when !SCALE)
+template <int LOGL, int C, int V, int U, bool BCSR, bool SPLIT, bool SCALE>
+__global__ void __launch_bounds__(512)
+psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
+                 const int *__restrict__ target_row, const float *__restrict__ A, const float *__restrict__ B,
+                 float *__restrict__ out, int nrows, int K, int tiles, int chunk)
+{
+    typedef typename psp_vec<V>::type vec_t;
+    constexpr int NR = BCSR ? 2 : 1;
+    constexpr int L = 1 << LOGL;
+    static_assert(U <= L, "unroll must not exceed the group width");
+
+    const int tile = psp_xcd_tile(chunk);
+    if (tile >= tiles) return;
+
+    const int lane = threadIdx.x & (PSP_WAVE - 1);
+    const int wave = threadIdx.x >> 6;
+    const int sub = lane & (L - 1);
+    const int grp_base = lane - sub;
+    const int row = ((tile * (int)(blockDim.x >> 6) + wave) << (6 - LOGL)) + (lane >> LOGL);
+
+    int lb = 0, hb = 0;
+    if (row < nrows) {
+        lb = rowPtr[row];
+        hb = rowPtr[row + 1];
+    }
+
+    int off[C];
+    bool live[C];
+#pragma unroll
+    for (int i = 0; i < C; i++) {
+        const int col = ((i << LOGL) + sub) * V;
+        live[i] = col < K;
+        off[i] = live[i] ? col : K - V;
+    }
+
+    // the A row(s) of this group; dead tail vectors are zero so they add nothing to the dot product
+    float a[NR][C][V];
+    {
+        const int arow = (SPLIT && lb < hb) ? target_row[row] : row;
+#pragma unroll
+        for (int r = 0; r < NR; r++)
+#pragma unroll
+            for (int i = 0; i < C; i++) {
+                vec_t t;
+                if constexpr (V == 1) t = 0.0f;
+                else {
+#pragma unroll
+                    for (int e = 0; e < V; e++) t[e] = 0.0f;
+                }
+                if (lb < hb && live[i]) t = *(const vec_t *)(A + (size_t)(arow * NR + r) * (size_t)K + off[i]);
+#pragma unroll
+                for (int e = 0; e < V; e++) a[r][i][e] = psp_elem<V>(t, e);
+            }
+    }
+
+    for (int base = lb; base < hb; base += L) {
+        const int p = base + sub;
+        const bool ok = p < hb;
+        const int pp = ok ? p : hb - 1;
+        const int c_cur = colIdx[pp];
+        float gate[NR];
+        if constexpr (BCSR) {
+            const psp_f32x2 t = ((const psp_f32x2 *)val)[pp];
+            gate[0] = t[0];
+            gate[1] = t[1];
+        } else {
+            gate[0] = SCALE ? val[pp] : 1.0f;
+        }
+        float res[NR];
+#pragma unroll
+        for (int r = 0; r < NR; r++) res[r] = 0.0f;
+
+        const int cnt = min(L, hb - base);
+        for (int k = 0; k < cnt; k += U) {
+            int ck[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) ck[u] = __builtin_amdgcn_ds_bpermute((grp_base + k + u) << 2, c_cur);
+            vec_t b[U][C];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float *br = B + (size_t)ck[u] * (size_t)K;
+#pragma unroll
+                for (int i = 0; i < C; i++) b[u][i] = *(const vec_t *)(br + off[i]);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int r = 0; r < NR; r++) {
+                    float part = 0.0f;
+#pragma unroll
+                    for (int i = 0; i < C; i++)
+#pragma unroll
+                        for (int e = 0; e < V; e++) part = __builtin_fmaf(a[r][i][e], psp_elem<V>(b[u][i], e), part);
+                    part = psp_group_sum<LOGL>(part);
+                    if (sub == k + u) res[r] = part;
+                }
+        }
+        if (ok) {
+            if constexpr (BCSR) {
+                // entries of a block whose value is zero are padding: written as zero (sddmm_kernel.cu:1103,1115)
+                psp_f32x2 o;
+                o[0] = gate[0] != 0.0f ? res[0] : 0.0f;
+                o[1] = gate[1] != 0.0f ? res[1] : 0.0f;
+                ((psp_f32x2 *)out)[p] = o;
+            } else {
+                out[p] = SCALE ? res[0] * gate[0] : res[0];
+            }
+        }
+    }
+}
+
+typedef void (*psp_sddmm_kernel_t)(const int *, const int *, const float *, const int *, const float *,
+                                   const float *, float *, int, int, int, int);
+
+// (LOGL, C, U) triples that exist.  C grows only once the group is 16 lanes wide (DPP-only reduction);
+// beyond 64 vectors the group widens to 32 and 64 lanes.
+#define PSP_SDDMM_FOR_EACH_LCU(M_) \
+    M_(0, 1, 1) M_(1, 1, 2) M_(2, 1, 4) M_(3, 1, 4) M_(4, 1, 4) \
+    M_(4, 2, 4) M_(4, 3, 2) M_(4, 4, 2) M_(5, 4, 2) M_(6, 4, 2)
+
+template <bool BCSR, bool SPLIT, bool SCALE>
+static psp_sddmm_kernel_t psp_sddmm_lookup(int logL, int C, int V)
+{
+#define PSP_CASE(L_, C_, U_)                                                               \
+    if (logL == L_ && C == C_) {                                                           \
+        if (V == 4) return psp_sddmm_kernel<L_, C_, 4, U_, BCSR, SPLIT, SCALE>;            \
+        if (V == 2) return psp_sddmm_kernel<L_, C_, 2, U_, BCSR, SPLIT, SCALE>;            \
+        return psp_sddmm_kernel<L_, C_, 1, U_, BCSR, SPLIT, SCALE>;                        \
+    }
+    PSP_SDDMM_FOR_EACH_LCU(PSP_CASE)
+#undef PSP_CASE
+    return nullptr;
+}
+
+template <bool BCSR, bool SPLIT>
+int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
+                     const float *A, const float *B, const float *scale, float *out, int nrows, int K,
+                     int blkWarpNum, hipStream_t stream);

@@ -1,0 +1,37 @@
+// Host launcher shared by the four SDDMM translation units.
+#pragma once
+#include "sddmm_kernel.h"
+
+template <bool BCSR, bool SPLIT>
+int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
+                     const float *A, const float *B, const float *scale, float *out, int nrows, int K,
+                     int blkWarpNum, hipStream_t stream)
+{
+    PSP_REQUIRE(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8");
+    PSP_REQUIRE(nrows >= 0 && K >= 1, "sddmm: bad size (rows %d, K %d)", nrows, K);
+    if (nrows == 0) return PSP_OK;
+    PSP_REQUIRE(rowPtr && colIdx && A && B && out, "sddmm: null pointer");
+    PSP_REQUIRE(!SPLIT || target_row, "sddmm: target_row is null");
+    PSP_REQUIRE(!BCSR || val, "sddmm: block values are null");
+    PSP_REQUIRE(!(BCSR && scale), "sddmm: scale is only supported for csr formats");
+
+    const int V = (K % 4 == 0) ? 4 : (K % 2 == 0) ? 2 : 1;
+    const int nvec = K / V;
+    int C = psp_ceil_div(nvec, 16);
+    if (C > 4) C = 4;
+    int logL = 0;
+    while ((C << logL) < nvec) logL++;
+    if (logL > 6) return psp_fail(PSP_ERR_RANGE, "sddmm: K = %d is too wide (max %d for this alignment)", K, 256 * V);
+    if (logL < 4 && C > 1) C = 1;
+
+    psp_sddmm_kernel_t k = scale ? psp_sddmm_lookup<BCSR, SPLIT, !BCSR>(logL, C, V)
+                                 : psp_sddmm_lookup<BCSR, SPLIT, false>(logL, C, V);
+    if (!k) return psp_fail(PSP_ERR_ARG, "sddmm: no kernel for logL %d coarsen %d vec %d", logL, C, V);
+
+    const int rows_per_block = blkWarpNum * (PSP_WAVE >> logL);
+    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, rows_per_block));
+    dim3 grid(g.launch, 1, 1), block(blkWarpNum * PSP_WAVE, 1, 1);
+    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, BCSR ? val : scale, target_row, A, B, out, nrows, K,
+                       g.real, g.chunk);
+    return psp_check_launch("sddmm kernel");
+}

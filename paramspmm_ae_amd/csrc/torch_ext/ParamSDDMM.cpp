@@ -1,0 +1,193 @@
+// Python module `ParamSDDMM`: the binding surface of the reference's SDDMM/sddmm.cpp:675-701, backed by
+// libparamsp_hip.so.
+#include "glue_common.h"
+
+using namespace pspglue;
+using torch::Tensor;
+
+// fmt: 0 csr, 1 csr_split, 2 bcsr, 3 bcsr_split
+static void check_sddmm_args(int fmt, const Tensor &A, const Tensor &B, const Tensor &rowPtr, const Tensor &colIdx,
+                             const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
+{
+    need_gpu(A, "A");
+    need_gpu(B, "B");
+    need_gpu(rowPtr, "rowPtr");
+    need_gpu(colIdx, "colIdx");
+    need_gpu(values, "values");
+    need_f32(A, "A", 2);
+    need_f32(B, "B", 2);
+    need_i32(rowPtr, "rowPtr");
+    need_i32(colIdx, "colIdx");
+    const bool blocked = fmt >= 2;
+    need_f32(values, "values", blocked ? 2 : 1);
+    if (blocked) TORCH_CHECK(values.size(1) == 2, "values of a bcsr format must be [nblk, 2]");
+    TORCH_CHECK(values.size(0) == colIdx.size(0), "values and colIdx disagree on the number of stored entries");
+    TORCH_CHECK(A.size(1) == B.size(1), "A and B must have the same number of columns");
+    TORCH_CHECK(A.size(1) >= 1, "A and B need at least one column");
+    check_rowptr_vs(rowPtr, "rowPtr");
+    same_device(A, B, "sddmm");
+    same_device(A, rowPtr, "sddmm");
+    same_device(A, colIdx, "sddmm");
+    same_device(A, values, "sddmm");
+    // the reference dispatches CF 1..4 only (SDDMM/sddmm.cpp:31-43); wider K is accepted here, CF stays a
+    // checked argument so that a caller's mistake still surfaces
+    TORCH_CHECK(CF >= 1 && CF <= 8, "CF must be 1..8");
+    TORCH_CHECK(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8");
+    const long rows = rowPtr.size(0) - 1;
+    if (target_row) {
+        need_gpu(*target_row, "target_row");
+        need_i32(*target_row, "target_row");
+        same_device(A, *target_row, "sddmm");
+        TORCH_CHECK(target_row->size(0) == rows, "target_row must have one entry per row segment");
+    }
+    if (fmt == 0) TORCH_CHECK(rows <= A.size(0), "rowPtr describes more rows than A has");
+    if (fmt == 2) TORCH_CHECK(2 * rows <= A.size(0), "A needs two rows per block-row (pad it to an even row count)");
+}
+
+static Tensor sddmm_new(int fmt, const Tensor &A, const Tensor &B, const Tensor &rowPtr, const Tensor &colIdx,
+                        const Tensor &values, const Tensor *target_row, const Tensor *scale, int CF, int blkWarpNum)
+{
+    check_sddmm_args(fmt, A, B, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
+    c10::hip::HIPGuard guard(A.device());
+    auto out = torch::empty_like(values);  // every stored entry is written by the kernel
+    const int nrows = (int)rowPtr.size(0) - 1, K = (int)A.size(1);
+    if (values.numel() == 0) return out;
+    psp_stream_t s = stream_of(A);
+    int rc;
+    switch (fmt) {
+    case 0: rc = psp_sddmm_csr_f32(ip(rowPtr), ip(colIdx), fp(A), fp(B), scale ? fp(*scale) : nullptr, fpw(out), nrows, K, blkWarpNum, s); break;
+    case 1: rc = psp_sddmm_csr_split_f32(ip(rowPtr), ip(colIdx), ip(*target_row), fp(A), fp(B), scale ? fp(*scale) : nullptr, fpw(out), nrows, K, blkWarpNum, s); break;
+    case 2: rc = psp_sddmm_bcsr_f32(ip(rowPtr), ip(colIdx), fp(values), fp(A), fp(B), fpw(out), nrows, K, blkWarpNum, s); break;
+    default: rc = psp_sddmm_bcsr_split_f32(ip(rowPtr), ip(colIdx), fp(values), ip(*target_row), fp(A), fp(B), fpw(out), nrows, K, blkWarpNum, s); break;
+    }
+    ok(rc);
+    return out;
+}
+
+static Tensor csr_sddmm(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, int CF, int blkWarpNum)
+{
+    return sddmm_new(0, A, B, rowPtr, colIdx, values, nullptr, nullptr, CF, blkWarpNum);
+}
+static Tensor csr_split_sddmm(Tensor A, Tensor B, Tensor rowPtr_split, Tensor colIdx, Tensor values, Tensor target_row,
+                              int CF, int blkWarpNum)
+{
+    return sddmm_new(1, A, B, rowPtr_split, colIdx, values, &target_row, nullptr, CF, blkWarpNum);
+}
+static Tensor bcsr_sddmm(Tensor A, Tensor B, Tensor rowPtr_bcsr, Tensor colIdx, Tensor values, int CF, int blkWarpNum)
+{
+    return sddmm_new(2, A, B, rowPtr_bcsr, colIdx, values, nullptr, nullptr, CF, blkWarpNum);
+}
+static Tensor bcsr_split_sddmm(Tensor A, Tensor B, Tensor rowPtr_bcsr_split, Tensor colIdx, Tensor values,
+                               Tensor target_row, int CF, int blkWarpNum)
+{
+    return sddmm_new(3, A, B, rowPtr_bcsr_split, colIdx, values, &target_row, nullptr, CF, blkWarpNum);
+}
+
+// out[p] = values[p] * <A[row], B[col]>: the attention-score form (an addition of this build; the reference op
+// never multiplies the stored value in)
+static Tensor csr_sddmm_scaled(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, int blkWarpNum)
+{
+    return sddmm_new(0, A, B, rowPtr, colIdx, values, nullptr, &values, 1, blkWarpNum);
+}
+
+// ---- *_profile twins (SDDMM/sddmm.cpp:338-661): int GFLOP/s = 2*nnz*K / t -------------------------------
+static int profile_impl(int fmt, const Tensor &A, const Tensor &B, const Tensor &rowPtr, const Tensor &colIdx,
+                        const Tensor &values, const Tensor *target_row, long nnz, int CF, int blkWarpNum)
+{
+    check_sddmm_args(fmt, A, B, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
+    c10::hip::HIPGuard guard(A.device());
+    hipStream_t s = (hipStream_t)stream_of(A);
+    const float ms = time_launches(s, kProfileWarmup, kProfileIters, [&] {
+        (void)sddmm_new(fmt, A, B, rowPtr, colIdx, values, target_row, nullptr, CF, blkWarpNum);
+    });
+    return gflops(2.0 * (double)nnz * (double)A.size(1), ms);
+}
+static int csr_sddmm_profile(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, int CF, int blkWarpNum)
+{
+    return profile_impl(0, A, B, rowPtr, colIdx, values, nullptr, values.size(0), CF, blkWarpNum);
+}
+static int csr_split_sddmm_profile(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, Tensor target_row,
+                                   int CF, int blkWarpNum)
+{
+    return profile_impl(1, A, B, rowPtr, colIdx, values, &target_row, values.size(0), CF, blkWarpNum);
+}
+static int bcsr_sddmm_profile(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, int nnz, int CF, int blkWarpNum)
+{
+    return profile_impl(2, A, B, rowPtr, colIdx, values, nullptr, nnz, CF, blkWarpNum);
+}
+static int bcsr_split_sddmm_profile(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, Tensor target_row,
+                                    int nnz, int CF, int blkWarpNum)
+{
+    return profile_impl(3, A, B, rowPtr, colIdx, values, &target_row, nnz, CF, blkWarpNum);
+}
+
+// ---- genmask (SDDMM/sddmm.cpp:663-673) -------------------------------------------------------------------
+static Tensor genmask(Tensor rowPtr_bcsr, Tensor rowPtr, Tensor blkval, int nnz)
+{
+    need_gpu(rowPtr_bcsr, "rowPtr_bcsr");
+    need_gpu(rowPtr, "rowPtr");
+    need_gpu(blkval, "blkval");
+    need_i32(rowPtr_bcsr, "rowPtr_bcsr");
+    need_i32(rowPtr, "rowPtr");
+    need_f32(blkval, "blkval", 2);
+    TORCH_CHECK(blkval.size(1) == 2, "blkval must be [nblk, 2]");
+    TORCH_CHECK(nnz >= 0, "nnz must not be negative");
+    same_device(rowPtr, rowPtr_bcsr, "genmask");
+    same_device(rowPtr, blkval, "genmask");
+    check_rowptr_vs(rowPtr_bcsr, "rowPtr_bcsr");
+    const int nbr = (int)rowPtr_bcsr.size(0) - 1;
+    // block-row t reads rowPtr[2t] and rowPtr[2t+1]
+    TORCH_CHECK(rowPtr.size(0) >= 2L * nbr, "rowPtr is too short for the block row pointer");
+    c10::hip::HIPGuard guard(rowPtr.device());
+    auto mask = torch::empty({(long)nnz}, rowPtr.options());
+    ok(psp_genmask(ip(rowPtr_bcsr), ip(rowPtr), fp(blkval), nbr, nnz, nnz ? mask.data_ptr<int>() : nullptr, stream_of(rowPtr)));
+    return mask;
+}
+
+// ---- row softmax over stored entries (an addition of this build) --------------------------------------
+static Tensor segment_softmax(Tensor rowPtr, Tensor e)
+{
+    need_gpu(rowPtr, "rowPtr");
+    need_gpu(e, "e");
+    need_i32(rowPtr, "rowPtr");
+    need_f32(e, "e", 1);
+    same_device(rowPtr, e, "segment_softmax");
+    check_rowptr_vs(rowPtr, "rowPtr");
+    c10::hip::HIPGuard guard(e.device());
+    auto out = torch::empty_like(e);
+    ok(psp_segment_softmax_f32(ip(rowPtr), fp(e), fpw(out), (int)rowPtr.size(0) - 1, stream_of(e)));
+    return out;
+}
+
+[[noreturn]] static void not_built(const char *what)
+{
+    TORCH_CHECK(false, what, " is not part of this build (only the PCSR operators csr/csr_split/bcsr/bcsr_split are)");
+}
+static Tensor vec_sddmm(Tensor, Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_sddmm (vec_size 3 blocks)"); }
+static Tensor vec_split_sddmm(Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_split_sddmm"); }
+static int vec_sddmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_sddmm_profile"); }
+static int vec_split_sddmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_split_sddmm_profile"); }
+static void cusparse_sddmm_compute(Tensor, Tensor, Tensor, Tensor, Tensor) { not_built("the cuSPARSE SDDMM comparison baseline"); }
+static int cusparse_sddmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor) { not_built("the cuSPARSE SDDMM comparison baseline"); }
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    m.def("csr_sddmm", &csr_sddmm, "CSR SDDMM (HIP, gfx950)");
+    m.def("csr_split_sddmm", &csr_split_sddmm, "row-split CSR SDDMM (HIP, gfx950)");
+    m.def("bcsr_sddmm", &bcsr_sddmm, "2x1 BCSR SDDMM (HIP, gfx950)");
+    m.def("bcsr_split_sddmm", &bcsr_split_sddmm, "row-split 2x1 BCSR SDDMM (HIP, gfx950)");
+    m.def("vec_sddmm", &vec_sddmm, "not built");
+    m.def("vec_split_sddmm", &vec_split_sddmm, "not built");
+    m.def("csr_sddmm_profile", &csr_sddmm_profile, "GFLOP/s of csr_sddmm");
+    m.def("csr_split_sddmm_profile", &csr_split_sddmm_profile, "GFLOP/s of csr_split_sddmm");
+    m.def("bcsr_sddmm_profile", &bcsr_sddmm_profile, "GFLOP/s of bcsr_sddmm");
+    m.def("bcsr_split_sddmm_profile", &bcsr_split_sddmm_profile, "GFLOP/s of bcsr_split_sddmm");
+    m.def("vec_sddmm_profile", &vec_sddmm_profile, "not built");
+    m.def("vec_split_sddmm_profile", &vec_split_sddmm_profile, "not built");
+    m.def("cusparse_sddmm_compute", &cusparse_sddmm_compute, "not built");
+    m.def("cusparse_sddmm_profile", &cusparse_sddmm_profile, "not built");
+    m.def("genmask", &genmask, "CSR slot -> flat index into the 2x1 block values");
+    // additions of this build
+    m.def("csr_sddmm_scaled", &csr_sddmm_scaled, "values[p] * <A[row], B[col]>");
+    m.def("segment_softmax", &segment_softmax, "softmax over the stored entries of each CSR row");
+}

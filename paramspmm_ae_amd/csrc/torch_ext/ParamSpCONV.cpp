@@ -1,0 +1,86 @@
+// Python module `ParamSpCONV`: the fused GCN layer ops of the reference's SpCONV/SpCONV.cpp:496-512
+// (glue in SpCONV/SpCONV.h:43-193): forward A*(H*W), backward [ (A*dY)*W^T, H^T*(A*dY) ].  The dense
+// products are torch::mm (hipBLASLt / rocBLAS under PyTorch-ROCm); the sparse product is libparamsp_hip.so.
+#include "glue_common.h"
+
+using namespace pspglue;
+using torch::Tensor;
+
+static void check_cf(int CF)
+{
+    // SpCONV dispatches CF 1..4 only (SpCONV/SpCONV.cpp:92-124)
+    TORCH_CHECK(CF >= 1 && CF <= 8, "CF must be 1..8");
+}
+
+// A*D for a dense D, result cut back to rows(D) (the blocked formats compute into an even-padded buffer,
+// SpCONV/SpCONV.h:115-118)
+static Tensor aggregate(int fmt, const Tensor &D, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values,
+                        const Tensor *target_row, int CF, int blkWarpNum)
+{
+    check_cf(CF);
+    Tensor Dc = D.contiguous();
+    Tensor Y = spmm_new(fmt, Dc, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
+    if (Y.size(0) != Dc.size(0)) Y = Y.narrow(0, 0, Dc.size(0));
+    return Y;
+}
+
+static Tensor forward_impl(int fmt, const Tensor &H, const Tensor &W, const Tensor &rowPtr, const Tensor &colIdx,
+                           const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
+{
+    need_gpu(H, "input");
+    need_gpu(W, "weight");
+    return aggregate(fmt, torch::mm(H, W), rowPtr, colIdx, values, target_row, CF, blkWarpNum);
+}
+
+static std::vector<Tensor> backward_impl(int fmt, const Tensor &dY, const Tensor &H, const Tensor &W, const Tensor &rowPtr,
+                                         const Tensor &colIdx, const Tensor &values, const Tensor *target_row, int CF,
+                                         int blkWarpNum)
+{
+    need_gpu(H, "H");
+    need_gpu(W, "weight");
+    // the reference multiplies by A, not A^T (SpCONV/SpCONV.h:67-71): exact for the symmetric matrices its
+    // loaders build
+    Tensor AG = aggregate(fmt, dY, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
+    return {torch::mm(AG, W.t()), torch::mm(H.t(), AG)};
+}
+
+#define PSP_CONV(NAME, FMT)                                                                                       \
+    static Tensor NAME##_forward(Tensor H, Tensor W, Tensor rowPtr, Tensor colIdx, Tensor values, int CF, int bw)  \
+    {                                                                                                             \
+        return forward_impl(FMT, H, W, rowPtr, colIdx, values, nullptr, CF, bw);                                  \
+    }                                                                                                             \
+    static std::vector<Tensor> NAME##_backward(Tensor dY, Tensor H, Tensor W, Tensor rowPtr, Tensor colIdx,       \
+                                               Tensor values, int CF, int bw)                                     \
+    {                                                                                                             \
+        return backward_impl(FMT, dY, H, W, rowPtr, colIdx, values, nullptr, CF, bw);                             \
+    }
+#define PSP_CONV_SPLIT(NAME, FMT)                                                                                 \
+    static Tensor NAME##_forward(Tensor H, Tensor W, Tensor rowPtr, Tensor colIdx, Tensor values, Tensor tr,      \
+                                 int CF, int bw)                                                                  \
+    {                                                                                                             \
+        return forward_impl(FMT, H, W, rowPtr, colIdx, values, &tr, CF, bw);                                      \
+    }                                                                                                             \
+    static std::vector<Tensor> NAME##_backward(Tensor dY, Tensor H, Tensor W, Tensor rowPtr, Tensor colIdx,       \
+                                               Tensor values, Tensor tr, int CF, int bw)                          \
+    {                                                                                                             \
+        return backward_impl(FMT, dY, H, W, rowPtr, colIdx, values, &tr, CF, bw);                                 \
+    }
+
+PSP_CONV(csr_spmm, 0)
+PSP_CONV_SPLIT(csr_split_spmm, 1)
+PSP_CONV(bcsr_spmm, 2)
+PSP_CONV_SPLIT(bcsr_split_spmm, 3)
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    m.def("split_csr", &pspglue::split_csr, "row split on the host");
+    m.def("split_csr_par", &pspglue::split_csr_par, "row split on the host with a precomputed segment prefix");
+    m.def("csr_spmm_forward", &csr_spmm_forward, "A*(H*W), CSR");
+    m.def("csr_spmm_backward", &csr_spmm_backward, "[dH, dW], CSR");
+    m.def("csr_split_spmm_forward", &csr_split_spmm_forward, "A*(H*W), row-split CSR");
+    m.def("csr_split_spmm_backward", &csr_split_spmm_backward, "[dH, dW], row-split CSR");
+    m.def("bcsr_spmm_forward", &bcsr_spmm_forward, "A*(H*W), 2x1 BCSR");
+    m.def("bcsr_spmm_backward", &bcsr_spmm_backward, "[dH, dW], 2x1 BCSR");
+    m.def("bcsr_split_spmm_forward", &bcsr_split_spmm_forward, "A*(H*W), row-split 2x1 BCSR");
+    m.def("bcsr_split_spmm_backward", &bcsr_split_spmm_backward, "[dH, dW], row-split 2x1 BCSR");
+}

@@ -1,0 +1,137 @@
+// Python module `ParamSpMM`: the binding surface of the reference's SpMM/SpMM.cpp:891-926, backed by
+// libparamsp_hip.so.  Argument order, tensor requirements and return types follow the reference bindings.
+#include "glue_common.h"
+
+using namespace pspglue;
+using torch::Tensor;
+
+// ---- the four PCSR SpMM operators (SpMM/SpMM.cpp:77-337) ---------------------------------------------
+static Tensor csr_spmm(Tensor input, Tensor rowPtr, Tensor colIdx, Tensor values, int CF, int blkWarpNum)
+{
+    return spmm_new(0, input, rowPtr, colIdx, values, nullptr, CF, blkWarpNum);
+}
+static Tensor csr_split_spmm(Tensor input, Tensor rowPtr_split, Tensor colIdx, Tensor values, Tensor target_row,
+                             int CF, int blkWarpNum)
+{
+    return spmm_new(1, input, rowPtr_split, colIdx, values, &target_row, CF, blkWarpNum);
+}
+static Tensor bcsr_spmm(Tensor input, Tensor rowPtr_bcsr, Tensor colIdx, Tensor values, int CF, int blkWarpNum)
+{
+    return spmm_new(2, input, rowPtr_bcsr, colIdx, values, nullptr, CF, blkWarpNum);
+}
+static Tensor bcsr_split_spmm(Tensor input, Tensor rowPtr_bcsr_split, Tensor colIdx, Tensor values, Tensor target_row,
+                              int CF, int blkWarpNum)
+{
+    return spmm_new(3, input, rowPtr_bcsr_split, colIdx, values, &target_row, CF, blkWarpNum);
+}
+
+// ---- *_profile twins (SpMM/SpMM.cpp:482-889): mean of 200 launches, int GFLOP/s = 2*nnz*N / t ----------
+static int profile_impl(int fmt, const Tensor &X, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values,
+                        const Tensor *target_row, long nnz, int CF, int blkWarpNum)
+{
+    check_spmm_args(fmt, X, rowPtr, colIdx, values, target_row);
+    c10::hip::HIPGuard guard(X.device());
+    const long rows_out = fmt >= 2 ? (X.size(0) + 1) / 2 * 2 : X.size(0);
+    auto Y = torch::empty({rows_out, X.size(1)}, X.options());
+    hipStream_t s = (hipStream_t)stream_of(X);
+    const float ms = time_launches(s, kProfileWarmup, kProfileIters,
+                                   [&] { spmm_into(fmt, Y, X, rowPtr, colIdx, values, target_row, CF, blkWarpNum); });
+    return gflops(2.0 * (double)nnz * (double)X.size(1), ms);
+}
+static int csr_spmm_profile(Tensor input, Tensor rowPtr, Tensor colIdx, Tensor values, int CF, int blkWarpNum)
+{
+    return profile_impl(0, input, rowPtr, colIdx, values, nullptr, values.size(0), CF, blkWarpNum);
+}
+static int csr_split_spmm_profile(Tensor input, Tensor rowPtr_split, Tensor colIdx, Tensor values, Tensor target_row,
+                                  int CF, int blkWarpNum)
+{
+    return profile_impl(1, input, rowPtr_split, colIdx, values, &target_row, values.size(0), CF, blkWarpNum);
+}
+// the blocked twins take the true non-zero count before CF (SpMM/SpMM.cpp:614-621)
+static int bcsr_spmm_profile(Tensor input, Tensor rowPtr_bcsr, Tensor colIdx, Tensor values, int nnz, int CF, int blkWarpNum)
+{
+    return profile_impl(2, input, rowPtr_bcsr, colIdx, values, nullptr, nnz, CF, blkWarpNum);
+}
+static int bcsr_split_spmm_profile(Tensor input, Tensor rowPtr_bcsr_split, Tensor colIdx, Tensor values,
+                                   Tensor target_row, int nnz, int CF, int blkWarpNum)
+{
+    return profile_impl(3, input, rowPtr_bcsr_split, colIdx, values, &target_row, nnz, CF, blkWarpNum);
+}
+
+// ---- explicit timing helper of this build: median-free mean over a caller-chosen iteration count -----
+static double spmm_time_ms(int fmt, Tensor input, Tensor rowPtr, Tensor colIdx, Tensor values,
+                           c10::optional<Tensor> target_row, int CF, int blkWarpNum, int warmup, int iters)
+{
+    TORCH_CHECK(fmt >= 0 && fmt <= 3, "fmt must be 0 (csr), 1 (csr_split), 2 (bcsr) or 3 (bcsr_split)");
+    TORCH_CHECK((fmt & 1) == (target_row.has_value() ? 1 : 0), "target_row must be given exactly for split formats");
+    TORCH_CHECK(warmup >= 0 && iters >= 1, "warmup >= 0 and iters >= 1 required");
+    const Tensor *tr = target_row.has_value() ? &target_row.value() : nullptr;
+    check_spmm_args(fmt, input, rowPtr, colIdx, values, tr);
+    c10::hip::HIPGuard guard(input.device());
+    const long rows_out = fmt >= 2 ? (input.size(0) + 1) / 2 * 2 : input.size(0);
+    auto Y = torch::empty({rows_out, input.size(1)}, input.options());
+    hipStream_t s = (hipStream_t)stream_of(input);
+    return (double)time_launches(s, warmup, iters,
+                                 [&] { spmm_into(fmt, Y, input, rowPtr, colIdx, values, tr, CF, blkWarpNum); });
+}
+
+// ---- generic vec_size x 1 blocks and vendor baselines ---------------------------------------------------
+// The reference instantiates vec_spmm only for vec_size 3 (SpMM/SpMM.cpp:352,406) and its decider never
+// selects it (decider.py:63); the cusparse_* / gespmm_* entries are third-party comparison baselines
+// (SpMM/Baseline_kernel.cu).  The names stay importable; calling them reports what is missing.
+[[noreturn]] static void not_built(const char *what)
+{
+    TORCH_CHECK(false, what, " is not part of this build (only the PCSR operators csr/csr_split/bcsr/bcsr_split are)");
+}
+static Tensor vec_spmm(Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_spmm (vec_size 3 blocks)"); }
+static Tensor vec_split_spmm(Tensor, Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_split_spmm (vec_size 3 blocks)"); }
+static int vec_spmm_profile(Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_spmm_profile"); }
+static int vec_split_spmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_split_spmm_profile"); }
+static Tensor baseline4(Tensor, Tensor, Tensor, Tensor) { not_built("the cuSPARSE / GE-SpMM comparison baseline"); }
+static int baseline4_profile(Tensor, Tensor, Tensor, Tensor) { not_built("the cuSPARSE / GE-SpMM comparison baseline"); }
+
+static py::dict spmm_plan(int N, int CF, int blkWarpNum)
+{
+    psp_spmm_plan p;
+    ok(psp_spmm_plan_for(N, CF, blkWarpNum, &p));
+    py::dict d;
+    d["vec"] = p.vec;
+    d["coarsen"] = p.coarsen;
+    d["lanes_per_row"] = p.lanes_per_row;
+    d["rows_per_wave"] = p.rows_per_wave;
+    d["unroll"] = p.unroll;
+    d["col_tiles"] = p.col_tiles;
+    d["waves_per_block"] = p.waves_per_block;
+    return d;
+}
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
+{
+    m.def("split_csr", &pspglue::split_csr, "row split on the host (CPU int32 rowPtr, granularity)");
+    m.def("split_csr_par", &pspglue::split_csr_par, "row split on the host with a precomputed segment prefix");
+    m.def("csr_spmm", &csr_spmm, "CSR SpMM (HIP, gfx950)");
+    m.def("csr_split_spmm", &csr_split_spmm, "row-split CSR SpMM (HIP, gfx950)");
+    m.def("bcsr_spmm", &bcsr_spmm, "2x1 BCSR SpMM (HIP, gfx950)");
+    m.def("bcsr_split_spmm", &bcsr_split_spmm, "row-split 2x1 BCSR SpMM (HIP, gfx950)");
+    m.def("vec_spmm", &vec_spmm, "not built");
+    m.def("vec_split_spmm", &vec_split_spmm, "not built");
+    m.def("csr_spmm_profile", &csr_spmm_profile, "GFLOP/s of csr_spmm");
+    m.def("csr_split_spmm_profile", &csr_split_spmm_profile, "GFLOP/s of csr_split_spmm");
+    m.def("bcsr_spmm_profile", &bcsr_spmm_profile, "GFLOP/s of bcsr_spmm");
+    m.def("bcsr_split_spmm_profile", &bcsr_split_spmm_profile, "GFLOP/s of bcsr_split_spmm");
+    m.def("vec_spmm_profile", &vec_spmm_profile, "not built");
+    m.def("vec_split_spmm_profile", &vec_split_spmm_profile, "not built");
+    m.def("cusparse_compute", &baseline4, "not built");
+    m.def("cusparse_profile", &baseline4_profile, "not built");
+    m.def("cusparse_compute_csr_alg2", &baseline4, "not built");
+    m.def("cusparse_profile_csr_alg2", &baseline4_profile, "not built");
+    m.def("cusparse_compute_coo_alg4", &baseline4, "not built");
+    m.def("cusparse_profile_coo_alg4", &baseline4_profile, "not built");
+    m.def("cusparse_compute_csc", &baseline4, "not built");
+    m.def("cusparse_profile_csc", &baseline4_profile, "not built");
+    m.def("gespmm_compute", &baseline4, "not built");
+    m.def("gespmm_profile", &baseline4_profile, "not built");
+    // additions of this build
+    m.def("spmm_time_ms", &spmm_time_ms, "mean ms per launch: (fmt, X, rowPtr, colIdx, val, target_row|None, CF, bw, warmup, iters)");
+    m.def("spmm_plan", &spmm_plan, "how (N, CF, blkWarpNum) maps onto the wave64 kernel");
+}
