@@ -1,0 +1,227 @@
+#!/usr/bin/env python3
+"""GCN / GIN / AGNN training driver with the command line of the reference's GNN.py:15-28 and its timing
+loop (1 warm-up epoch + ``num_epoches`` timed epochs, Adam lr 0.01, prints ``training time per epoch``).
+
+Besides ``--path/--mtx_name`` (MatrixMarket files) it accepts ``--synthetic NAME`` (a seeded generator of
+``synth.config_graph``: C1, C2, C3, C3s, C5, C5p) because no dataset ships with this build.
+
+    python -m paramspmm_ae_amd.GNN --net GCN --synthetic C1 --hidden_list 16 --num_classes 16 --num_epoches 20
+"""
+import argparse
+import glob
+import os
+import time
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .decider import SpMMDecider, DEFAULT_PICKLE_PATH
+from .gnn_conv import AGNNConv, GCNConv, GINConv
+from .graph_input import graph_input
+from .PCSR import pcsr_spmm
+
+
+class Net_5layers(torch.nn.Module):
+    """Five GCN layers, ReLU between, log-softmax out (GNN.py:43-61)."""
+
+    def __init__(self, num_classes, num_features, x, spmm_dict, hidden):
+        super().__init__()
+        self.spmm_dict = spmm_dict
+        self.x = x
+        widths = [num_features, hidden, hidden, hidden, hidden, num_classes]
+        self.conv1, self.conv2, self.conv3, self.conv4, self.conv5 = (
+            GCNConv(widths[i], widths[i + 1]) for i in range(5)
+        )
+
+    def forward(self):
+        x = self.x
+        for conv in (self.conv1, self.conv2, self.conv3, self.conv4):
+            x = F.relu(conv(x, self.spmm_dict))
+        return F.log_softmax(self.conv5(x, self.spmm_dict), dim=1)
+
+
+class GIN(torch.nn.Module):
+    """Five GIN layers (GNN.py:104-123)."""
+
+    def __init__(self, num_classes, num_features, x, spmm_dict, hidden):
+        super().__init__()
+        self.spmm_dict = spmm_dict
+        self.x = x
+        widths = [num_features, hidden, hidden, hidden, hidden, num_classes]
+        self.conv1, self.conv2, self.conv3, self.conv4, self.conv5 = (
+            GINConv(widths[i], widths[i + 1]) for i in range(5)
+        )
+
+    def forward(self):
+        x = self.x
+        for conv in (self.conv1, self.conv2, self.conv3, self.conv4):
+            x = F.relu(conv(x, self.spmm_dict))
+        return F.log_softmax(self.conv5(x, self.spmm_dict), dim=1)
+
+
+class AGNN(torch.nn.Module):
+    """num_layers attention layers with dropout after the first (GNN.py:82-101)."""
+
+    def __init__(self, num_classes, num_features, x, spmm_dict, hidden, colIdx, num_layers=5):
+        super().__init__()
+        self.x = x
+        self.spmm_dict = spmm_dict
+        self.colIdx = colIdx
+        self.conv1 = AGNNConv(num_features, hidden)
+        self.hidden_layers = nn.ModuleList(AGNNConv(hidden, hidden) for _ in range(num_layers - 2))
+        self.conv2 = AGNNConv(hidden, num_classes)
+        self.relu = nn.ReLU()
+
+    def forward(self):
+        x = self.relu(self.conv1(self.x, self.spmm_dict, self.colIdx))
+        x = F.dropout(x, training=self.training)
+        for conv in self.hidden_layers:
+            x = self.relu(conv(x, self.spmm_dict, self.colIdx))
+        return F.log_softmax(self.conv2(x, self.spmm_dict, self.colIdx), dim=1)
+
+
+def train_profiling(model, labels, num_epoches, verbose=False, progress=False):
+    """1 untimed epoch (unless verbose) + num_epoches timed epochs; returns ms per epoch (GNN.py:126-151)."""
+    optimizer = torch.optim.Adam(model.parameters(), lr=0.01, capturable=True)
+
+    def epoch():
+        model.train()
+        optimizer.zero_grad()
+        loss = F.nll_loss(model(), labels)
+        loss.backward()
+        optimizer.step()
+        return loss
+
+    if not verbose:
+        epoch()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    steps = range(num_epoches)
+    if progress:
+        from tqdm import tqdm
+
+        steps = tqdm(steps)
+    for _ in steps:
+        epoch()
+    torch.cuda.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / num_epoches
+    print("training time per epoch: {:.3f} (ms)".format(ms))
+    return ms
+
+
+def load_graph(net, path=None, mtx_name=None, synthetic=None, verbose=True):
+    """The per-network loader choices of GNN.py:189-195."""
+    graph = graph_input(mtx_name=mtx_name if synthetic is None else synthetic, path=path)
+    graph.verbose = verbose
+    if synthetic is not None:
+        from . import synth
+
+        if net == "GIN":
+            # GIN_epsilon=0.5 on a symmetric pattern: off-diagonal 1, diagonal 1.5 (graph_input.py:381-390)
+            r, c, n = _synthetic_edges(synthetic)
+            rowPtr, colIdx, val = synth.to_unit_csr(r, c, n, self_loops=True)
+            val[colIdx == _row_of(rowPtr)] = 1.5
+        else:
+            rowPtr, colIdx, val, n = synth.config_graph(synthetic)
+        graph.load_from_csr(rowPtr, colIdx, val, if_mask=(net == "AGNN"))
+    elif net == "GIN":
+        graph.load(load_from_mtx=True, GIN_epsilon=0.5)
+    elif net == "AGNN":
+        graph.load(load_from_mtx=True, is_normalize=True, if_mask=True)
+    else:
+        graph.load(load_from_mtx=True, is_normalize=True)
+    return graph
+
+
+def _row_of(rowPtr):
+    import numpy as np
+
+    return np.repeat(np.arange(rowPtr.size - 1, dtype=np.int32), np.diff(rowPtr))
+
+
+def _synthetic_edges(name):
+    from . import synth
+
+    rowPtr, colIdx, _, n = synth.config_graph(name)
+    rows = _row_of(rowPtr)
+    keep = rows < colIdx
+    return rows[keep].astype("int64"), colIdx[keep].astype("int64"), n
+
+
+def build_model(net, graph, operators, hidden, num_features, num_classes, num_layers=5):
+    """Feature / label initialisation and model construction of GNN.py:196-238."""
+    device = torch.device("cuda")
+    if net == "GCN":
+        graph.init_feat_embedding(num_features)
+        graph.init_labels(num_classes)
+        return Net_5layers(num_classes, num_features, graph.x, operators, hidden).to(device)
+    # AGNN and GIN run on inputs padded to an even number of rows so that 2x1 blocks fit (GNN.py:226-238)
+    graph.init_feat_embedding(num_features, 2)
+    graph.init_labels(num_classes, 2)
+    if net == "AGNN":
+        colIdx = graph.csr_data.colIdx.to(device).unsqueeze(-1)
+        return AGNN(num_classes, num_features, graph.x, operators, hidden, colIdx, num_layers).to(device)
+    return GIN(num_classes, num_features, graph.x, operators, hidden).to(device)
+
+
+def configure_operators(decider, graph, dims, override=None):
+    """One pcsr_spmm per layer width, configured by the decider (GNN.py:200-209) or by ``override`` =
+    (if_split, vec_size, CF, blkWarpNum)."""
+    ops = {}
+    for dim in dims:
+        if_split, vec_size, CF, blkWarpNum = override if override is not None else decider.config_PCSR(graph, dim)
+        ops[dim] = pcsr_spmm(graph=graph, vec_size=vec_size, if_split=if_split, CF=CF, blkWarpNum=blkWarpNum)
+    return ops
+
+
+def main(argv=None):
+    p = argparse.ArgumentParser()
+    p.add_argument("--verbose", type=str, choices=["True", "False"], default="False")
+    p.add_argument("--hidden_list", nargs="*", type=int, default=[32], help="hidden size list")
+    p.add_argument("--num_classes", type=int, default=32)
+    p.add_argument("--num_features", type=int, default=32)
+    p.add_argument("--num_epoches", type=int, default=200)
+    p.add_argument("--num_layers", type=int, default=5)
+    p.add_argument("--path", type=str, default="./dataset/")
+    p.add_argument("--pickle_path", type=str, default=DEFAULT_PICKLE_PATH)
+    p.add_argument("--mtx_name", type=str, default="")
+    p.add_argument("--net", type=str, choices=["GCN", "GIN", "AGNN"], default="AGNN")
+    p.add_argument("--synthetic", type=str, default=None, help="C1, C2, C3, C3s, C5 or C5p instead of a .mtx file")
+    p.add_argument("--config", nargs=4, type=int, default=None, metavar=("IF_SPLIT", "VEC", "CF", "BW"),
+                   help="skip the decider and use this configuration for every layer width")
+    args = p.parse_args(argv)
+    print(args)
+    assert torch.cuda.is_available()
+
+    if args.synthetic is not None:
+        names = [args.synthetic]
+    elif args.mtx_name:
+        names = [args.mtx_name]
+    else:
+        names = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(args.path, "*.mtx")))
+
+    decider = None
+    if args.config is None:
+        decider = SpMMDecider(args.pickle_path)
+        decider.gen_model_dict([16, 32, 48, 64, 80, 96, 112, 128])
+
+    results = {}
+    for hidden in args.hidden_list:
+        for name in names:
+            print("-------------mtx: {} hidden_size: {}-------------".format(name, hidden))
+            t0 = time.perf_counter()
+            graph = load_graph(args.net, args.path, name, args.synthetic)
+            t1 = time.perf_counter()
+            ops = configure_operators(decider, graph, [hidden, args.num_classes],
+                                      None if args.config is None else tuple(args.config))
+            print("SpMM-decider config time: {:.3f} (ms)".format((time.perf_counter() - t1) * 1e3))
+            model = build_model(args.net, graph, ops, hidden, args.num_features, args.num_classes, args.num_layers)
+            torch.cuda.synchronize()
+            results[(name, hidden)] = train_profiling(model, graph.y, args.num_epoches, verbose=args.verbose == "True")
+            print("end2end time: {:.3f} (ms)".format((time.perf_counter() - t0) * 1e3))
+    return results
+
+
+if __name__ == "__main__":
+    main()

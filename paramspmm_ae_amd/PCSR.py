@@ -1,0 +1,175 @@
+"""Operator facade over one PCSR variant (same surface as the reference's PCSR.py:19-657).
+
+``pcsr_spmm`` keeps the device tensors of the variant selected by ``<if_split, vec_size>`` and forwards to the
+extension modules ParamSpMM / ParamSDDMM / ParamSpCONV of this build.  Public attributes read by the GNN layers
+(gnn_conv.py:19-105): rowPtr, colIdx, val, target_row, mask, if_split, vec_size, CF, blkWarpNum, mtx_nodes,
+mtx_edges, result.
+
+``CF`` keeps the meaning "column coarsening" and ``blkWarpNum`` "wavefronts per workgroup"; how they map onto
+64-lane wavefronts is reported by ``ParamSpMM.spmm_plan(dim, CF, blkWarpNum)``.
+"""
+import math
+
+import torch
+
+import paramspmm_ae_amd  # noqa: F401  (puts lib/ on sys.path)
+import ParamSpMM as SpMM
+import ParamSDDMM as SDDMM
+import ParamSpCONV as SpCONV
+
+
+def gap_calculator(dim, CF, warp_size=32):
+    """Columns a CF*warp_size wide tile leaves unused on its last pass over ``dim`` (PCSR.py:19-26)."""
+    width = warp_size * CF
+    rest = dim % width
+    return 0 if rest == 0 else min(dim, width) - rest
+
+
+def dynamic_CF_prompter(dim, CF_set=None, warp_size=32, verbose=False):
+    """Coarsening factors worth sweeping for ``dim``: CF <= ceil(dim/32) whose gap is below one 32-column
+    slab (PCSR.py:30-42).  The list and its order define the decider's class encoding."""
+    candidates = list(range(1, 9)) if CF_set is None else list(CF_set)
+    candidates = candidates[: math.ceil(dim / 32)]
+    keep = []
+    for cf in candidates:
+        gap = gap_calculator(dim, cf, warp_size)
+        if verbose:
+            print("dim({})->CF:{} gap:{}".format(dim, cf, gap))
+        if gap < 32:
+            keep.append(cf)
+    return keep
+
+
+# (if_split, blocked) -> operator names in the three modules
+_SPMM = {(False, False): "csr_spmm", (True, False): "csr_split_spmm", (False, True): "bcsr_spmm", (True, True): "bcsr_split_spmm"}
+_SDDMM = {(False, False): "csr_sddmm", (True, False): "csr_split_sddmm", (False, True): "bcsr_sddmm", (True, True): "bcsr_split_sddmm"}
+
+
+class pcsr_spmm(object):
+    def __init__(self, graph, vec_size, if_split, mtx_nodes=None, mtx_edges=None, rowPtr=None, colIdx=None,
+                 val=None, target_row=None, CF=1, blkWarpNum=4, device="cuda"):
+        if vec_size not in (1, 2):
+            raise ValueError("this build has vec_size 1 (CSR) and 2 (2x1 BCSR)")
+        if_split = bool(if_split)
+        self.mask = None
+        if graph is None:
+            if mtx_edges is None or mtx_nodes is None or rowPtr is None or colIdx is None or val is None:
+                raise ValueError("when graph is None, mtx_nodes, mtx_edges, rowPtr, colIdx, val should be given")
+            if if_split and target_row is None:
+                raise ValueError("target_row should be given when if_split is True")
+            if not if_split and target_row is not None:
+                raise ValueError("target_row should not be given when if_split is False")
+            if (vec_size == 1) != (val.dim() == 1):
+                raise ValueError("val must be 1-D for vec_size 1 and [nblk, vec_size] otherwise")
+            self.mtx_nodes, self.mtx_edges = mtx_nodes, mtx_edges
+            self.rowPtr, self.colIdx, self.val = rowPtr.to(device), colIdx.to(device), val.to(device)
+            self.target_row = None if target_row is None else target_row.to(device)
+        else:
+            self.mtx_nodes, self.mtx_edges = graph.mtx_nodes, graph.mtx_edges
+            fmt = graph.csr_data if vec_size == 1 else graph.bcsr_data
+            self.rowPtr = (fmt.rowPtr_split if if_split else fmt.rowPtr).to(device)
+            self.colIdx = fmt.colIdx.to(device)
+            self.val = fmt.val.to(device)
+            self.target_row = fmt.target_row.to(device) if if_split else None
+            if vec_size != 1 and getattr(graph, "mask", None) is not None:
+                self.mask = graph.mask.to(device)
+        self.vec_size = vec_size
+        self.if_split = if_split
+        self.CF = CF
+        self.blkWarpNum = blkWarpNum
+        self.result = None
+
+    # ---- plumbing ---------------------------------------------------------------------------
+    def _key(self):
+        return (self.if_split, self.vec_size != 1)
+
+    def _sparse_args(self, val=None):
+        args = [self.rowPtr, self.colIdx, self.val if val is None else val]
+        if self.if_split:
+            args.append(self.target_row)
+        return args
+
+    def _spmm(self, X, val=None, CF=None, blkWarpNum=None):
+        fn = getattr(SpMM, _SPMM[self._key()])
+        return fn(X, *self._sparse_args(val), self.CF if CF is None else CF,
+                  self.blkWarpNum if blkWarpNum is None else blkWarpNum)
+
+    def _dense_input(self, dim, x):
+        if x is None and dim is None:
+            raise ValueError("at least one of x and dim should be given")
+        if dim is not None:
+            return torch.ones(self.mtx_nodes, dim, device="cuda")
+        return x.to("cuda")
+
+    # ---- SpMM -------------------------------------------------------------------------------
+    def get_spmm_result(self, dim=None, x=None, CF=None, blkWarpNum=None):
+        """A*X with X = ones(n, dim) or x; the first mtx_nodes rows land on the CPU in ``self.result``."""
+        assert torch.cuda.is_available()
+        X = self._dense_input(dim, x)
+        out = self._spmm(X, CF=CF, blkWarpNum=blkWarpNum)
+        self.result = out[0 : self.mtx_nodes, :].to("cpu")
+        del X
+        torch.cuda.empty_cache()
+
+    def AGNN_spmm(self, spVal, X):
+        """SpMM with caller-supplied values (edge attentions) in this variant's layout."""
+        return self._spmm(X, val=spVal)
+
+    def GIN_spmm(self, X):
+        return self._spmm(X)
+
+    # ---- SDDMM ------------------------------------------------------------------------------
+    def _sddmm(self, A, B, blkWarpNum):
+        fn = getattr(SDDMM, _SDDMM[self._key()])
+        CF = (A.size(1) + 31) // 32
+        return fn(A, B, *self._sparse_args(), CF, blkWarpNum)
+
+    def AGNN_sddmm(self, A):
+        """Per stored entry <A[row], A[col]>; for 2x1 blocks the result is [nblk, 2] (PCSR.py:290-320)."""
+        if self.vec_size != 1 and self.mask is None:
+            raise ValueError("mask should be given when vec_size=2")
+        return self._sddmm(A, A, self.blkWarpNum)
+
+    def get_sddmm_result(self, dim, blkWarpNum):
+        assert torch.cuda.is_available()
+        A = torch.ones((self.mtx_nodes + 1) // 2 * 2, dim, device="cuda")
+        B = torch.ones(self.mtx_nodes, dim, device="cuda")
+        return self._sddmm(A, B, blkWarpNum)
+
+    # ---- fused GCN layer ----------------------------------------------------------------------
+    def forward(self, H, w):
+        if H is None or w is None:
+            raise ValueError("H and w should be given")
+        fn = getattr(SpCONV, _SPMM[self._key()] + "_forward")
+        return fn(H, w, *self._sparse_args(), self.CF, self.blkWarpNum)
+
+    def backward(self, d_output, H, w):
+        if d_output is None or H is None:
+            raise ValueError("d_output and H should be given")
+        fn = getattr(SpCONV, _SPMM[self._key()] + "_backward")
+        d_input, d_weight = fn(d_output, H, w, *self._sparse_args(), self.CF, self.blkWarpNum)
+        return d_input, d_weight
+
+    # ---- timing -----------------------------------------------------------------------------
+    def cf_warpnum_profiling(self, CF, blkWarpNum, dim=None, x=None, verbose=True):
+        """GFLOP/s (int) of this variant with an explicit (CF, blkWarpNum) (PCSR.py:433-505)."""
+        assert torch.cuda.is_available()
+        X = self._dense_input(dim, x)
+        fn = getattr(SpMM, _SPMM[self._key()] + "_profile")
+        args = self._sparse_args()
+        if self.vec_size != 1:
+            args.append(self.mtx_edges)  # blocked twins take the true nnz before CF
+        throughput = fn(X, *args, CF, blkWarpNum)
+        if verbose:
+            print("dim: {} gflops: {:.0f}".format(X.size(1), throughput))
+        return throughput
+
+    def profiling(self, dim=None, x=None, verbose=True):
+        return self.cf_warpnum_profiling(self.CF, self.blkWarpNum, dim=dim, x=x, verbose=verbose)
+
+    def time_ms(self, X, CF=None, blkWarpNum=None, warmup=5, iters=20):
+        """Mean milliseconds per SpMM launch (an addition of this build; used by the sweep harness)."""
+        fmt = (1 if self.if_split else 0) + (2 if self.vec_size != 1 else 0)
+        return SpMM.spmm_time_ms(fmt, X, self.rowPtr, self.colIdx, self.val, self.target_row,
+                                 self.CF if CF is None else CF, self.blkWarpNum if blkWarpNum is None else blkWarpNum,
+                                 warmup, iters)

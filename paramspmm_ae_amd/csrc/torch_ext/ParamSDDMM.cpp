@@ -48,7 +48,7 @@ static Tensor sddmm_new(int fmt, const Tensor &A, const Tensor &B, const Tensor 
                         const Tensor &values, const Tensor *target_row, const Tensor *scale, int CF, int blkWarpNum)
 {
     check_sddmm_args(fmt, A, B, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
-    c10::hip::HIPGuard guard(A.device());
+    pspglue::DeviceGuard guard(A.device());
     auto out = torch::empty_like(values);  // every stored entry is written by the kernel
     const int nrows = (int)rowPtr.size(0) - 1, K = (int)A.size(1);
     if (values.numel() == 0) return out;
@@ -95,7 +95,7 @@ static int profile_impl(int fmt, const Tensor &A, const Tensor &B, const Tensor 
                         const Tensor &values, const Tensor *target_row, long nnz, int CF, int blkWarpNum)
 {
     check_sddmm_args(fmt, A, B, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
-    c10::hip::HIPGuard guard(A.device());
+    pspglue::DeviceGuard guard(A.device());
     hipStream_t s = (hipStream_t)stream_of(A);
     const float ms = time_launches(s, kProfileWarmup, kProfileIters, [&] {
         (void)sddmm_new(fmt, A, B, rowPtr, colIdx, values, target_row, nullptr, CF, blkWarpNum);
@@ -138,7 +138,7 @@ static Tensor genmask(Tensor rowPtr_bcsr, Tensor rowPtr, Tensor blkval, int nnz)
     const int nbr = (int)rowPtr_bcsr.size(0) - 1;
     // block-row t reads rowPtr[2t] and rowPtr[2t+1]
     TORCH_CHECK(rowPtr.size(0) >= 2L * nbr, "rowPtr is too short for the block row pointer");
-    c10::hip::HIPGuard guard(rowPtr.device());
+    pspglue::DeviceGuard guard(rowPtr.device());
     auto mask = torch::empty({(long)nnz}, rowPtr.options());
     ok(psp_genmask(ip(rowPtr_bcsr), ip(rowPtr), fp(blkval), nbr, nnz, nnz ? mask.data_ptr<int>() : nullptr, stream_of(rowPtr)));
     return mask;
@@ -153,7 +153,7 @@ static Tensor segment_softmax(Tensor rowPtr, Tensor e)
     need_f32(e, "e", 1);
     same_device(rowPtr, e, "segment_softmax");
     check_rowptr_vs(rowPtr, "rowPtr");
-    c10::hip::HIPGuard guard(e.device());
+    pspglue::DeviceGuard guard(e.device());
     auto out = torch::empty_like(e);
     ok(psp_segment_softmax_f32(ip(rowPtr), fp(e), fpw(out), (int)rowPtr.size(0) - 1, stream_of(e)));
     return out;

@@ -30,7 +30,7 @@ static int profile_impl(int fmt, const Tensor &X, const Tensor &rowPtr, const Te
                         const Tensor *target_row, long nnz, int CF, int blkWarpNum)
 {
     check_spmm_args(fmt, X, rowPtr, colIdx, values, target_row);
-    c10::hip::HIPGuard guard(X.device());
+    pspglue::DeviceGuard guard(X.device());
     const long rows_out = fmt >= 2 ? (X.size(0) + 1) / 2 * 2 : X.size(0);
     auto Y = torch::empty({rows_out, X.size(1)}, X.options());
     hipStream_t s = (hipStream_t)stream_of(X);
@@ -67,7 +67,7 @@ static double spmm_time_ms(int fmt, Tensor input, Tensor rowPtr, Tensor colIdx, 
     TORCH_CHECK(warmup >= 0 && iters >= 1, "warmup >= 0 and iters >= 1 required");
     const Tensor *tr = target_row.has_value() ? &target_row.value() : nullptr;
     check_spmm_args(fmt, input, rowPtr, colIdx, values, tr);
-    c10::hip::HIPGuard guard(input.device());
+    pspglue::DeviceGuard guard(input.device());
     const long rows_out = fmt >= 2 ? (input.size(0) + 1) / 2 * 2 : input.size(0);
     auto Y = torch::empty({rows_out, input.size(1)}, input.options());
     hipStream_t s = (hipStream_t)stream_of(input);

@@ -4,12 +4,16 @@
 #pragma once
 #include <torch/extension.h>
 #include <ATen/hip/HIPContext.h>
-#include <c10/hip/HIPGuard.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <hip/hip_runtime_api.h>
 #include <vector>
 #include "paramsp.h"
 
 namespace pspglue {
+
+// PyTorch-ROCm presents HIP devices under the "cuda" device type; these are its guard / stream types for that.
+using DeviceGuard = c10::hip::HIPGuardMasqueradingAsCUDA;
 
 // Same contract as the reference's CHECK_INPUT / CHECK_CPU_INPUT (SpMM/SpMM.cpp:5-13): a violation is a
 // RuntimeError in Python.  Index tensors must be int32 and value / feature tensors float32 (the reference
@@ -50,7 +54,7 @@ inline float *fpw(torch::Tensor &t) { return t.numel() ? t.data_ptr<float>() : n
 
 inline psp_stream_t stream_of(const torch::Tensor &t)
 {
-    return (psp_stream_t)at::hip::getCurrentHIPStream(t.device().index()).stream();
+    return (psp_stream_t)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.device().index()).stream();
 }
 
 // Range checks the device cannot afford: done once per call on the host from tensor sizes only.
@@ -147,7 +151,7 @@ inline torch::Tensor spmm_new(int fmt, const torch::Tensor &X, const torch::Tens
                               const torch::Tensor &values, const torch::Tensor *target_row, int CF, int blkWarpNum)
 {
     check_spmm_args(fmt, X, rowPtr, colIdx, values, target_row);
-    c10::hip::HIPGuard guard(X.device());
+    pspglue::DeviceGuard guard(X.device());
     const long rows_out = fmt >= 2 ? (X.size(0) + 1) / 2 * 2 : X.size(0);
     // the library defines every element of Y, so no zero-initialised allocation is needed
     auto Y = torch::empty({rows_out, X.size(1)}, X.options());

@@ -1,0 +1,127 @@
+"""GCN / AGNN / GIN layers as autograd Functions over the PCSR operators (same surface and the same forward /
+backward algebra as the reference's gnn_conv.py:13-238).  Layers look their operator up in ``spmm_dict`` by
+output width (gnn_conv.py:121-124)."""
+import math
+
+import torch
+
+import paramspmm_ae_amd  # noqa: F401
+import ParamSpCONV as SpCONV
+
+n_heads = 1
+
+_CONV = {(False, False): "csr_spmm", (True, False): "csr_split_spmm", (False, True): "bcsr_spmm", (True, True): "bcsr_split_spmm"}
+
+
+def _conv_args(op):
+    args = [op.rowPtr, op.colIdx, op.val]
+    if op.if_split:
+        args.append(op.target_row)
+    return args + [op.CF, op.blkWarpNum]
+
+
+def _conv_name(op):
+    return _CONV[(bool(op.if_split), op.vec_size != 1)]
+
+
+class GCNFunction(torch.autograd.Function):
+    """forward A(HW); backward dH = (A dY) W^T, dW = H^T (A dY) -- A is symmetric (gnn_conv.py:13-107)."""
+
+    @staticmethod
+    def forward(ctx, H, weight, ParamSpMM):
+        ctx.save_for_backward(H, weight)
+        ctx.ParamSpMM = ParamSpMM
+        return getattr(SpCONV, _conv_name(ParamSpMM) + "_forward")(H, weight, *_conv_args(ParamSpMM))
+
+    @staticmethod
+    def backward(ctx, d_output):
+        H, weight = ctx.saved_tensors
+        op = ctx.ParamSpMM
+        d_input, d_weight = getattr(SpCONV, _conv_name(op) + "_backward")(d_output.contiguous(), H, weight, *_conv_args(op))
+        return d_input, d_weight, None
+
+
+class _Layer(torch.nn.Module):
+    def __init__(self, input_dim, output_dim):
+        super().__init__()
+        self.weights = torch.nn.Parameter(torch.randn(input_dim, output_dim))
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        bound = 1.0 / math.sqrt(self.weights.size(1))
+        self.weights.data.uniform_(-bound, bound)
+
+    def _operator(self, spmm_dict):
+        width = self.weights.size(1)
+        if width not in spmm_dict:
+            raise ValueError("SpMMDecider not support dim: " + str(width))
+        return spmm_dict[width]
+
+
+class GCNConv(_Layer):
+    def forward(self, H, spmm_dict):
+        return GCNFunction.apply(H, self.weights, self._operator(spmm_dict))
+
+
+class AGNNFunction(torch.autograd.Function):
+    """X' = XW; e = <X'_i, X'_j> per stored entry; attention = e * w; out = SpMM(attention, X')
+    (gnn_conv.py:128-180).  No softmax, as in the reference."""
+
+    @staticmethod
+    def forward(ctx, X, weights, attention_w, ParamSpMM, colIdx):
+        X_prime = torch.mm(X, weights)
+        edge_feature = ParamSpMM.AGNN_sddmm(X_prime)
+        # csr: [nnz] ; 2x1 blocks: [nblk, 2] -- a single head scales both the same way
+        edge_attentions = (edge_feature * attention_w.reshape(())).contiguous()
+        out = ParamSpMM.AGNN_spmm(edge_attentions, X_prime)
+        ctx.save_for_backward(X, weights, edge_attentions)
+        ctx.colIdx = colIdx
+        ctx.ParamSpMM = ParamSpMM
+        return out
+
+    @staticmethod
+    def backward(ctx, d_output):
+        op = ctx.ParamSpMM
+        X, weights, edge_attentions = ctx.saved_tensors
+        d_output = d_output.contiguous()
+        d_input_prime = op.AGNN_spmm(edge_attentions, d_output)
+        d_input = torch.mm(d_input_prime, weights.t().contiguous())
+        d_weights = torch.mm(X.t().contiguous(), d_input_prime)
+        d_attention = op.AGNN_sddmm(d_output)
+        if d_attention.dim() != 1:
+            d_attention = d_attention.view(-1)[op.mask]  # block layout -> CSR slots
+        # the reference's literal formula for the attention weight gradient (gnn_conv.py:172)
+        d_attention_w = torch.mm(d_attention[None, :].expand(n_heads, -1), ctx.colIdx.float()).transpose(0, 1)
+        return d_input, d_weights, d_attention_w, None, None
+
+
+class AGNNConv(_Layer):
+    def __init__(self, input_dim, output_dim):
+        super().__init__(input_dim, output_dim)
+        self.attention_w = torch.nn.Parameter(torch.randn(1, n_heads))
+
+    def forward(self, X, spmm_dict, colIdx):
+        return AGNNFunction.apply(X, self.weights, self.attention_w, self._operator(spmm_dict), colIdx)
+
+
+class GINFunction(torch.autograd.Function):
+    """forward (A X) W; backward dW = (A X)^T dY, dX = A (dY W^T) (gnn_conv.py:202-220)."""
+
+    @staticmethod
+    def forward(ctx, X, weight, ParamSpMM):
+        X_agg = ParamSpMM.GIN_spmm(X)
+        ctx.save_for_backward(X_agg, weight)
+        ctx.ParamSpMM = ParamSpMM
+        return torch.mm(X_agg, weight)
+
+    @staticmethod
+    def backward(ctx, d_output):
+        X_agg, weights = ctx.saved_tensors
+        d_weights = torch.mm(X_agg.t(), d_output)
+        d_input = ctx.ParamSpMM.GIN_spmm(torch.mm(d_output, weights.t()).contiguous())
+        return d_input, d_weights, None
+
+
+class GINConv(_Layer):
+    def forward(self, X, spmm_dict):
+        return GINFunction.apply(X, self.weights, self._operator(spmm_dict))

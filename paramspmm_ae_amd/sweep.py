@@ -1,0 +1,53 @@
+"""Configuration sweep: times every ``<representation, CF, blkWarpNum>`` of a graph for a list of feature
+widths.  It is the counterpart of the reference's ``profile_engine`` (PCSR.py:672-806) and produces the same
+column order -- blkWarpNum-major, then CF in ``dynamic_CF_prompter`` order, then the representations vec1,
+vec1_split, vec2, vec2_split -- so that the arg-max column index is the class code ``decode_tree`` expects.
+"""
+import numpy as np
+import torch
+
+from .PCSR import dynamic_CF_prompter, pcsr_spmm
+
+WARP_NUMS = (4, 8)
+REPRESENTATIONS = (("vec1", 1, False), ("vec1_split", 1, True), ("vec2", 2, False), ("vec2_split", 2, True))
+
+
+def column_names(dim):
+    return ["%s_TP_%d%d" % (rep, cf, bw) for bw in WARP_NUMS for cf in dynamic_CF_prompter(dim) for rep, _, _ in REPRESENTATIONS]
+
+
+def decode_column(dim, col):
+    """column index -> (if_split, vec_size, CF, blkWarpNum): the arithmetic of decider.py:63-80."""
+    cfs = dynamic_CF_prompter(dim)
+    _, vec_size, if_split = REPRESENTATIONS[col % 4]
+    cf = cfs[col // 4 % len(cfs)]
+    bw = WARP_NUMS[col // (4 * len(cfs))]
+    return int(if_split), vec_size, cf, bw
+
+
+def operators_of(graph):
+    """The four representations of a loaded graph_input on the GPU, in column order."""
+    return [pcsr_spmm(graph, vec_size=v, if_split=s) for _, v, s in REPRESENTATIONS]
+
+
+def sweep_dim(ops, dim, nnz, n_rows, warmup=3, iters=10, X=None, verify=None):
+    """Times all columns for one width.  Returns (ms[cols], gflops[cols]).
+
+    ``verify``: optional callable(result_tensor, column_name) run once per column on A*X before timing
+    (the reference verifies every swept configuration, PCSR.py:759-770).
+    """
+    rows = (n_rows + 1) // 2 * 2
+    if X is None:
+        X = torch.ones(rows, dim, device="cuda")
+    names = column_names(dim)
+    ms = np.zeros(len(names))
+    col = 0
+    for bw in WARP_NUMS:
+        for cf in dynamic_CF_prompter(dim):
+            for op in ops:
+                if verify is not None:
+                    verify(op._spmm(X, CF=cf, blkWarpNum=bw)[:n_rows], names[col])
+                ms[col] = op.time_ms(X, CF=cf, blkWarpNum=bw, warmup=warmup, iters=iters)
+                col += 1
+    gflops = 2.0 * nnz * dim / 1e6 / ms
+    return ms, gflops

@@ -1,0 +1,203 @@
+"""GPU tests of the PyTorch extension modules (ParamSpMM / ParamSDDMM / ParamSpCONV), the pcsr_spmm facade,
+the format builder with its device-side mask, and the GNN layers against dense torch autograd."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import random_csr
+
+pytestmark = pytest.mark.gpu
+
+VARIANTS = [(1, False), (1, True), (2, False), (2, True)]
+
+
+def sym_graph(n, seed):
+    """Symmetric normalised test graph as a loaded graph_input (values D^-1/2 (A+I) D^-1/2)."""
+    from paramspmm_ae_amd import synth
+    from paramspmm_ae_amd.graph_input import graph_input
+
+    rng = np.random.default_rng(seed)
+    m = n * 4
+    r, c = rng.integers(0, n, m), rng.integers(0, n, m)
+    keep = r != c
+    rowPtr, colIdx, val = synth.to_gcn_csr(r[keep], c[keep], n)
+    g = graph_input("t", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val, if_mask=True)
+    return g, rowPtr, colIdx, val
+
+
+def dense(rowPtr, colIdx, val, n):
+    A = torch.zeros(n, n, dtype=torch.float64)
+    rows = np.repeat(np.arange(n), np.diff(rowPtr))
+    A[torch.from_numpy(rows), torch.from_numpy(colIdx.astype(np.int64))] = torch.from_numpy(val.astype(np.float64))
+    return A
+
+
+@pytest.mark.parametrize("n", [257, 300])
+def test_facade_dispatch_matrix(oracle, n):
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from gpu_util import assert_close
+
+    g, rowPtr, colIdx, val = sym_graph(n, n)
+    rows = (n + 1) // 2 * 2
+    X = np.random.default_rng(1).standard_normal((rows, 64)).astype(np.float32)
+    X[n:] = 0
+    Xd = torch.from_numpy(X).cuda()
+    want = oracle.spmm_csr(rowPtr, colIdx, val, X)
+    scale = oracle.spmm_csr(rowPtr, colIdx, np.abs(val), np.abs(X))
+    A = X / np.maximum(np.linalg.norm(X, axis=1, keepdims=True), 1e-9)
+    Ad = torch.from_numpy(A).cuda()
+    sd = oracle.sddmm_csr(rowPtr, colIdx, A, A)
+    for vec, split in VARIANTS:
+        op = pcsr_spmm(g, vec_size=vec, if_split=split, CF=2, blkWarpNum=8)
+        y = op.GIN_spmm(Xd)
+        assert y.shape[0] == rows and bool((y[n:] == 0).all())
+        assert_close(y[:n], want[:n], what="GIN_spmm %d %s" % (vec, split), scale=scale[:n])
+        op.get_spmm_result(x=Xd[:n].contiguous() if vec == 1 else Xd)
+        assert op.result.shape[0] == n and op.result.device.type == "cpu"
+        assert_close(op.result, want[:n], what="get_spmm_result", scale=scale[:n])
+        e = op.AGNN_sddmm(Ad)
+        if vec == 2:
+            assert e.shape == (op.colIdx.numel(), 2)
+            e = e.view(-1)[op.mask]
+            # block order inside odd rows differs from CSR order: compare row-wise sorted
+            ecpu = e.cpu().numpy()
+            for r in range(n):
+                a, b = rowPtr[r], rowPtr[r + 1]
+                np.testing.assert_allclose(np.sort(ecpu[a:b]), np.sort(sd[a:b]), rtol=1e-5, atol=1e-6)
+        else:
+            assert_close(e, sd, what="AGNN_sddmm")
+        # SpMM with per-entry values in the variant's own layout equals SpMM of the matrix those values form
+        ev = op.val * 0.5
+        y2 = op.AGNN_spmm(ev, Xd)
+        assert_close(y2[:n], 0.5 * want[:n], what="AGNN_spmm", scale=scale[:n])
+        assert op.profiling(dim=16, verbose=False) > 0
+
+
+def test_extension_argument_errors():
+    import paramspmm_ae_amd  # noqa: F401
+    import ParamSpMM
+    import ParamSDDMM
+
+    x = torch.zeros(8, 16, device="cuda")
+    rp = torch.zeros(9, dtype=torch.int32, device="cuda")
+    ci = torch.zeros(0, dtype=torch.int32, device="cuda")
+    v = torch.zeros(0, device="cuda")
+    assert ParamSpMM.csr_spmm(x, rp, ci, v, 1, 4).shape == (8, 16)
+    with pytest.raises(RuntimeError, match="CF must be"):
+        ParamSpMM.csr_spmm(x, rp, ci, v, 9, 4)
+    with pytest.raises(RuntimeError, match="blkWarpNum must be 4 or 8"):
+        ParamSpMM.csr_spmm(x, rp, ci, v, 1, 6)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ParamSpMM.csr_spmm(torch.zeros(16, 8, device="cuda").t(), rp, ci, v, 1, 4)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        ParamSpMM.csr_spmm(x.cpu(), rp, ci, v, 1, 4)
+    with pytest.raises(RuntimeError, match="int32"):
+        ParamSpMM.csr_spmm(x, rp.long(), ci, v, 1, 4)
+    with pytest.raises(RuntimeError, match="float32"):
+        ParamSpMM.csr_spmm(x.double(), rp, ci, v.double(), 1, 4)
+    with pytest.raises(RuntimeError, match="not part of this build"):
+        ParamSpMM.cusparse_compute(x, rp, ci, v)
+    with pytest.raises(RuntimeError, match="same number of columns"):
+        ParamSDDMM.csr_sddmm(x, torch.zeros(8, 8, device="cuda"), rp, ci, v, 1, 4)
+    # bcsr output is padded to an even number of rows
+    xo = torch.zeros(7, 16, device="cuda")
+    rpb = torch.zeros(5, dtype=torch.int32, device="cuda")
+    assert ParamSpMM.bcsr_spmm(xo, rpb, ci, torch.zeros(0, 2, device="cuda"), 1, 4).shape == (8, 16)
+
+
+def test_spconv_forward_backward(oracle):
+    import ParamSpCONV
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+
+    n = 301
+    g, rowPtr, colIdx, val = sym_graph(n, 4)
+    A = dense(rowPtr, colIdx, val, n)
+    H = torch.randn(n, 24, dtype=torch.float64)
+    W = torch.randn(24, 48, dtype=torch.float64) * 0.2
+    dY = torch.randn(n, 48, dtype=torch.float64)
+    fwd = A @ (H @ W)
+    AG = A @ dY
+    dH, dW = AG @ W.t(), H.t() @ AG
+    for vec, split in VARIANTS:
+        op = pcsr_spmm(g, vec_size=vec, if_split=split, CF=1, blkWarpNum=4)
+        out = op.forward(H.float().cuda(), W.float().cuda())
+        assert out.shape == (n, 48)
+        torch.testing.assert_close(out.cpu().double(), fwd, rtol=1e-4, atol=1e-5)
+        gi, gw = op.backward(dY.float().cuda(), H.float().cuda(), W.float().cuda())
+        torch.testing.assert_close(gi.cpu().double(), dH, rtol=1e-4, atol=1e-4)
+        torch.testing.assert_close(gw.cpu().double(), dW, rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("vec,split", VARIANTS)
+def test_gcn_and_gin_layers_match_dense_autograd(vec, split):
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from paramspmm_ae_amd.gnn_conv import GCNConv, GINConv
+
+    n = 200  # even: GIN runs on inputs padded to an even row count
+    g, rowPtr, colIdx, val = sym_graph(n, 9)
+    A = dense(rowPtr, colIdx, val, n).float().cuda()
+    op = pcsr_spmm(g, vec_size=vec, if_split=split, CF=1, blkWarpNum=8)
+    torch.manual_seed(0)
+    for Layer, ref in ((GCNConv, lambda X, W: A @ (X @ W)), (GINConv, lambda X, W: (A @ X) @ W)):
+        layer = Layer(32, 16).cuda()
+        X = torch.randn(n, 32, device="cuda", requires_grad=True)
+        y = layer(X, {16: op})
+        (y * y).sum().backward()
+        Xr = X.detach().clone().requires_grad_(True)
+        Wr = layer.weights.detach().clone().requires_grad_(True)
+        yr = ref(Xr, Wr)
+        (yr * yr).sum().backward()
+        torch.testing.assert_close(y, yr, rtol=1e-4, atol=1e-5)
+        torch.testing.assert_close(X.grad, Xr.grad, rtol=1e-3, atol=1e-4)
+        torch.testing.assert_close(layer.weights.grad, Wr.grad, rtol=1e-3, atol=1e-3)
+    with pytest.raises(ValueError):
+        GCNConv(32, 24).cuda()(X, {16: op})
+
+
+@pytest.mark.parametrize("vec,split", VARIANTS)
+def test_agnn_layer_forward_and_literal_backward(vec, split):
+    """Forward against dense algebra; backward against the reference's literal formulas (gnn_conv.py:153-180)."""
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from paramspmm_ae_amd.gnn_conv import AGNNConv
+
+    n = 120
+    g, rowPtr, colIdx, val = sym_graph(n, 2)
+    pattern = (dense(rowPtr, colIdx, val, n) != 0).float().cuda()
+    op = pcsr_spmm(g, vec_size=vec, if_split=split, CF=1, blkWarpNum=4)
+    torch.manual_seed(1)
+    layer = AGNNConv(20, 32).cuda()
+    X = torch.randn(n, 20, device="cuda", requires_grad=True)
+    ci = g.csr_data.colIdx.cuda().unsqueeze(-1)
+    y = layer(X, {32: op}, ci)
+    Xp = X.detach() @ layer.weights.detach()
+    att = pattern * (Xp @ Xp.t()) * layer.attention_w.detach().reshape(())
+    torch.testing.assert_close(y, att @ Xp, rtol=1e-4, atol=1e-4)
+    dY = torch.randn_like(y)
+    y.backward(dY)
+    d_in_prime = att @ dY
+    torch.testing.assert_close(X.grad, d_in_prime @ layer.weights.detach().t(), rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(layer.weights.grad, X.detach().t() @ d_in_prime, rtol=1e-3, atol=1e-3)
+    if vec == 1:
+        rows = torch.from_numpy(np.repeat(np.arange(n), np.diff(rowPtr))).cuda()
+        d_att = (dY[rows] * dY[g.csr_data.colIdx.cuda().long()]).sum(1)
+    else:
+        # block layout -> CSR slots through the mask: inside odd rows the slots follow block order, not column
+        # order, and the reference multiplies them with colIdx in CSR order all the same (gnn_conv.py:166-172)
+        b = g.bcsr_data
+        t = torch.from_numpy(np.repeat(np.arange(b.rowPtr.numel() - 1), np.diff(b.rowPtr.numpy()))).cuda()
+        cb = b.colIdx.cuda().long()
+        e = torch.stack([(dY[2 * t] * dY[cb]).sum(1), (dY[2 * t + 1] * dY[cb]).sum(1)], 1) * (b.val.cuda() != 0)
+        d_att = e.view(-1)[g.mask.cuda()]
+    want = (d_att[None, :] @ ci.float()).t()
+    torch.testing.assert_close(layer.attention_w.grad, want, rtol=1e-3, atol=1e-1)
+
+
+def test_training_driver_runs_gcn_gin_agnn():
+    from paramspmm_ae_amd import GNN
+
+    for net in ("GCN", "GIN", "AGNN"):
+        res = GNN.main(["--net", net, "--synthetic", "C1", "--hidden_list", "16", "--num_classes", "16",
+                        "--num_features", "32", "--num_epoches", "3", "--config", "0", "2", "1", "4"])
+        assert all(ms > 0 for ms in res.values())

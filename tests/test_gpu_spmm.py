@@ -1,0 +1,129 @@
+"""GPU parity of the SpMM kernels against the CPU oracle, through the C ABI.  Tolerance: rel 1e-5 / abs 1e-6
+(fp32), the bar the north star states.  Inputs: seeded; values in (0.1, 1), features N(0,1)."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import random_csr
+
+pytestmark = pytest.mark.gpu
+
+FMTS = ["csr", "csr_split", "bcsr", "bcsr_split"]
+
+
+@pytest.fixture(scope="module")
+def small(oracle):
+    from gpu_util import Formats
+
+    rowPtr, colIdx, val = random_csr(3001, 12, 7, empty_frac=0.1, hub=(5, 900), values="uniform")
+    return Formats(oracle, rowPtr, colIdx, val)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("N", [16, 32, 48, 64, 96, 128, 160, 192, 224, 256])
+def test_spmm_decider_dims_all_cf(oracle, small, fmt, N):
+    from gpu_util import spmm_capi, spmm_oracle, spmm_abs_scale, assert_close
+    from oracle.oracle import CF_TABLE
+
+    F = small
+    print("case", fmt, N, flush=True)
+    X = np.random.default_rng(N).standard_normal((F.n + (F.n & 1), N)).astype(np.float32)
+    want = spmm_oracle(oracle, fmt, F, X)
+    scale = spmm_abs_scale(oracle, F, X, want.shape[0]) if "split" in fmt else None
+    Xd = torch.from_numpy(X).cuda()
+    for CF in CF_TABLE[N]:
+        for bw in (4, 8):
+            got = spmm_capi(fmt, F, Xd, CF, bw)
+            torch.cuda.synchronize()
+            assert_close(got, want, what="%s N=%d CF=%d bw=%d" % (fmt, N, CF, bw), scale=scale)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+@pytest.mark.parametrize("N", [1, 2, 3, 6, 8, 20, 50, 100, 250, 260, 513])
+def test_spmm_odd_widths(oracle, small, fmt, N):
+    from gpu_util import spmm_capi, spmm_oracle, spmm_abs_scale, assert_close
+
+    F = small
+    print("case", fmt, N, flush=True)
+    X = np.random.default_rng(N).standard_normal((F.n + (F.n & 1), N)).astype(np.float32)
+    want = spmm_oracle(oracle, fmt, F, X)
+    scale = spmm_abs_scale(oracle, F, X, want.shape[0]) if "split" in fmt else None
+    Xd = torch.from_numpy(X).cuda()
+    for CF in (1, 2, 3, 5, 8):
+        got = spmm_capi(fmt, F, Xd, CF, 4)
+        torch.cuda.synchronize()
+        assert_close(got, want, what="%s N=%d CF=%d" % (fmt, N, CF), scale=scale)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_spmm_ones_gives_row_sums(oracle, small, fmt):
+    """The reference's own known answer: X = ones -> every column holds the row sums (verification.py:26,43)."""
+    from gpu_util import spmm_capi, assert_close
+
+    F = small
+    X = torch.ones(F.n + (F.n & 1), 32, device="cuda")
+    got = spmm_capi(fmt, F, X, 1, 4)[: F.n]
+    rs = np.array([F.val[F.rowPtr[i]:F.rowPtr[i + 1]].astype(np.float64).sum() for i in range(F.n)])
+    # the reference's check: |ref - res| <= 1e-4 |ref|, exact zeros must match exactly (verification.py:82-84)
+    g = got.cpu().numpy().astype(np.float64)
+    assert np.all(np.abs(g - rs[:, None]) <= 1e-4 * np.abs(rs[:, None]))
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_spmm_edge_shapes(oracle, fmt):
+    """empty matrix, all rows empty, single row, one very long row, odd row count."""
+    from gpu_util import Formats, spmm_capi, spmm_oracle, spmm_abs_scale, assert_close
+
+    cases = {
+        "all_empty": (np.zeros(8, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32)),
+        "single": (np.array([0, 3], np.int32), np.array([0, 0, 0], np.int32)[:1].repeat(1), np.ones(1, np.float32)),
+        "long_row": random_csr(70, 1, 1, hub=(33, 70), values="uniform"),
+        "odd_rows": random_csr(129, 9, 2, values="uniform"),
+    }
+    cases["single"] = (np.array([0, 1], np.int32), np.array([0], np.int32), np.array([2.5], np.float32))
+    for name, (rowPtr, colIdx, val) in cases.items():
+        print("case", fmt, name, flush=True)
+        F = Formats(oracle, rowPtr, colIdx, val)
+        X = np.random.default_rng(0).standard_normal((F.n + (F.n & 1), 64)).astype(np.float32)
+        got = spmm_capi(fmt, F, torch.from_numpy(X).cuda(), 2, 8)
+        torch.cuda.synchronize()
+        want = spmm_oracle(oracle, fmt, F, X)
+        scale = spmm_abs_scale(oracle, F, X, want.shape[0]) if "split" in fmt else None
+        assert_close(got, want, what=fmt + " " + name, scale=scale)
+
+
+def test_spmm_bad_arguments_are_errors_not_crashes():
+    from paramspmm_ae_amd import _capi
+
+    x = torch.zeros(4, 16, device="cuda")
+    rp = torch.zeros(5, dtype=torch.int32, device="cuda")
+    p = _capi.ptr
+    for CF, bw in ((0, 4), (9, 4), (1, 5)):
+        rc = _capi.lib.psp_spmm_csr_f32(p(rp), None, None, p(x), p(x), 4, 16, 4, CF, bw, None)
+        assert rc == -1 and _capi.lib.psp_last_error()
+    assert _capi.lib.psp_spmm_csr_f32(p(rp), None, None, p(x), p(x), 4, 16, 2, 1, 4, None) == -1  # Y too short
+
+
+def test_spmm_linearity_and_format_agreement_at_scale(oracle):
+    """Size-independent properties on a 2^17-node R-MAT graph (too big for the scalar oracle to be quick at all
+    widths): the four formats agree, and A(X1+X2) = AX1 + AX2."""
+    from gpu_util import Formats, spmm_capi, assert_close
+    from paramspmm_ae_amd import synth
+
+    r, c, n = synth.rmat(17, 8 << 17, seed=5)
+    rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+    F = Formats(oracle, rowPtr, colIdx, val)
+    g = torch.Generator(device="cuda").manual_seed(1)
+    X1 = torch.randn(n, 128, device="cuda", generator=g)
+    X2 = torch.randn(n, 128, device="cuda", generator=g)
+    base = spmm_capi("csr", F, X1, 1, 4)
+    scale = spmm_capi("csr", F, X1.abs(), 1, 4).cpu().numpy()  # values are positive: this is |A||X|
+    for fmt in FMTS[1:]:
+        for CF in (1, 2, 4):
+            y = spmm_capi(fmt, F, X1, CF, 8)
+            assert_close(y, base.cpu().numpy(), what=fmt, scale=scale)
+    lin = spmm_capi("csr", F, X1 + X2, 2, 4)
+    assert_close(lin, (base + spmm_capi("csr", F, X2, 2, 4)).cpu().numpy(), rtol=1e-4, atol=1e-5, what="linearity")
+    # and one width against the oracle at this size
+    want = oracle.spmm_csr(rowPtr, colIdx, val, X1[:, :16].contiguous().cpu().numpy())
+    assert_close(spmm_capi("csr", F, X1[:, :16].contiguous(), 1, 4), want, what="rmat17 N=16")
