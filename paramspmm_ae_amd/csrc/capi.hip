@@ -294,7 +294,7 @@ PSP_EXPORT int psp_bcsr_build(const int *rowPtr, const int *colIdx, const float 
 PSP_EXPORT int psp_spmm_csr_f32(const int *rowPtr, const int *colIdx, const float *val, const float *X, float *Y,
                                 int M, int N, int rows_out, int CF, int blkWarpNum, psp_stream_t stream)
 {
-    return psp_spmm_launch<false, false>(rowPtr, colIdx, val, nullptr, X, Y, M, N, rows_out, CF, blkWarpNum,
+    return psp_spmm_launch<1, false>(rowPtr, colIdx, val, nullptr, X, Y, M, N, rows_out, CF, blkWarpNum,
                                          (hipStream_t)stream);
 }
 
@@ -302,14 +302,14 @@ PSP_EXPORT int psp_spmm_csr_split_f32(const int *rowPtr_split, const int *colIdx
                                       const int *target_row, const float *X, float *Y, int S, int N, int rows_out,
                                       int CF, int blkWarpNum, psp_stream_t stream)
 {
-    return psp_spmm_launch<false, true>(rowPtr_split, colIdx, val, target_row, X, Y, S, N, rows_out, CF, blkWarpNum,
+    return psp_spmm_launch<1, true>(rowPtr_split, colIdx, val, target_row, X, Y, S, N, rows_out, CF, blkWarpNum,
                                         (hipStream_t)stream);
 }
 
 PSP_EXPORT int psp_spmm_bcsr_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *X,
                                  float *Y, int Mb, int N, int rows_out, int CF, int blkWarpNum, psp_stream_t stream)
 {
-    return psp_spmm_launch<true, false>(rowPtr_b, colIdx_b, val_b, nullptr, X, Y, Mb, N, rows_out, CF, blkWarpNum,
+    return psp_spmm_launch<2, false>(rowPtr_b, colIdx_b, val_b, nullptr, X, Y, Mb, N, rows_out, CF, blkWarpNum,
                                         (hipStream_t)stream);
 }
 
@@ -317,7 +317,7 @@ PSP_EXPORT int psp_spmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b
                                        const int *target_row, const float *X, float *Y, int Sb, int N,
                                        int rows_out, int CF, int blkWarpNum, psp_stream_t stream)
 {
-    return psp_spmm_launch<true, true>(rowPtr_bs, colIdx_b, val_b, target_row, X, Y, Sb, N, rows_out, CF, blkWarpNum,
+    return psp_spmm_launch<2, true>(rowPtr_bs, colIdx_b, val_b, target_row, X, Y, Sb, N, rows_out, CF, blkWarpNum,
                                        (hipStream_t)stream);
 }
 

@@ -1,18 +1,25 @@
 // Parameterised SpMM kernel for gfx950 (wave64).  One template serves the four PCSR formats
 // (CSR / 2x1 BCSR, each plain or row-split).  Semantics follow the reference kernels
-// SpMM/SpMM_kernel.cu:1157-1651: per output element one fp32 FMA per stored non-zero, in storage order.
+// SpMM/SpMM_kernel.cu:1157-1651: per output element one fp32 FMA per stored non-zero, in storage order
+// (rows that are cut between lane groups or wavefronts are summed piecewise, see below).
 //
 // Work decomposition (what replaces "one 32-lane warp per row, CF columns per lane"):
-//   * a sparse row (or block-row, or row segment) is owned by a group of L = 2^logL lanes of a wavefront,
-//     so one wavefront carries 64/L rows;
+//   * a wavefront owns W = 2^logW consecutive segments (rows, block-rows or row-split segments), i.e. one
+//     contiguous range [P0,P1) of stored entries; their bounds and output rows sit in LDS;
+//   * the wavefront is cut into R = 64/L groups of L = 2^logL lanes; the range [P0,P1) is divided evenly
+//     between the groups, whatever the row lengths are, so a group walks ceil((P1-P0)/R) entries and
+//     writes a row out whenever it crosses a row end.  Skewed rows therefore cost no idle lanes;
 //   * every lane owns C column vectors of V floats (V = 4 -> global_load_dwordx4); vector i of lane s
 //     covers columns tile*L*C*V + (i*L + s)*V .. +V, so the L lanes of a group read L*V*4 contiguous bytes
 //     of an X row per load;
-//   * colIdx / values are read once per L non-zeros, coalesced (lane s takes non-zero base+s), and handed
+//   * colIdx / values are read once per L entries, coalesced (lane s takes entry base+s), and handed
 //     round the group with ds_bpermute; the next L are prefetched while the current ones are consumed;
-//   * U non-zeros are unrolled so U*C feature loads are in flight per lane before the first FMA.
+//   * U entries are unrolled so U*C feature loads are in flight per lane before the first FMA;
+//   * a row cut by a group boundary is summed across the groups in registers (ds_bpermute), in group order,
+//     so plain CSR needs neither atomics nor a cleared Y.  Only a row whose segments lie in several
+//     wavefronts (row-split formats) is accumulated with fp32 atomics, once per wavefront.
 // Tail columns (N not a multiple of L*C*V): loads are redirected to the last valid vector, stores are
-// predicated.  Lanes past the end of a row hold (last valid column, value 0).
+// predicated.  Lanes past the end of a group's range hold (last valid column, value 0).
 #pragma once
 #include "psp_common.h"
 
@@ -38,24 +45,103 @@ template <int V> __device__ __forceinline__ void psp_store_vec(float *p, const f
     *(typename psp_vec<V>::type *)p = t;
 }
 
-template <int C, int V, int U, bool BCSR, bool SPLIT>
+__device__ __forceinline__ int psp_bperm_i(int src_lane, int v) { return __builtin_amdgcn_ds_bpermute(src_lane << 2, v); }
+__device__ __forceinline__ float psp_bperm_f(int src_lane, float v)
+{
+    return __int_as_float(__builtin_amdgcn_ds_bpermute(src_lane << 2, __float_as_int(v)));
+}
+
+#define PSP_MAX_WAVES 8  // blkWarpNum is 4 or 8
+
+// NR: rows per stored entry (1 = CSR, 2 = 2x1 BCSR).  SPLIT: segments carry an explicit output row.
+template <int C, int V, int U, int NR, bool SPLIT>
 __global__ void __launch_bounds__(512)
 psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
                 const int *__restrict__ target_row, const float *__restrict__ X, float *__restrict__ Y,
-                int nrows, int N, int logL, int tiles, int chunk)
+                int nseg, int N, int logL, int logW, int tiles, int chunk)
 {
     typedef typename psp_vec<V>::type vec_t;
-    constexpr int NR = BCSR ? 2 : 1;
+    __shared__ int2 s_seg[PSP_MAX_WAVES][PSP_WAVE];  // (end offset, output row) of the wavefront's segments
 
     const int tile = psp_xcd_tile(chunk);
     if (tile >= tiles) return;
 
-    const int L = 1 << logL;
+    const int L = 1 << logL, W = 1 << logW;
     const int lane = threadIdx.x & (PSP_WAVE - 1);
     const int wave = threadIdx.x >> 6;
     const int sub = lane & (L - 1);
+    const int grp = lane >> logL;
     const int grp_base = lane - sub;
-    const int row = ((tile * (int)(blockDim.x >> 6) + wave) << (6 - logL)) + (lane >> logL);
+    const int s0 = (tile * (int)(blockDim.x >> 6) + wave) << logW;  // first segment of this wavefront
+    if (s0 >= nseg) return;                                         // wave-uniform
+    const int nvalid = min(W, nseg - s0);
+
+    // ---- segment table of this wavefront: only segments that hold entries, packed to the front ----------
+    const int P0 = rowPtr[s0];
+    const int P1 = rowPtr[s0 + nvalid];
+    {
+        const bool in = lane < nvalid;
+        const int e = in ? rowPtr[s0 + lane + 1] : P1;
+        const int e_up = __shfl_up(e, 1);  // cross-lane reads stay outside any lane-dependent branch
+        const int b_ = (lane == 0) ? P0 : e_up;
+        const bool filled = in && e != b_;
+        const unsigned long long fmask = __ballot(filled);
+        const int slot = __popcll(fmask & ((1ull << lane) - 1ull));
+        s_seg[wave][lane] = make_int2(P1, -1);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (filled) s_seg[wave][slot] = make_int2(e, SPLIT ? target_row[s0 + lane] : s0 + lane);
+        if constexpr (!SPLIT) {
+            // rows without entries are never visited below: write their zeros here, one row per lane group
+            unsigned long long empties = __ballot(in && e == b_);
+            int turn = 0;
+            while (empties) {
+                const int i = __ffsll((long long)empties) - 1;
+                empties &= empties - 1;
+                if ((turn++ & ((PSP_WAVE >> logL) - 1)) == grp) {
+                    const int tile_col0 = blockIdx.y * ((C * V) << logL);
+#pragma unroll
+                    for (int r = 0; r < NR; r++) {
+                        float *yr = Y + (size_t)((s0 + i) * NR + r) * (size_t)N;
+#pragma unroll
+                        for (int c = 0; c < C; c++) {
+                            const int col = tile_col0 + ((c << logL) + sub) * V;
+                            const float z[V] = {};
+                            if (col < N) psp_store_vec<V>(yr + col, z);
+                        }
+                    }
+                }
+            }
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int2 *w_seg = s_seg[wave];  // .x = end offset, .y = output row (block-row for NR = 2)
+    if (P0 == P1) return;
+
+    bool ext_head = false, ext_tail = false;  // the first / last row of this wavefront also has entries elsewhere
+    int tr_prev = -1, tr_next = -1;
+    if constexpr (SPLIT) {
+        if (s0 > 0) tr_prev = target_row[s0 - 1];
+        if (s0 + nvalid < nseg) tr_next = target_row[s0 + nvalid];
+    }
+
+    // ---- this group's share of [P0,P1) ---------------------------------------------------------------
+    const int R = PSP_WAVE >> logL;
+    const int q = (P1 - P0 + R - 1) >> (6 - logL);
+    int a = P0 + grp * q;
+    if (a > P1) a = P1;
+    const int b = min(P1, a + q);
+    const bool busy = a < b;
+
+    // segment that holds entry x: the first whose end exceeds x (unused table slots end at P1)
+    auto seg_of = [&](int x) {
+        int lo = 0;
+        for (int step = W >> 1; step >= 1; step >>= 1)
+            if (w_seg[lo + step - 1].x <= x) lo += step;
+        return lo;
+    };
 
     int off[C];
     bool live[C];
@@ -69,33 +155,60 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         }
     }
 
-    int lb = 0, hb = 0;
-    if (row < nrows) {
-        lb = rowPtr[row];
-        hb = rowPtr[row + 1];
-    }
-
-    float acc[NR][C][V];
+    float acc[NR][C][V], head[NR][C][V];
 #pragma unroll
     for (int r = 0; r < NR; r++)
 #pragma unroll
         for (int i = 0; i < C; i++)
 #pragma unroll
-            for (int e = 0; e < V; e++) acc[r][i][e] = 0.0f;
+            for (int e = 0; e < V; e++) acc[r][i][e] = head[r][i][e] = 0.0f;
 
-    int c_cur = 0;
-    float v_cur[NR];
+    // out: a finished row goes to Y; `shared` = other wavefronts add to the same row (row-split formats)
+    auto write_out = [&](int key, bool shared) {
 #pragma unroll
-    for (int r = 0; r < NR; r++) v_cur[r] = 0.0f;
+        for (int r = 0; r < NR; r++) {
+            float *yr = Y + (size_t)(key * NR + r) * (size_t)N;
+#pragma unroll
+            for (int i = 0; i < C; i++) {
+                if (!live[i]) continue;
+                if (!SPLIT || !shared) {
+                    psp_store_vec<V>(yr + off[i], acc[r][i]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < V; e++) unsafeAtomicAdd(yr + off[i] + e, acc[r][i][e]);
+                }
+            }
+        }
+    };
 
-    // lane `sub` of the group picks up non-zero base+sub; past the end: (last column of the row, 0)
+    enum { F_HEAD = 1, F_CLOSED = 2, F_SHARED = 4 };
+    int flags = 0;        // what `head` holds, for the groups before this one
+    bool has_tail = false;  // acc holds the start of a row that goes on in the next group
+    bool tail_shared = false;
+    int cur = 0, row_end = 0, mykey = -1;
+    bool first_run = true, head_valid = false;
+
+    if (busy) {
+        cur = seg_of(a);
+        const int2 sg = w_seg[cur];
+        row_end = sg.x;
+        mykey = sg.y;
+        const int seg_begin = cur == 0 ? P0 : w_seg[cur - 1].x;
+        head_valid = a > seg_begin;
+        if constexpr (SPLIT) {
+            if (!head_valid && cur > 0) head_valid = w_seg[cur - 1].y == mykey;
+            if (a == P0) ext_head = tr_prev == mykey;
+        }
+    }
+
+    // lane `sub` of the group picks up entry base+sub; past the end of the range: (last column, 0)
 #define PSP_FETCH(base, c_out, v_out)                                      \
     {                                                                      \
         const int p_ = (base) + sub;                                       \
-        const bool ok_ = p_ < hb;                                          \
-        const int pp_ = ok_ ? p_ : hb - 1;                                 \
+        const bool ok_ = p_ < b;                                           \
+        const int pp_ = ok_ ? p_ : b - 1;                                  \
         c_out = colIdx[pp_];                                               \
-        if constexpr (BCSR) {                                              \
+        if constexpr (NR == 2) {                                           \
             const psp_f32x2 t_ = ((const psp_f32x2 *)val)[pp_];            \
             v_out[0] = ok_ ? t_[0] : 0.0f;                                 \
             v_out[1] = ok_ ? t_[1] : 0.0f;                                 \
@@ -105,26 +218,30 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         }                                                                  \
     }
 
-    if (lb < hb) PSP_FETCH(lb, c_cur, v_cur);
+    int c_cur = 0;
+    float v_cur[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) v_cur[r] = 0.0f;
+    if (busy) PSP_FETCH(a, c_cur, v_cur);
 
-    for (int base = lb; base < hb; base += L) {
+    int p = a;
+    for (int base = a; base < b; base += L) {
         int c_nxt = 0;
         float v_nxt[NR];
 #pragma unroll
         for (int r = 0; r < NR; r++) v_nxt[r] = 0.0f;
-        if (base + L < hb) PSP_FETCH(base + L, c_nxt, v_nxt);
+        if (base + L < b) PSP_FETCH(base + L, c_nxt, v_nxt);
 
-        const int cnt = min(L, hb - base);
+        const int cnt = min(L, b - base);
         for (int k = 0; k < cnt; k += U) {
             int ck[U];
             float vk[U][NR];
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const int src = (grp_base + k + u) << 2;
-                ck[u] = __builtin_amdgcn_ds_bpermute(src, c_cur);
+                const int src = grp_base + k + u;
+                ck[u] = psp_bperm_i(src, c_cur);
 #pragma unroll
-                for (int r = 0; r < NR; r++)
-                    vk[u][r] = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(v_cur[r])));
+                for (int r = 0; r < NR; r++) vk[u][r] = psp_bperm_f(src, v_cur[r]);
             }
             vec_t x[U][C];
 #pragma unroll
@@ -134,18 +251,49 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
                 for (int i = 0; i < C; i++) x[u][i] = *(const vec_t *)(xr + off[i]);
             }
 #pragma unroll
-            for (int u = 0; u < U; u++)
+            for (int u = 0; u < U; u++) {
+                if (k + u < cnt) {
 #pragma unroll
-                for (int r = 0; r < NR; r++) {
-                    // 2x1 blocks: a zero entry is skipped (SpMM_kernel.cu:1399,1405)
-                    if (!BCSR || vk[u][r] != 0.0f) {
+                    for (int r = 0; r < NR; r++) {
+                        // 2x1 blocks: a zero entry is skipped (SpMM_kernel.cu:1399,1405)
+                        if (NR == 1 || vk[u][r] != 0.0f) {
 #pragma unroll
-                        for (int i = 0; i < C; i++)
+                            for (int i = 0; i < C; i++)
 #pragma unroll
-                            for (int e = 0; e < V; e++)
-                                acc[r][i][e] = __builtin_fmaf(vk[u][r], psp_elem<V>(x[u][i], e), acc[r][i][e]);
+                                for (int e = 0; e < V; e++)
+                                    acc[r][i][e] = __builtin_fmaf(vk[u][r], psp_elem<V>(x[u][i], e), acc[r][i][e]);
+                        }
+                    }
+                    p++;
+                    if (p == row_end && p < b) {
+                        // next segment (the table holds filled segments only, and p < b <= P1)
+                        const int2 nx = w_seg[++cur];
+                        row_end = nx.x;
+                        const int nkey = nx.y;
+                        if (nkey != mykey) {
+                            if (first_run && head_valid) {
+#pragma unroll
+                                for (int r = 0; r < NR; r++)
+#pragma unroll
+                                    for (int i = 0; i < C; i++)
+#pragma unroll
+                                        for (int e = 0; e < V; e++) head[r][i][e] = acc[r][i][e];
+                                flags = F_HEAD | F_CLOSED;
+                            } else {
+                                write_out(mykey, first_run && ext_head);
+                            }
+#pragma unroll
+                            for (int r = 0; r < NR; r++)
+#pragma unroll
+                                for (int i = 0; i < C; i++)
+#pragma unroll
+                                    for (int e = 0; e < V; e++) acc[r][i][e] = 0.0f;
+                            first_run = false;
+                            mykey = nkey;
+                        }
                     }
                 }
+            }
         }
         c_cur = c_nxt;
 #pragma unroll
@@ -153,35 +301,61 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     }
 #undef PSP_FETCH
 
-    if (row >= nrows) return;
-
-    if constexpr (!SPLIT) {
-        // every covered row is written, empty ones as zeros: the caller need not clear Y first
+    // ---- the row this group stopped in ----------------------------------------------------------------
+    if (busy) {
+        bool goes_on = false;  // does the row continue in the next group?
+        if (b < P1) {
+            if (b < row_end) goes_on = true;
+            else if (SPLIT) goes_on = w_seg[cur + 1].y == mykey;
+        }
+        if (SPLIT && b == P1) ext_tail = tr_next == mykey;
+        const bool partial_head = first_run && head_valid;
+        if (goes_on) {
+            if (partial_head) {
+                // the whole range lies inside one row that began earlier and goes on
 #pragma unroll
-        for (int r = 0; r < NR; r++) {
-            float *yr = Y + (size_t)(row * NR + r) * (size_t)N;
+                for (int r = 0; r < NR; r++)
+#pragma unroll
+                    for (int i = 0; i < C; i++)
+#pragma unroll
+                        for (int e = 0; e < V; e++) head[r][i][e] = acc[r][i][e];
+                flags = F_HEAD;
+            } else {
+                has_tail = true;
+                tail_shared = first_run && ext_head;
+            }
+        } else if (partial_head) {
+#pragma unroll
+            for (int r = 0; r < NR; r++)
+#pragma unroll
+                for (int i = 0; i < C; i++)
+#pragma unroll
+                    for (int e = 0; e < V; e++) head[r][i][e] = acc[r][i][e];
+            flags = F_HEAD | F_CLOSED | (ext_tail ? F_SHARED : 0);
+        } else {
+            write_out(mykey, (first_run && ext_head) || ext_tail);
+        }
+    }
+
+    // ---- rows cut by group boundaries: the group holding the start adds the following groups' heads ---
+    // (all lanes take part in every ds_bpermute; only groups with an open tail accumulate)
+    for (int d = 1; __ballot(has_tail) != 0ull; d++) {
+        const int src = lane + (d << logL);
+        const int src_c = src & (PSP_WAVE - 1);
+        const int hf_any = psp_bperm_i(src_c, flags);  // executed by every lane, then masked
+        const int hf = (src < PSP_WAVE) ? hf_any : 0;
+#pragma unroll
+        for (int r = 0; r < NR; r++)
 #pragma unroll
             for (int i = 0; i < C; i++)
-                if (live[i]) psp_store_vec<V>(yr + off[i], acc[r][i]);
-        }
-    } else {
-        if (lb == hb) return;
-        const int t = target_row[row];
-        const bool shared = (row > 0 && target_row[row - 1] == t) || (row + 1 < nrows && target_row[row + 1] == t);
 #pragma unroll
-        for (int r = 0; r < NR; r++) {
-            float *yr = Y + (size_t)(t * NR + r) * (size_t)N;
-#pragma unroll
-            for (int i = 0; i < C; i++) {
-                if (!live[i]) continue;
-                if (!shared) {
-                    // the only segment of its row: Y was cleared, a plain store equals 0 + partial
-                    psp_store_vec<V>(yr + off[i], acc[r][i]);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < V; e++) unsafeAtomicAdd(yr + off[i] + e, acc[r][i][e]);
+                for (int e = 0; e < V; e++) {
+                    const float h = psp_bperm_f(src_c, head[r][i][e]);
+                    if (has_tail && (hf & F_HEAD)) acc[r][i][e] += h;
                 }
-            }
+        if (has_tail && (!(hf & F_HEAD) || (hf & F_CLOSED) || src >= PSP_WAVE)) {
+            write_out(mykey, tail_shared || (hf & F_SHARED));
+            has_tail = false;
         }
     }
 }
@@ -194,16 +368,16 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     M_(5, 1) M_(6, 1) M_(7, 1) M_(8, 1)
 
 typedef void (*psp_spmm_kernel_t)(const int *, const int *, const float *, const int *, const float *, float *,
-                                  int, int, int, int, int);
+                                  int, int, int, int, int, int);
 
-template <bool BCSR, bool SPLIT>
+template <int NR, bool SPLIT>
 static psp_spmm_kernel_t psp_spmm_lookup(int C, int V, int U)
 {
-#define PSP_CASE(C_, U_)                                                          \
-    if (C == C_ && U == U_) {                                                     \
-        if (V == 4) return psp_spmm_kernel<C_, 4, U_, BCSR, SPLIT>;               \
-        if (V == 2) return psp_spmm_kernel<C_, 2, U_, BCSR, SPLIT>;               \
-        return psp_spmm_kernel<C_, 1, U_, BCSR, SPLIT>;                           \
+#define PSP_CASE(C_, U_)                                                        \
+    if (C == C_ && U == U_) {                                                   \
+        if (V == 4) return psp_spmm_kernel<C_, 4, U_, NR, SPLIT>;               \
+        if (V == 2) return psp_spmm_kernel<C_, 2, U_, NR, SPLIT>;               \
+        return psp_spmm_kernel<C_, 1, U_, NR, SPLIT>;                           \
     }
     PSP_SPMM_FOR_EACH_CU(PSP_CASE)
 #undef PSP_CASE
@@ -211,7 +385,7 @@ static psp_spmm_kernel_t psp_spmm_lookup(int C, int V, int U)
 }
 
 // nrows: rows / block-rows / segments.  Y rows covered: nrows*NR (plain) or all of rows_out (split, cleared first).
-template <bool BCSR, bool SPLIT>
+template <int NR, bool SPLIT>
 int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
                     const float *X, float *Y, int nrows, int N, int rows_out, int CF, int blkWarpNum,
                     hipStream_t stream);

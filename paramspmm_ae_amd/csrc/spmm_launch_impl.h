@@ -2,12 +2,11 @@
 #pragma once
 #include "spmm_kernel.h"
 
-template <bool BCSR, bool SPLIT>
+template <int NR, bool SPLIT>
 int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
                     const float *X, float *Y, int nrows, int N, int rows_out, int CF, int blkWarpNum,
                     hipStream_t stream)
 {
-    constexpr int NR = BCSR ? 2 : 1;
     psp_spmm_plan plan;
     int rc = psp_spmm_plan_for(N, CF, blkWarpNum, &plan);
     if (rc != PSP_OK) return rc;
@@ -33,12 +32,18 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
 
     int logL = 0;
     while ((1 << logL) < plan.lanes_per_row) logL++;
-    psp_spmm_kernel_t k = psp_spmm_lookup<BCSR, SPLIT>(plan.coarsen, plan.vec, plan.unroll);
+    psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll);
     if (!k) return psp_fail(PSP_ERR_ARG, "spmm: no kernel for coarsen %d vec %d unroll %d", plan.coarsen, plan.vec, plan.unroll);
 
-    const int rows_per_block = plan.waves_per_block * plan.rows_per_wave;
-    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, rows_per_block));
+    // segments per wavefront: 64 when that still leaves thousands of wavefronts, fewer for small matrices,
+    // but not so few that most lane groups of a wavefront would find nothing to do
+    int logW = 6;
+    while (logW > 0 && (nrows >> logW) < 4096) logW--;
+    const int logR = 6 - logL;
+    if (logW < logR - 1) logW = logR - 1;
+    const int segs_per_block = plan.waves_per_block << logW;
+    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block));
     dim3 grid(g.launch, plan.col_tiles, 1), block(plan.waves_per_block * PSP_WAVE, 1, 1);
-    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, g.real, g.chunk);
+    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.chunk);
     return psp_check_launch("spmm kernel");
 }

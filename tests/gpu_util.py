@@ -101,9 +101,10 @@ def sddmm_oracle(oracle, fmt, F, A, B):
 
 
 def spmm_abs_scale(oracle, F, X, rows_out):
-    """(|A| |X|): the magnitude a row's terms add up to.  Row-split formats accumulate the segments of a long
-    row with atomics in no fixed order (as the reference does), so their rounding error scales with this sum
-    of magnitudes and not with the possibly cancelled result."""
+    """(|A| |X|): the magnitude a row's terms add up to.  A long row is summed piecewise (lane groups of a
+    wavefront each take a share of it; row-split formats add segments with atomics in no fixed order, as the
+    reference does), so the rounding error scales with this sum of magnitudes and not with the possibly
+    cancelled result."""
     return oracle.spmm_csr(F.rowPtr, F.colIdx, np.abs(F.val), np.abs(X), rows_out=rows_out)
 
 

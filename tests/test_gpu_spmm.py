@@ -29,7 +29,7 @@ def test_spmm_decider_dims_all_cf(oracle, small, fmt, N):
     print("case", fmt, N, flush=True)
     X = np.random.default_rng(N).standard_normal((F.n + (F.n & 1), N)).astype(np.float32)
     want = spmm_oracle(oracle, fmt, F, X)
-    scale = spmm_abs_scale(oracle, F, X, want.shape[0]) if "split" in fmt else None
+    scale = spmm_abs_scale(oracle, F, X, want.shape[0])
     Xd = torch.from_numpy(X).cuda()
     for CF in CF_TABLE[N]:
         for bw in (4, 8):
@@ -47,7 +47,7 @@ def test_spmm_odd_widths(oracle, small, fmt, N):
     print("case", fmt, N, flush=True)
     X = np.random.default_rng(N).standard_normal((F.n + (F.n & 1), N)).astype(np.float32)
     want = spmm_oracle(oracle, fmt, F, X)
-    scale = spmm_abs_scale(oracle, F, X, want.shape[0]) if "split" in fmt else None
+    scale = spmm_abs_scale(oracle, F, X, want.shape[0])
     Xd = torch.from_numpy(X).cuda()
     for CF in (1, 2, 3, 5, 8):
         got = spmm_capi(fmt, F, Xd, CF, 4)
@@ -88,7 +88,7 @@ def test_spmm_edge_shapes(oracle, fmt):
         got = spmm_capi(fmt, F, torch.from_numpy(X).cuda(), 2, 8)
         torch.cuda.synchronize()
         want = spmm_oracle(oracle, fmt, F, X)
-        scale = spmm_abs_scale(oracle, F, X, want.shape[0]) if "split" in fmt else None
+        scale = spmm_abs_scale(oracle, F, X, want.shape[0])
         assert_close(got, want, what=fmt + " " + name, scale=scale)
 
 
