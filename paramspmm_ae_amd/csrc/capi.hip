@@ -4,6 +4,7 @@
 #include <thread>
 #include <vector>
 #include <string.h>
+#include <stdlib.h>
 #include "psp_common.h"
 #include "spmm_kernel.h"
 #include "sddmm_kernel.h"
@@ -20,6 +21,16 @@ int psp_fail(int code, const char *fmt, ...)
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
     return code;
+}
+
+int psp_stripe_rows(void)
+{
+    static int rows = [] {
+        const char *e = getenv("PSP_XCD_STRIPE_ROWS");
+        const int v = e ? atoi(e) : 0;
+        return v > 0 ? v : 8192;
+    }();
+    return rows;
 }
 
 PSP_EXPORT const char *psp_last_error(void) { return g_err; }
@@ -39,6 +50,10 @@ PSP_EXPORT int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *p
     int C = std::min(CF, nvec);
     int L = 1;
     while (L < PSP_WAVE && L * C < nvec) L <<= 1;
+    if (const char *e = getenv("PSP_FORCE_LANES")) {  // tuning aid: narrower groups -> column tiles
+        const int f = atoi(e);
+        if (f >= 1 && f <= 64 && (f & (f - 1)) == 0 && f < L) L = f;
+    }
     // in-flight budget: about 8 feature vectors per lane
     int U = C == 1 ? 8 : C == 2 ? 4 : C <= 4 ? 2 : 1;
     while (U > L) U >>= 1;

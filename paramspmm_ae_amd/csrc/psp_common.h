@@ -27,24 +27,33 @@ static inline int psp_check_launch(const char *what)
 
 static inline int psp_ceil_div(long long a, long long b) { return (int)((a + b - 1) / b); }
 
-// Workgroups are handed to the 8 XCDs round-robin by linear workgroup id.  Launching
-// PSP_XCDS*chunk workgroups and giving workgroup b the logical tile (b%8)*chunk + b/8 makes each XCD
-// (one L2) work on one contiguous band of sparse rows, so neighbouring rows that gather the same rows
-// of X find them in the same L2.
+// Workgroups are handed to the 8 XCDs round-robin by linear workgroup id.  To give each XCD (one L2) runs of
+// neighbouring sparse rows -- so that rows which gather the same rows of X find them in the same L2 -- the
+// logical tiles are dealt out in stripes: XCD x works on tiles [s*8*G + x*G, s*8*G + (x+1)*G) for s = 0,1,..
+// (G = tiles per stripe).  Stripes are short enough (a few thousand rows) that a matrix whose long rows
+// cluster in one index range still spreads over all XCDs.  G = 1 is the identity mapping.
 struct psp_grid1d {
-    int real;   // logical tiles
-    int chunk;  // tiles per XCD
-    int launch; // workgroups launched (>= real)
+    int real;    // logical tiles
+    int stripe;  // G: consecutive tiles that go to one XCD
+    int launch;  // workgroups launched (>= real, a multiple of 8*G)
 };
-static inline psp_grid1d psp_xcd_grid(int tiles)
+static inline psp_grid1d psp_xcd_grid(int tiles, int stripe)
 {
     psp_grid1d g;
     g.real = tiles;
-    g.chunk = (tiles + PSP_XCDS - 1) / PSP_XCDS;
-    g.launch = g.chunk * PSP_XCDS;
+    const int band = (tiles + PSP_XCDS - 1) / PSP_XCDS;  // one stripe per XCD is the widest useful setting
+    g.stripe = stripe < 1 ? 1 : (stripe > band ? (band < 1 ? 1 : band) : stripe);
+    const int round = PSP_XCDS * g.stripe;
+    g.launch = (tiles + round - 1) / round * round;
     return g;
 }
-__device__ __forceinline__ int psp_xcd_tile(int chunk) { return (blockIdx.x % PSP_XCDS) * chunk + blockIdx.x / PSP_XCDS; }
+__device__ __forceinline__ int psp_xcd_tile(int stripe)
+{
+    const int xcd = blockIdx.x % PSP_XCDS, idx = blockIdx.x / PSP_XCDS;
+    return ((idx / stripe) * PSP_XCDS + xcd) * stripe + idx % stripe;
+}
+// rows (or segments) one stripe should span; PSP_XCD_STRIPE_ROWS in the environment overrides it (tuning aid)
+int psp_stripe_rows(void);
 
 // zero-fill used instead of hipMemsetAsync (callers may capture these launches in a HIP graph)
 int psp_zero_f32(float *p, size_t n, hipStream_t stream);

@@ -34,14 +34,14 @@ template <int LOGL, int C, int V, int U, bool BCSR, bool SPLIT, bool SCALE>
 __global__ void __launch_bounds__(512)
 psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
                  const int *__restrict__ target_row, const float *__restrict__ A, const float *__restrict__ B,
-                 float *__restrict__ out, int nrows, int K, int tiles, int chunk)
+                 float *__restrict__ out, int nrows, int K, int tiles, int stripe)
 {
     typedef typename psp_vec<V>::type vec_t;
     constexpr int NR = BCSR ? 2 : 1;
     constexpr int L = 1 << LOGL;
     static_assert(U <= L, "unroll must not exceed the group width");
 
-    const int tile = psp_xcd_tile(chunk);
+    const int tile = psp_xcd_tile(stripe);
     if (tile >= tiles) return;
 
     const int lane = threadIdx.x & (PSP_WAVE - 1);

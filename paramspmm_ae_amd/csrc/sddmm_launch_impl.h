@@ -29,9 +29,9 @@ int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, con
     if (!k) return psp_fail(PSP_ERR_ARG, "sddmm: no kernel for logL %d coarsen %d vec %d", logL, C, V);
 
     const int rows_per_block = blkWarpNum * (PSP_WAVE >> logL);
-    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, rows_per_block));
+    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, rows_per_block), psp_stripe_rows() / rows_per_block);
     dim3 grid(g.launch, 1, 1), block(blkWarpNum * PSP_WAVE, 1, 1);
     hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, BCSR ? val : scale, target_row, A, B, out, nrows, K,
-                       g.real, g.chunk);
+                       g.real, g.stripe);
     return psp_check_launch("sddmm kernel");
 }

@@ -58,12 +58,12 @@ template <int C, int V, int U, int NR, bool SPLIT>
 __global__ void __launch_bounds__(512)
 psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
                 const int *__restrict__ target_row, const float *__restrict__ X, float *__restrict__ Y,
-                int nseg, int N, int logL, int logW, int tiles, int chunk)
+                int nseg, int N, int logL, int logW, int tiles, int stripe, int align_pct)
 {
     typedef typename psp_vec<V>::type vec_t;
     __shared__ int2 s_seg[PSP_MAX_WAVES][PSP_WAVE];  // (end offset, output row) of the wavefront's segments
 
-    const int tile = psp_xcd_tile(chunk);
+    const int tile = psp_xcd_tile(stripe);
     if (tile >= tiles) return;
 
     const int L = 1 << logL, W = 1 << logW;
@@ -79,9 +79,11 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     // ---- segment table of this wavefront: only segments that hold entries, packed to the front ----------
     const int P0 = rowPtr[s0];
     const int P1 = rowPtr[s0 + nvalid];
+    int e_lane;  // end offset of segment `lane` of this wavefront
     {
         const bool in = lane < nvalid;
         const int e = in ? rowPtr[s0 + lane + 1] : P1;
+        e_lane = e;
         const int e_up = __shfl_up(e, 1);  // cross-lane reads stay outside any lane-dependent branch
         const int b_ = (lane == 0) ? P0 : e_up;
         const bool filled = in && e != b_;
@@ -128,11 +130,28 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     }
 
     // ---- this group's share of [P0,P1) ---------------------------------------------------------------
+    // Even division by default.  When giving every group whole segments (W/R each) costs at most align_pct
+    // percent more steps than that, the segments are not cut: neighbouring rows then advance together and no
+    // partial sums have to be merged.
     const int R = PSP_WAVE >> logL;
     const int q = (P1 - P0 + R - 1) >> (6 - logL);
     int a = P0 + grp * q;
     if (a > P1) a = P1;
-    const int b = min(P1, a + q);
+    int b = min(P1, a + q);
+    if (logW + logL >= 6) {
+        const int m = 1 << (logW + logL - 6);  // segments per group
+        const int first = grp * m;
+        const int a_up = psp_bperm_i((first + PSP_WAVE - 1) & (PSP_WAVE - 1), e_lane);
+        const int a_al = first == 0 ? P0 : a_up;
+        const int b_al = psp_bperm_i(first + m - 1, e_lane);
+        int longest = b_al - a_al;
+#pragma unroll
+        for (int d = 1; d < PSP_WAVE; d <<= 1) longest = max(longest, psp_bperm_i(lane ^ d, longest));
+        if ((long long)longest * 100 <= (long long)q * (100 + align_pct)) {
+            a = a_al;
+            b = b_al;
+        }
+    }
     const bool busy = a < b;
 
     // segment that holds entry x: the first whose end exceeds x (unused table slots end at P1)
@@ -182,7 +201,8 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     };
 
     enum { F_HEAD = 1, F_CLOSED = 2, F_SHARED = 4 };
-    int flags = 0;        // what `head` holds, for the groups before this one
+    // what `head` holds, for the groups before this one; a group without entries passes a row on unchanged
+    int flags = busy ? 0 : F_HEAD;
     bool has_tail = false;  // acc holds the start of a row that goes on in the next group
     bool tail_shared = false;
     int cur = 0, row_end = 0, mykey = -1;
@@ -224,7 +244,40 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     for (int r = 0; r < NR; r++) v_cur[r] = 0.0f;
     if (busy) PSP_FETCH(a, c_cur, v_cur);
 
-    int p = a;
+    // One step of the walk: U entries starting at chunk position k, all of the current row.  `guard` keeps
+    // entries past run_end (they belong to the next row or lie past the range) out of the sums.
+#define PSP_BATCH(GUARDED)                                                                          \
+    {                                                                                               \
+        int ck[U];                                                                                  \
+        float vk[U][NR];                                                                            \
+        _Pragma("unroll") for (int u = 0; u < U; u++)                                               \
+        {                                                                                           \
+            const int src = grp_base + min(k + u, L - 1);                                           \
+            ck[u] = psp_bperm_i(src, c_cur);                                                        \
+            _Pragma("unroll") for (int r = 0; r < NR; r++) vk[u][r] = psp_bperm_f(src, v_cur[r]);   \
+        }                                                                                           \
+        vec_t x[U][C];                                                                              \
+        _Pragma("unroll") for (int u = 0; u < U; u++)                                               \
+        {                                                                                           \
+            const float *xr = X + (size_t)ck[u] * (size_t)N;                                        \
+            _Pragma("unroll") for (int i = 0; i < C; i++) x[u][i] = *(const vec_t *)(xr + off[i]);  \
+        }                                                                                           \
+        _Pragma("unroll") for (int u = 0; u < U; u++)                                               \
+        {                                                                                           \
+            if (!(GUARDED) || k + u < run_end) {                                                    \
+                _Pragma("unroll") for (int r = 0; r < NR; r++)                                      \
+                {                                                                                   \
+                    /* 2x1 blocks: a zero entry is skipped (SpMM_kernel.cu:1399,1405) */            \
+                    if (NR == 1 || vk[u][r] != 0.0f) {                                              \
+                        _Pragma("unroll") for (int i = 0; i < C; i++)                               \
+                            _Pragma("unroll") for (int e = 0; e < V; e++)                           \
+                                acc[r][i][e] = __builtin_fmaf(vk[u][r], psp_elem<V>(x[u][i], e), acc[r][i][e]); \
+                    }                                                                               \
+                }                                                                                   \
+            }                                                                                       \
+        }                                                                                           \
+    }
+
     for (int base = a; base < b; base += L) {
         int c_nxt = 0;
         float v_nxt[NR];
@@ -233,65 +286,39 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         if (base + L < b) PSP_FETCH(base + L, c_nxt, v_nxt);
 
         const int cnt = min(L, b - base);
-        for (int k = 0; k < cnt; k += U) {
-            int ck[U];
-            float vk[U][NR];
+        int k = 0;
+        while (k < cnt) {
+            // the current row's entries inside this chunk: positions [k, run_end)
+            const int run_end = min(cnt, row_end - base);
+            for (; k + U <= run_end; k += U) PSP_BATCH(false)
+            if (k < run_end) PSP_BATCH(true)
+            k = run_end;
+            const int p = base + k;
+            if (p == row_end && p < b) {
+                // next segment (the table holds filled segments only, and p < b <= P1)
+                const int2 nx = w_seg[++cur];
+                row_end = nx.x;
+                const int nkey = nx.y;
+                if (nkey != mykey) {
+                    if (first_run && head_valid) {
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                const int src = grp_base + k + u;
-                ck[u] = psp_bperm_i(src, c_cur);
-#pragma unroll
-                for (int r = 0; r < NR; r++) vk[u][r] = psp_bperm_f(src, v_cur[r]);
-            }
-            vec_t x[U][C];
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                const float *xr = X + (size_t)ck[u] * (size_t)N;
-#pragma unroll
-                for (int i = 0; i < C; i++) x[u][i] = *(const vec_t *)(xr + off[i]);
-            }
-#pragma unroll
-            for (int u = 0; u < U; u++) {
-                if (k + u < cnt) {
-#pragma unroll
-                    for (int r = 0; r < NR; r++) {
-                        // 2x1 blocks: a zero entry is skipped (SpMM_kernel.cu:1399,1405)
-                        if (NR == 1 || vk[u][r] != 0.0f) {
+                        for (int r = 0; r < NR; r++)
 #pragma unroll
                             for (int i = 0; i < C; i++)
 #pragma unroll
-                                for (int e = 0; e < V; e++)
-                                    acc[r][i][e] = __builtin_fmaf(vk[u][r], psp_elem<V>(x[u][i], e), acc[r][i][e]);
-                        }
+                                for (int e = 0; e < V; e++) head[r][i][e] = acc[r][i][e];
+                        flags = F_HEAD | F_CLOSED;
+                    } else {
+                        write_out(mykey, first_run && ext_head);
                     }
-                    p++;
-                    if (p == row_end && p < b) {
-                        // next segment (the table holds filled segments only, and p < b <= P1)
-                        const int2 nx = w_seg[++cur];
-                        row_end = nx.x;
-                        const int nkey = nx.y;
-                        if (nkey != mykey) {
-                            if (first_run && head_valid) {
 #pragma unroll
-                                for (int r = 0; r < NR; r++)
+                    for (int r = 0; r < NR; r++)
 #pragma unroll
-                                    for (int i = 0; i < C; i++)
+                        for (int i = 0; i < C; i++)
 #pragma unroll
-                                        for (int e = 0; e < V; e++) head[r][i][e] = acc[r][i][e];
-                                flags = F_HEAD | F_CLOSED;
-                            } else {
-                                write_out(mykey, first_run && ext_head);
-                            }
-#pragma unroll
-                            for (int r = 0; r < NR; r++)
-#pragma unroll
-                                for (int i = 0; i < C; i++)
-#pragma unroll
-                                    for (int e = 0; e < V; e++) acc[r][i][e] = 0.0f;
-                            first_run = false;
-                            mykey = nkey;
-                        }
-                    }
+                            for (int e = 0; e < V; e++) acc[r][i][e] = 0.0f;
+                    first_run = false;
+                    mykey = nkey;
                 }
             }
         }
@@ -299,6 +326,7 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
 #pragma unroll
         for (int r = 0; r < NR; r++) v_cur[r] = v_nxt[r];
     }
+#undef PSP_BATCH
 #undef PSP_FETCH
 
     // ---- the row this group stopped in ----------------------------------------------------------------
@@ -368,7 +396,7 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     M_(5, 1) M_(6, 1) M_(7, 1) M_(8, 1)
 
 typedef void (*psp_spmm_kernel_t)(const int *, const int *, const float *, const int *, const float *, float *,
-                                  int, int, int, int, int, int);
+                                  int, int, int, int, int, int, int);
 
 template <int NR, bool SPLIT>
 static psp_spmm_kernel_t psp_spmm_lookup(int C, int V, int U)

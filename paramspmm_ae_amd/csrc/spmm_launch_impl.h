@@ -1,5 +1,6 @@
 // Host launcher shared by the four SpMM translation units (one per format, to compile in parallel).
 #pragma once
+#include <stdlib.h>
 #include "spmm_kernel.h"
 
 template <int NR, bool SPLIT>
@@ -35,15 +36,24 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll);
     if (!k) return psp_fail(PSP_ERR_ARG, "spmm: no kernel for coarsen %d vec %d unroll %d", plan.coarsen, plan.vec, plan.unroll);
 
-    // segments per wavefront: 64 when that still leaves thousands of wavefronts, fewer for small matrices,
-    // but not so few that most lane groups of a wavefront would find nothing to do
-    int logW = 6;
-    while (logW > 0 && (nrows >> logW) < 4096) logW--;
+    // Segments per wavefront.  Row-split input means the caller expects skewed rows: 64 segments per wavefront
+    // give the lane groups long, even shares and fold up to 64 partial sums of a long row before one atomic.
+    // Plain input gets one row per lane group on average: rows that are neighbours in the matrix are then walked
+    // at the same time and share their X rows in the L1 / L2, while the even division of the wavefront's entries
+    // still levels moderate differences in row length.  Small matrices use fewer segments per wavefront so
+    // that there are wavefronts for every SIMD.
     const int logR = 6 - logL;
+    int logW = SPLIT ? 6 : logR;
+    const char *w_env = getenv("PSP_LOG_SEGS_PER_WAVE");  // tuning aid
+    if (w_env && atoi(w_env) >= 0 && atoi(w_env) <= 6) logW = atoi(w_env);
+    while (logW > 0 && (nrows >> logW) < 4096) logW--;
     if (logW < logR - 1) logW = logR - 1;
+    int align_pct = 50;
+    const char *a_env = getenv("PSP_ALIGN_PCT");  // tuning aid
+    if (a_env) align_pct = atoi(a_env);
     const int segs_per_block = plan.waves_per_block << logW;
-    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block));
+    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block), psp_stripe_rows() / segs_per_block);
     dim3 grid(g.launch, plan.col_tiles, 1), block(plan.waves_per_block * PSP_WAVE, 1, 1);
-    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.chunk);
+    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.stripe, align_pct);
     return psp_check_launch("spmm kernel");
 }
