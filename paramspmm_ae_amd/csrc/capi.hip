@@ -45,17 +45,25 @@ PSP_EXPORT int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *p
     PSP_REQUIRE(N >= 1, "feature dimension must be positive (got %d)", N);
     PSP_REQUIRE(CF >= 1 && CF <= 8, "CF must be 1..8 (got %d)", CF);
     PSP_REQUIRE(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8 (got %d)", blkWarpNum);
+    // A lane group owns a tile of 32*CF columns, as the reference's warp does (CF columns per lane of a 32-lane
+    // warp, SpMM_kernel.cu:162-165); the remaining columns go to further column tiles (grid.y).  Natively the
+    // 32-column slab is 8 lanes x float4 (16 x float2 / 32 x float when N is not a multiple of 4) and CF is the
+    // number of such vectors per lane, so a wavefront carries 8 rows whatever CF is.
     const int V = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
     const int nvec = N / V;
     int C = std::min(CF, nvec);
-    int L = 1;
-    while (L < PSP_WAVE && L * C < nvec) L <<= 1;
-    if (const char *e = getenv("PSP_FORCE_LANES")) {  // tuning aid: narrower groups -> column tiles
+    int L = 32 / V;
+    while (L > 1 && (L / 2) * C >= nvec) L >>= 1;  // one tile already covers N: no wider than needed
+    if (const char *e = getenv("PSP_FORCE_LANES")) {  // tuning aid
         const int f = atoi(e);
-        if (f >= 1 && f <= 64 && (f & (f - 1)) == 0 && f < L) L = f;
+        if (f >= 1 && f <= 64 && (f & (f - 1)) == 0) L = f;
     }
-    // in-flight budget: about 8 feature vectors per lane
-    int U = C == 1 ? 8 : C == 2 ? 4 : C <= 4 ? 2 : 1;
+    // feature vectors in flight per lane: U entries x C vectors
+    int U = C == 1 ? 4 : C <= 4 ? 2 : 1;
+    if (const char *e = getenv("PSP_FORCE_UNROLL")) {  // tuning aid
+        const int f = atoi(e);
+        if (f == 1 || f == 2 || f == 4 || f == 8) U = (C * f <= 8) ? f : U;
+    }
     while (U > L) U >>= 1;
     plan->vec = V;
     plan->coarsen = C;

@@ -36,14 +36,15 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll);
     if (!k) return psp_fail(PSP_ERR_ARG, "spmm: no kernel for coarsen %d vec %d unroll %d", plan.coarsen, plan.vec, plan.unroll);
 
-    // Segments per wavefront.  Row-split input means the caller expects skewed rows: 64 segments per wavefront
-    // give the lane groups long, even shares and fold up to 64 partial sums of a long row before one atomic.
-    // Plain input gets one row per lane group on average: rows that are neighbours in the matrix are then walked
-    // at the same time and share their X rows in the L1 / L2, while the even division of the wavefront's entries
-    // still levels moderate differences in row length.  Small matrices use fewer segments per wavefront so
-    // that there are wavefronts for every SIMD.
+    // Segments per wavefront.  Plain input gets one row per lane group on average: rows that are neighbours in
+    // the matrix are then walked at the same time and share their X rows in the L1 / L2, while the even division
+    // of the wavefront's entries still levels moderate differences in row length.  Row-split input means the
+    // caller expects skewed rows: 16 segments per wavefront give the lane groups longer, even shares and fold the
+    // partial sums of a long row before the single atomic per wavefront (measured on a scale-20 R-MAT graph:
+    // 16 beats 8, 32 and 64 at every width).  Small matrices use fewer segments per wavefront so that there are
+    // wavefronts for every SIMD.
     const int logR = 6 - logL;
-    int logW = SPLIT ? 6 : logR;
+    int logW = SPLIT ? (logR > 4 ? logR : 4) : logR;
     const char *w_env = getenv("PSP_LOG_SEGS_PER_WAVE");  // tuning aid
     if (w_env && atoi(w_env) >= 0 && atoi(w_env) <= 6) logW = atoi(w_env);
     while (logW > 0 && (nrows >> logW) < 4096) logW--;
