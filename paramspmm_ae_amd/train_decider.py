@@ -1,0 +1,277 @@
+#!/usr/bin/env python3
+"""Retrains the SpMM-decider on MI355X timings of synthetic matrices.
+
+Counterpart of the reference's training-set construction (PCSR.py:672-823, script/1_construct_training_set.sh)
+and of its training notebook (models/rnd_tree.ipynb cells 3-21), with synthetic matrices instead of the
+SuiteSparse / OGB collection the reference downloads.
+
+  sweep  (GPU)  for every matrix of the corpus: build the PCSR formats, record the 15 decider features and time
+                every <representation, CF, blkWarpNum> at every width 16..256 -> csv files with the reference's
+                schema: mtx_info.csv, dim<N>.csv (GFLOP/s per column), dim<N>_OP_SpMM.csv (features + arg-max
+                column = class code).
+  fit    (CPU)  80/20 split, one RandomForestClassifier per width -> rnd_tree_<N>.pkl, and a report with the
+                reference's two statistics (test accuracy, mean normalised performance) plus the share of test
+                matrices whose pick is within 10 % of the best swept configuration.
+
+    python -m paramspmm_ae_amd.train_decider sweep --out gpurun_out/decider [--part 0/3]
+    python -m paramspmm_ae_amd.train_decider fit --data paramspmm_ae_amd/models/train_data --out paramspmm_ae_amd/models
+"""
+import argparse
+import json
+import os
+import pickle
+import sys
+import time
+
+import numpy as np
+
+DIMS = list(range(16, 257, 16))
+FEATURES = [
+    "graph_nodes", "graph_edges", "graph_density", "csr_max_row_nnz", "csr_real_nrow", "csr_nonempty_rate",
+    "csr_avg_degree", "csr_COV", "csr_real_avg_degree", "csr_real_COV", "csr_max_bw", "csr_avg_bw",
+    "csr_split_ratio", "bcsr_split_ratio", "pack_rate",
+]
+NNZ_CAP = 24_000_000
+
+
+# ------------------------------------------------------------------------------------------------------------
+# corpus
+# ------------------------------------------------------------------------------------------------------------
+def banded(n, k, width, seed):
+    """k random neighbours per node inside a band of +-width around the diagonal."""
+    rng = np.random.default_rng(seed)
+    u = np.repeat(np.arange(n, dtype=np.int64), k)
+    v = u + rng.integers(-width, width + 1, u.size)
+    np.clip(v, 0, n - 1, out=v)
+    return u, v, n
+
+
+def grid_with_holes(nx, ny, drop, seed):
+    """2-D 5-point grid with a fraction of the edges removed (road-network like: degree 2-4, high diameter)."""
+    from . import synth
+
+    r, c, n = synth.stencil2d(nx, ny)
+    keep = np.random.default_rng(seed).random(r.size) >= drop
+    return r[keep], c[keep], n
+
+
+def corpus():
+    """Deterministic list of (name, builder) covering power-law, R-MAT, community, mesh and banded structure."""
+    from . import synth
+
+    items = []
+    rng = np.random.default_rng(2024)
+
+    def add(name, fn):
+        items.append((name, fn))
+
+    # Chung-Lu power law
+    for n in (10_000, 20_000, 60_000, 200_000, 600_000, 1_500_000):
+        for avg in (3, 6, 12, 25, 50):
+            if n * avg > NNZ_CAP:
+                continue
+            for expo in (1.8, 2.1, 2.4, 3.0):
+                if rng.random() < 0.2:
+                    continue
+                maxd = int(min(n // 4, rng.choice([200, 2000, 20000])))
+                perm = bool(rng.random() < 0.7)
+                seed = int(rng.integers(1 << 30))
+                add("cl_n%d_d%d_e%.1f_m%d_%s" % (n, avg, expo, maxd, "p" if perm else "s"),
+                    lambda n=n, avg=avg, expo=expo, maxd=maxd, perm=perm, seed=seed:
+                    synth.chung_lu(n, n * avg // 2, exponent=expo, max_degree=maxd, seed=seed, permute=perm))
+    # R-MAT, from Graph500-like skew to Erdos-Renyi
+    for scale in (13, 15, 16, 17, 18, 19, 20):
+        for ef in (2, 4, 8, 16, 32):
+            if (1 << scale) * ef * 2 > NNZ_CAP:
+                continue
+            for abc in ((0.57, 0.19, 0.19), (0.5, 0.2, 0.2), (0.45, 0.22, 0.22), (0.35, 0.25, 0.25), (0.25, 0.25, 0.25)):
+                if rng.random() < 0.1:
+                    continue
+                seed = int(rng.integers(1 << 30))
+                add("rmat_s%d_e%d_a%.2f" % (scale, ef, abc[0]),
+                    lambda scale=scale, ef=ef, abc=abc, seed=seed: synth.rmat(scale, ef << scale, *abc, seed=seed))
+    # stochastic block models, community-ordered and permuted
+    for n in (20_000, 50_000, 200_000, 500_000, 1_000_000):
+        for size in (20, 50, 100, 500, 2000):
+            for din, dout in ((5, 0.5), (20, 2), (40, 8), (10, 10), (3, 3)):
+                if n * (din + dout) > NNZ_CAP or rng.random() < 0.55:
+                    continue
+                for perm in (False, True):
+                    seed = int(rng.integers(1 << 30))
+                    add("sbm_n%d_c%d_i%g_o%g_%s" % (n, size, din, dout, "p" if perm else "s"),
+                        lambda n=n, size=size, din=din, dout=dout, perm=perm, seed=seed:
+                        synth.sbm(n, n // size, din, dout, seed=seed, permute=perm))
+    # meshes
+    for nx, ny in ((128, 128), (256, 256), (512, 512), (1024, 1024), (2048, 1024), (2048, 2048), (4096, 1024), (8192, 256),
+                   (100, 100), (300, 700), (1000, 500), (3000, 1000), (64, 4096), (1536, 1536)):
+        add("stencil_%dx%d" % (nx, ny), lambda nx=nx, ny=ny: synth.stencil2d(nx, ny))
+    for nx, ny, drop in ((512, 512, 0.3), (1024, 1024, 0.25), (2048, 1024, 0.4), (1500, 1500, 0.1), (256, 256, 0.2),
+                         (2048, 2048, 0.3), (700, 900, 0.5), (400, 4000, 0.15)):
+        seed = int(rng.integers(1 << 30))
+        add("grid_%dx%d_h%.2f" % (nx, ny, drop), lambda nx=nx, ny=ny, drop=drop, seed=seed: grid_with_holes(nx, ny, drop, seed))
+    # banded random
+    for n in (15_000, 30_000, 150_000, 700_000, 2_000_000):
+        for k, w in ((2, 8), (6, 64), (16, 512), (30, 4096), (4, 20000), (10, 100)):
+            if n * k * 2 > NNZ_CAP or rng.random() < 0.2:
+                continue
+            seed = int(rng.integers(1 << 30))
+            add("band_n%d_k%d_w%d" % (n, k, w), lambda n=n, k=k, w=w, seed=seed: banded(n, k, w, seed))
+    return items
+
+
+# ------------------------------------------------------------------------------------------------------------
+# sweep (GPU)
+# ------------------------------------------------------------------------------------------------------------
+def sweep_main(args):
+    import pandas as pd
+    import torch
+
+    from . import sweep as sw
+    from . import synth
+    from .graph_input import graph_input
+
+    assert torch.cuda.is_available(), "the sweep needs the GPU"
+    items = corpus()
+    part, nparts = (int(x) for x in args.part.split("/"))
+    items = [it for i, it in enumerate(items) if i % nparts == part]
+    if args.limit:
+        items = items[: args.limit]
+    os.makedirs(args.out, exist_ok=True)
+    tag = "" if nparts == 1 else "_part%d" % part
+    info_rows, names = [], []
+    tp = {d: [] for d in DIMS}
+    t_start = time.time()
+    for idx, (name, build) in enumerate(items):
+        t0 = time.time()
+        r, c, n = build()
+        rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+        g = graph_input(name, "")
+        g.verbose = False
+        g.load_from_csr(rowPtr, colIdx, val)
+        ops = sw.operators_of(g)
+        nnz = g.mtx_edges
+        rows = (n + 1) // 2 * 2
+        # every representation must give the same product before it is timed
+        X = torch.randn(rows, 32, device="cuda")
+        if rows != n:
+            X[n:] = 0
+        ref = ops[0]._spmm(X)[:n]
+        scale = ref.abs().max().item() + 1e-6
+        for op in ops[1:]:
+            err = (op._spmm(X)[:n] - ref).abs().max().item()
+            assert err <= 1e-4 * scale, (name, err, scale)
+        del X, ref
+        for d in DIMS:
+            ms, gf = sw.sweep_dim(ops, d, nnz, n, warmup=args.warmup, iters=args.iters)
+            tp[d].append(gf)
+        info_rows.append([name] + g._feature_values())
+        names.append(name)
+        del ops, g
+        torch.cuda.empty_cache()
+        print("[%d/%d] %-34s n=%-8d nnz=%-9d %.1fs (total %.0fs)" % (idx + 1, len(items), name, n, nnz, time.time() - t0,
+                                                                   time.time() - t_start), flush=True)
+        # keep what is done on disk: a run that is cut short still leaves usable csv files
+        info = pd.DataFrame(info_rows, columns=["mtx_name"] + FEATURES)
+        info.to_csv(os.path.join(args.out, "mtx_info%s.csv" % tag), index=False)
+        if (idx + 1) % 10 == 0 or idx + 1 == len(items):
+            for d in DIMS:
+                pd.DataFrame(np.array(tp[d]), columns=sw.column_names(d)).to_csv(
+                    os.path.join(args.out, "dim%d%s.csv" % (d, tag)), index=False)
+
+
+# ------------------------------------------------------------------------------------------------------------
+# fit (CPU)
+# ------------------------------------------------------------------------------------------------------------
+def load_training_data(data_dir):
+    import glob
+
+    import pandas as pd
+
+    info_files = sorted(glob.glob(os.path.join(data_dir, "mtx_info*.csv")))
+    assert info_files, "no mtx_info*.csv under " + data_dir
+    infos, tps = [], {d: [] for d in DIMS}
+    for f in info_files:
+        tag = os.path.basename(f)[len("mtx_info"):-len(".csv")]
+        info = pd.read_csv(f)
+        per_dim = {d: pd.read_csv(os.path.join(data_dir, "dim%d%s.csv" % (d, tag))) for d in DIMS}
+        rows = min([len(info)] + [len(v) for v in per_dim.values()])
+        infos.append(info.iloc[:rows])
+        for d in DIMS:
+            tps[d].append(per_dim[d].iloc[:rows])
+    info = pd.concat(infos, ignore_index=True)
+    return info, {d: pd.concat(tps[d], ignore_index=True) for d in DIMS}
+
+
+def fit_main(args):
+    import pandas as pd
+    from sklearn.ensemble import RandomForestClassifier
+    from sklearn.model_selection import train_test_split
+
+    info, tps = load_training_data(args.data)
+    X = info[FEATURES].to_numpy(dtype=np.float64)
+    os.makedirs(args.out, exist_ok=True)
+    report = {"matrices": int(len(info)), "per_dim": {}}
+    idx = np.arange(len(info))
+    tr, te = train_test_split(idx, test_size=0.2, random_state=17)
+    for d in DIMS:
+        TP = tps[d].to_numpy(dtype=np.float64)
+        y = TP.argmax(axis=1)  # class code = column index (PCSR.py:815-818)
+        # label csv in the reference's schema
+        lab = pd.concat([info, pd.DataFrame({"OP_SpMM": y})], axis=1)
+        lab.to_csv(os.path.join(args.data, "dim%d_OP_SpMM.csv" % d), index=False)
+        best = None
+        for n_est in (30, 50, 80):
+            clf = RandomForestClassifier(n_estimators=n_est, n_jobs=-1, random_state=17)
+            clf.fit(X[tr], y[tr])
+            pick = clf.predict(X[te])
+            norm = TP[te, pick] / TP[te].max(axis=1)  # normalised performance of the pick
+            score = (float(np.mean(norm >= 1 / 1.10)), float(norm.mean()))
+            if best is None or score > best[0]:
+                best = (score, n_est, clf, pick, norm)
+        (within10, mean_norm), n_est, clf, pick, norm = best
+        report["per_dim"][d] = {
+            "n_estimators": n_est, "classes": int(TP.shape[1]), "test_matrices": int(len(te)),
+            "test_accuracy": float(np.mean(pick == y[te])), "mean_normalised_performance": mean_norm,
+            "share_within_10pct_of_best": within10, "worst_normalised_performance": float(norm.min()),
+        }
+        # the shipped model is refitted on every matrix
+        final = RandomForestClassifier(n_estimators=n_est, n_jobs=-1, random_state=17).fit(X, y)
+        final.n_jobs = 1
+        with open(os.path.join(args.out, "rnd_tree_%d.pkl" % d), "wb") as f:
+            pickle.dump(final, f)
+        print("dim %3d: %2d classes  n_estimators %d  test acc %.3f  mean norm perf %.4f  within 10%%: %.3f  worst %.3f" % (
+            d, TP.shape[1], n_est, report["per_dim"][d]["test_accuracy"], mean_norm, within10, norm.min()), flush=True)
+    allw = [v["share_within_10pct_of_best"] for v in report["per_dim"].values()]
+    report["share_within_10pct_mean"] = float(np.mean(allw))
+    report["share_within_10pct_min"] = float(np.min(allw))
+    with open(os.path.join(args.out, "decider_report.json"), "w") as f:
+        json.dump(report, f, indent=1)
+    print("matrices %d; within 10%% of best: mean %.3f, min over widths %.3f" % (len(info), np.mean(allw), np.min(allw)))
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    sub = ap.add_subparsers(dest="cmd", required=True)
+    s = sub.add_parser("sweep")
+    s.add_argument("--out", default="gpurun_out/decider")
+    s.add_argument("--part", default="0/1", help="i/n: every n-th matrix starting at i")
+    s.add_argument("--limit", type=int, default=0)
+    s.add_argument("--warmup", type=int, default=2)
+    s.add_argument("--iters", type=int, default=6)
+    f = sub.add_parser("fit")
+    here = os.path.dirname(os.path.abspath(__file__))
+    f.add_argument("--data", default=os.path.join(here, "models", "train_data"))
+    f.add_argument("--out", default=os.path.join(here, "models"))
+    ls = sub.add_parser("list")
+    args = ap.parse_args(argv)
+    if args.cmd == "sweep":
+        sweep_main(args)
+    elif args.cmd == "fit":
+        fit_main(args)
+    else:
+        for name, _ in corpus():
+            print(name)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,297 @@
+"""CPU-side tests of the product: the C ABI library loads and exports every declared symbol, the host-side index
+construction (row split, 2x1 BCSR) is bit-exact against the oracle / SciPy, the format builder reproduces the
+reference's statistics and normalisation, the CF search space and the decider decoding match the reference's
+integer functions, and the extension modules export the reference's binding names."""
+import ctypes
+import math
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import ROOT, pubmed_pattern, random_csr
+
+
+def test_c_abi_exports_every_declared_symbol():
+    from paramspmm_ae_amd import _capi
+
+    header = open(os.path.join(ROOT, "include", "paramsp.h")).read()
+    declared = set(re.findall(r"\b(psp_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 18
+    for name in declared:
+        assert hasattr(_capi.lib, name), name
+    assert _capi.lib.psp_version() >= 100
+    # every entry point the python binding types is declared in the header
+    assert set(_capi.SIGNATURES) <= declared
+
+
+def test_spmm_plan_mapping():
+    from paramspmm_ae_amd import _capi
+    from oracle.oracle import CF_TABLE
+
+    for N, cfs in CF_TABLE.items():
+        for cf in cfs:
+            for bw in (4, 8):
+                p = _capi.spmm_plan(N, cf, bw)
+                assert p["vec"] == 4 and p["waves_per_block"] == bw
+                tile = p["lanes_per_row"] * p["coarsen"] * p["vec"]
+                assert tile * p["col_tiles"] >= N > tile * (p["col_tiles"] - 1)
+                assert tile <= 32 * cf or p["col_tiles"] == 1  # a lane group never owns more than 32*CF columns
+                assert p["rows_per_wave"] * p["lanes_per_row"] == 64
+                assert 1 <= p["unroll"] <= p["lanes_per_row"]
+    assert _capi.spmm_plan(50, 1, 4)["vec"] == 2 and _capi.spmm_plan(51, 1, 4)["vec"] == 1
+    for bad in ((16, 0, 4), (16, 9, 4), (16, 1, 6), (0, 1, 4)):
+        with pytest.raises(_capi.ParamSpError):
+            _capi.spmm_plan(*bad)
+
+
+@pytest.mark.parametrize("g", [1, 7, 32, 96])
+def test_split_host_functions_match_oracle(oracle, g):
+    import paramspmm_ae_amd  # noqa: F401
+    import ParamSpMM
+    import ParamSpCONV
+
+    rowPtr, _, _ = random_csr(100_000, 9, 3, empty_frac=0.2, hub=(11, 5000))
+    want_rps, want_tr = oracle.split_csr(rowPtr, g)
+    rp_t = torch.from_numpy(rowPtr)
+    for mod in (ParamSpMM, ParamSpCONV):
+        rps, tr = mod.split_csr(rp_t, g)
+        assert rps.dtype == torch.int32 and tr.dtype == torch.int32
+        assert np.array_equal(rps.numpy(), want_rps) and np.array_equal(tr.numpy(), want_tr)
+        k = np.diff(rowPtr)
+        off = torch.from_numpy(np.concatenate([[0], np.cumsum(-(-k // g))]).astype(np.int32))
+        rps2, tr2 = mod.split_csr_par(rp_t, off, g)  # 100k rows: the threaded path
+        assert np.array_equal(rps2.numpy(), want_rps) and np.array_equal(tr2.numpy(), want_tr)
+
+
+def test_split_host_errors():
+    import paramspmm_ae_amd  # noqa: F401
+    import ParamSpMM
+
+    rp = torch.tensor([0, 3, 5], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="granularity"):
+        ParamSpMM.split_csr(rp, 0)
+    with pytest.raises(RuntimeError, match="int32"):
+        ParamSpMM.split_csr(rp.long(), 4)
+    with pytest.raises(RuntimeError, match="prefix sum"):
+        ParamSpMM.split_csr_par(rp, torch.tensor([0, 1, 5], dtype=torch.int32), 4)
+    rps, tr = ParamSpMM.split_csr(torch.zeros(4, dtype=torch.int32), 32)
+    assert rps.tolist() == [0] and tr.numel() == 0
+
+
+@pytest.mark.parametrize("n", [1, 2, 9, 1000, 4001])
+def test_bcsr_host_builder_matches_oracle_and_scipy(oracle, n):
+    import scipy.sparse as sp
+    from paramspmm_ae_amd.graph_input import build_bcsr
+
+    rowPtr, colIdx, val = random_csr(n, min(7, n), n, empty_frac=0.2)
+    rpb, cib, vb = build_bcsr(rowPtr, colIdx, val)
+    o = oracle.bcsr_build(rowPtr, colIdx, val, ncols=n + (n & 1))
+    assert np.array_equal(rpb, o[0]) and np.array_equal(cib, o[1]) and np.array_equal(vb, o[2])
+    m = n + (n & 1)
+    indptr = np.concatenate([rowPtr, [rowPtr[-1]] * (m - n)])
+    b = sp.csr_matrix((val, colIdx, indptr), shape=(m, m)).tobsr(blocksize=(2, 1))
+    assert np.array_equal(rpb, b.indptr) and np.array_equal(cib, b.indices)
+    assert np.array_equal(vb, b.data.reshape(-1, 2))
+
+
+def test_bcsr_rejects_bad_columns():
+    from paramspmm_ae_amd import _capi
+
+    rp = np.array([0, 1], np.int32)
+    ci = np.array([5], np.int32)
+    assert _capi.lib.psp_bcsr_count(_capi.ptr(rp), _capi.ptr(ci), 1, 2) == -1
+    assert b"out of range" in _capi.lib.psp_last_error()
+
+
+@pytest.mark.parametrize("which", ["orig", "rabbit"])
+def test_format_builder_on_pubmed(oracle, which, tmp_path):
+    """load() from a MatrixMarket file of the reference's pubmed pattern: counts, statistics, normalisation."""
+    import scipy.io
+    from paramspmm_ae_amd.graph_input import graph_input
+
+    m = pubmed_pattern(which)
+    import scipy.sparse as sp
+
+    scipy.io.mmwrite(str(tmp_path / "pm.mtx"), sp.tril(m).tocoo(), symmetry="symmetric")
+    g = graph_input("pm", str(tmp_path) + os.sep)
+    g.verbose = False
+    g.load(load_from_mtx=True)
+    assert (g.mtx_nodes, g.mtx_edges) == (19717, 88651)
+    assert g.csr_data.split_granularity == 32 and g.bcsr_data.split_granularity == 32
+    assert g.csr_data.target_row.numel() == 20005
+    assert g.bcsr_data.colIdx.numel() == (88469 if which == "orig" else 81018)
+    assert g.bcsr_data.target_row.numel() == (10293 if which == "orig" else 10240)
+    assert int(g.csr_data.max_row_nnz) == 171 and int(g.csr_data.real_nrow) == 19717
+    assert g.bcsr_data.val.shape[1] == 2 and g.bcsr_data.num_nodes == 9859
+    # statistics against the numpy restatement of graph_input.py:48-129
+    st = oracle.format_stats(m.indptr, m.indices, m.nnz)
+    info = g.get_info()
+    assert info.shape == (1, 15)
+    np.testing.assert_allclose(
+        info[0, :13],
+        [19717, 88651, 88651 / 19717**2, 171, 19717, 1.0, st["avg_degree"], st["COV"], st["real_avg_degree"],
+         st["real_COV"], st["max_bw"], st["avg_bw"], st["split_ratio"]], rtol=1e-6)
+    assert abs(info[0, 14] - (0.501 if which == "orig" else 0.547)) < 1e-3
+    assert np.array_equal(g.csr_data.rowPtr_split.numpy(), oracle.split_csr(m.indptr, 32)[0])
+    # normalised load: D^-1/2 (A+I) D^-1/2 in float64, rounded once to fp32
+    g2 = graph_input("pm", str(tmp_path) + os.sep)
+    g2.verbose = False
+    g2.load(load_from_mtx=True, is_normalize=True)
+    coo = m.tocoo()
+    rp, ci, v = oracle.normalize_adj_closed_form(coo.row, coo.col, 19717)
+    assert g2.mtx_edges == 108365
+    assert np.array_equal(g2.csr_data.rowPtr.numpy(), rp) and np.array_equal(g2.csr_data.colIdx.numpy(), ci)
+    assert np.array_equal(g2.csr_data.val.numpy(), v)
+    # GIN: off-diagonal 1, diagonal 1.5
+    g3 = graph_input("pm", str(tmp_path) + os.sep)
+    g3.verbose = False
+    g3.load(load_from_mtx=True, GIN_epsilon=0.5)
+    rows = np.repeat(np.arange(19717), np.diff(g3.csr_data.rowPtr.numpy()))
+    d = rows == g3.csr_data.colIdx.numpy()
+    vv = g3.csr_data.val.numpy()
+    assert np.all(vv[d] == 1.5) and np.all(vv[~d] == 1.0) and g3.mtx_edges == 108365
+
+
+def test_format_builder_from_arrays_and_synthetic_closed_form(oracle):
+    from paramspmm_ae_amd import synth
+    from paramspmm_ae_amd.graph_input import graph_input
+
+    r, c, n = synth.chung_lu(5001, 20000, seed=3, max_degree=300)
+    rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+    rp2, ci2, v2 = oracle.normalize_adj_closed_form(np.concatenate([r, c]), np.concatenate([c, r]), n)
+    assert np.array_equal(rowPtr, rp2) and np.array_equal(colIdx, ci2) and np.array_equal(val, v2)
+    g = graph_input("cl", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val, manual_granularity=8)
+    assert g.csr_data.split_granularity == 8 and g.bcsr_data.num_nodes == 2501
+    st = oracle.format_stats(rowPtr, colIdx, colIdx.size, manual_granularity=8)
+    assert abs(float(g.csr_data.split_ratio) - st["split_ratio"]) < 1e-6
+    assert g.csr_data.target_row.numel() == int(st["row_split_nnz"].sum())
+    stb = oracle.format_stats(g.bcsr_data.rowPtr.numpy(), None, float(g.bcsr_data.colIdx.numel()), csr_flag=False,
+                              manual_granularity=8)
+    assert abs(float(g.bcsr_data.split_ratio) - stb["split_ratio"]) < 1e-6
+    g.load_from_csr(rowPtr, colIdx, val, is_avg_granularity=True)
+    assert g.csr_data.split_granularity == int(colIdx.size / n)
+    if not torch.cuda.is_available():
+        with pytest.raises(RuntimeError, match="no GPU"):
+            g.load_from_csr(rowPtr, colIdx, val, if_mask=True)
+
+
+def test_cf_search_space_and_decoding_match_reference_integers(oracle):
+    from oracle.oracle import CF_TABLE
+    from paramspmm_ae_amd.PCSR import dynamic_CF_prompter, gap_calculator
+    from paramspmm_ae_amd.decider import SpMMDecider, model_dim_for
+    from paramspmm_ae_amd import sweep
+
+    for dim in range(1, 300):
+        assert dynamic_CF_prompter(dim) == oracle.dynamic_CF_prompter(dim)
+        for cf in range(1, 9):
+            assert gap_calculator(dim, cf) == oracle.gap_calculator(dim, cf)
+        assert model_dim_for(dim) == oracle.model_dim(dim)
+    for dim, cfs in CF_TABLE.items():
+        assert dynamic_CF_prompter(dim) == cfs
+    d = SpMMDecider("unused/")
+    for dim, cfs in CF_TABLE.items():
+        names = sweep.column_names(dim)
+        assert len(names) == 8 * len(cfs)
+        for code in range(8 * len(cfs)):
+            got = d.decode_tree(code, dim)
+            assert got == oracle.decode_tree(code, dim) == sweep.decode_column(dim, code)
+            rep = ["vec1", "vec1_split", "vec2", "vec2_split"][code % 4]
+            assert names[code] == "%s_TP_%d%d" % (rep, got[2], got[3])
+    assert [model_dim_for(x) for x in (16, 24, 32, 40, 48, 100, 128, 250)] == [16, 16, 32, 48, 48, 112, 128, 240]
+
+
+def test_decider_round_trip_with_a_forest_trained_in_test(tmp_path):
+    import pickle
+    from sklearn.ensemble import RandomForestClassifier
+    from paramspmm_ae_amd.decider import SpMMDecider
+
+    rng = np.random.default_rng(0)
+    X = np.repeat(rng.random((60, 1)), 15, axis=1)  # every feature carries the same signal
+    y = (X[:, 0] > 0.5).astype(int) * 5 + 1  # classes 1 and 6 of the 16 codes of width 64
+    clf = RandomForestClassifier(n_estimators=10, random_state=0).fit(X, y)
+    with open(tmp_path / "rnd_tree_64.pkl", "wb") as f:
+        pickle.dump(clf, f)
+
+    class G:
+        def __init__(self, v):
+            self.v = v
+
+        def get_info(self):
+            return self.v.reshape(1, -1)
+
+    d = SpMMDecider(str(tmp_path) + os.sep)
+    with pytest.raises(ValueError, match="pickle file not found"):
+        d.gen_model_dict([64, 40])  # 40 is served by the forest of 48, which is missing
+    import shutil
+
+    shutil.copy(tmp_path / "rnd_tree_64.pkl", tmp_path / "rnd_tree_48.pkl")
+    d.gen_model_dict([64, 40, 48])  # 40 and 48 share the forest of 48
+    assert d.model_dict[40] is d.model_dict[48]
+    lo, hi = np.full(15, 0.1), np.full(15, 0.9)
+    assert d.config_PCSR(G(lo), 64) == d.decode_tree(1, 64) == (1, 1, 1, 4)
+    assert d.config_PCSR(G(hi), 64) == d.decode_tree(6, 64) == (0, 2, 2, 4)
+    with pytest.raises(ValueError, match="not found in model_dict"):
+        d.config_PCSR(G(lo), 128)
+
+
+def test_extension_modules_export_the_reference_binding_names():
+    import paramspmm_ae_amd  # noqa: F401
+    import ParamSpMM
+    import ParamSDDMM
+    import ParamSpCONV
+
+    spmm = ["split_csr", "split_csr_par", "csr_spmm", "csr_split_spmm", "bcsr_spmm", "bcsr_split_spmm", "vec_spmm",
+            "vec_split_spmm", "csr_spmm_profile", "csr_split_spmm_profile", "bcsr_spmm_profile",
+            "bcsr_split_spmm_profile", "vec_spmm_profile", "vec_split_spmm_profile", "cusparse_compute",
+            "cusparse_profile", "cusparse_compute_csr_alg2", "cusparse_profile_csr_alg2", "cusparse_compute_coo_alg4",
+            "cusparse_profile_coo_alg4", "cusparse_compute_csc", "cusparse_profile_csc", "gespmm_compute", "gespmm_profile"]
+    sddmm = ["csr_sddmm", "csr_split_sddmm", "bcsr_sddmm", "bcsr_split_sddmm", "vec_sddmm", "vec_split_sddmm",
+             "csr_sddmm_profile", "csr_split_sddmm_profile", "bcsr_sddmm_profile", "bcsr_split_sddmm_profile",
+             "vec_sddmm_profile", "vec_split_sddmm_profile", "cusparse_sddmm_compute", "cusparse_sddmm_profile", "genmask"]
+    conv = ["split_csr", "split_csr_par"] + [f + s for f in ("csr_spmm", "csr_split_spmm", "bcsr_spmm", "bcsr_split_spmm")
+                                             for s in ("_forward", "_backward")]
+    for mod, names in ((ParamSpMM, spmm), (ParamSDDMM, sddmm), (ParamSpCONV, conv)):
+        for n in names:
+            assert callable(getattr(mod, n)), (mod.__name__, n)
+    # device entry points refuse CPU tensors instead of falling back
+    x = torch.zeros(4, 16)
+    rp = torch.zeros(5, dtype=torch.int32)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        ParamSpMM.csr_spmm(x, rp, rp[:0], x[:0, 0], 1, 4)
+    with pytest.raises(RuntimeError, match="CUDA tensor"):
+        ParamSDDMM.csr_sddmm(x, x, rp, rp[:0], x[:0, 0], 1, 4)
+
+
+@pytest.mark.skipif(not os.path.isdir("/root/reference"), reason="the reference is only mounted in the build container")
+def test_reference_python_only_uses_exported_names():
+    """Parses the reference's .py files as text (no import, no execution) and checks that every attribute they
+    access on the three extension modules exists in this build."""
+    import ast
+
+    import paramspmm_ae_amd  # noqa: F401
+    import ParamSpMM
+    import ParamSDDMM
+    import ParamSpCONV
+
+    alias = {"SpMM": ParamSpMM, "SDDMM": ParamSDDMM, "SpCONV": ParamSpCONV,
+             "ParamSpMM": ParamSpMM, "ParamSDDMM": ParamSDDMM, "ParamSpCONV": ParamSpCONV}
+    used = set()
+    for fn in ("PCSR.py", "graph_input.py", "gnn_conv.py", "SDDMM.py", "decider.py", "GNN.py"):
+        tree = ast.parse(open(os.path.join("/root/reference", fn)).read())
+        imported = {}
+        for node in ast.walk(tree):
+            if isinstance(node, ast.Import):
+                for a in node.names:
+                    if a.name in ("ParamSpMM", "ParamSDDMM", "ParamSpCONV"):
+                        imported[a.asname or a.name] = alias[a.name]
+        for node in ast.walk(tree):
+            if isinstance(node, ast.Attribute) and isinstance(node.value, ast.Name) and node.value.id in imported:
+                used.add((imported[node.value.id], node.attr))
+    assert len(used) > 30
+    for mod, attr in used:
+        assert hasattr(mod, attr), (mod.__name__, attr)
