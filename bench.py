@@ -43,6 +43,101 @@ def algorithmic_bytes(fmt, F, n_x_rows, N):
     return b + 4 * n_x_rows * N + 4 * 2 * Mb * N
 
 
+def measured_traffic(graph, rows_of):
+    """HBM bytes per launch of the dominant kernel, from the committed rocprofv3 counter summary
+    (profiles/psp_spmm_kernel_<graph>_pmc.md: FETCH_SIZE x2 + WRITE_SIZE, both in KiB, per width).  None when the
+    summary has no line for one of the widths / configurations that ran."""
+    path = os.path.join(ROOT, "profiles", "psp_spmm_kernel_%s_pmc.md" % graph)
+    if not os.path.exists(path):
+        return None
+    table = {}
+    for line in open(path):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 7 and cells[0].isdigit():
+            # | dim | format | CF | blkWarpNum | FETCH_SIZE KiB | WRITE_SIZE KiB | HBM bytes |
+            table[(int(cells[0]), cells[1], int(cells[2]), int(cells[3]))] = int(cells[6])
+    total = 0
+    for r in rows_of:
+        key = (r["dim"], r["format"], r["CF"], r["blkWarpNum"])
+        if key not in table:
+            return None
+        total += table[key]
+    return int(total / len(rows_of))
+
+
+def bench_agnn(args):
+    """Attention layers on the R-MAT pattern (BASELINE.json configs[3]): per layer e = A_e * <X_i, Y_j> on the
+    stored entries (SDDMM, K = 32 and 64, rows L2-normalised), softmax over each row's entries, then SpMM with
+    H [n, 32].  Five layers per step.  The reference's AGNN has neither the A_e factor nor the softmax; they are
+    the additions `csr_sddmm_scaled` and `segment_softmax` of this build."""
+    import torch
+
+    import paramspmm_ae_amd  # noqa: F401
+    import ParamSDDMM
+    import ParamSpMM
+    from paramspmm_ae_amd import synth
+
+    graph = "C2" if args.graph == "C2" else args.graph
+    rowPtr, colIdx, val, n = synth.config_graph(graph)
+    nnz = colIdx.size
+    rp, ci, v = (torch.from_numpy(a).cuda() for a in (rowPtr, colIdx, val))
+    gen = torch.Generator(device="cuda").manual_seed(7)
+    out = {"metric": "AGNN attention layer stack: SDDMM + row softmax + SpMM(N=32), 5 layers", "unit": "ms per 5 layers",
+           "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": False, "scaling": "weak",
+           "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+           "config": {"workload": "%s pattern, K in (32, 64), H [n, 32]" % graph, "nodes": n, "nnz": nnz}, "per_K": []}
+    H = torch.randn(n, 32, device="cuda", generator=gen)
+    for K in (32, 64):
+        X = torch.nn.functional.normalize(torch.randn(n, K, device="cuda", generator=gen), dim=1).contiguous()
+        Y = torch.nn.functional.normalize(torch.randn(n, K, device="cuda", generator=gen), dim=1).contiguous()
+
+        def layers():
+            h = H
+            for _ in range(5):
+                e = ParamSDDMM.csr_sddmm_scaled(X, Y, rp, ci, v, 8)
+                a = ParamSDDMM.segment_softmax(rp, e)
+                h = ParamSpMM.csr_spmm(h, rp, ci, a, 1, 8)
+            return h
+
+        for _ in range(args.warmup):
+            layers()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            layers()
+        torch.cuda.synchronize()
+        ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        flops = 5 * (2.0 * nnz * K + 2.0 * nnz * 32)
+        # algorithmic bytes per layer: SDDMM 4(M+1)+4nnz+4nnz(A_e)+8nK+4nnz ; softmax 4(M+1)+8nnz ; SpMM 4(M+1)+8nnz+8n*32
+        b = 5 * ((4 * (n + 1) + 12 * nnz + 8 * n * K) + (4 * (n + 1) + 8 * nnz) + (4 * (n + 1) + 8 * nnz + 8 * n * 32))
+        out["per_K"].append({"K": K, "ms": round(ms, 4), "gflops": round(flops / ms / 1e6, 1),
+                             "alg_GBps": round(b / ms / 1e6, 1), "frac_hbm": round(b / ms / 1e6 / HBM_PEAK_GBS, 4)})
+    out["value"] = out["per_K"][-1]["ms"]
+    out["ms_per_step"] = out["value"]
+    print(json.dumps(out))
+
+
+def bench_gcn(args):
+    """GCN and GIN training epochs (BASELINE.json configs[4]): 5 layers, hidden 16 / 32 / 128, 16 classes, random
+    features and weights, forward + backward + Adam, on the 1M-node stochastic block model in community order
+    (C5) and randomly permuted (C5p).  --steps is the number of timed epochs (the reference times 200)."""
+    from paramspmm_ae_amd import GNN
+
+    out = {"metric": "GCN / GIN epoch ms (5 layers, fwd+bwd+Adam), SBM 1M nodes", "unit": "ms per epoch", "n_gpus": 1,
+           "steps": args.steps, "warmup": 1, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+           "dtype": "f32", "data": "synthetic", "config": {"workload": "C5 / C5p, hidden 16 32 128, 16 classes"}, "epochs": []}
+    graphs = [args.graph] if args.graph in ("C5", "C5p", "C1") else ["C5", "C5p"]
+    for g in graphs:
+        for net in ("GCN", "GIN"):
+            res = GNN.main(["--net", net, "--synthetic", g, "--hidden_list", "16", "32", "128", "--num_classes", "16",
+                            "--num_features", "32", "--num_epoches", str(args.steps)])
+            for (name, hidden), ms in res.items():
+                out["epochs"].append({"graph": name, "net": net, "hidden": hidden, "ms_per_epoch": round(ms, 3)})
+    out["value"] = out["epochs"][0]["ms_per_epoch"]
+    out["ms_per_step"] = out["value"]
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -50,9 +145,16 @@ def main():
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--graph", default="C2", help="C1, C2, C3, C3s, C5, C5p (synth.config_graph)")
     ap.add_argument("--dims", default=",".join(str(d) for d in range(16, 257, 16)))
-    ap.add_argument("--pick", choices=["sweep", "decider", "csr"], default="sweep")
+    ap.add_argument("--pick", default="auto",
+                    help="auto (decider if its forests are built, else sweep) | sweep | decider | "
+                         "fixed:<csr|csr_split|bcsr|bcsr_split>:<CF>:<blkWarpNum>")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run one plain device copy of X (known size) so a counter run can be calibrated")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--dump", default=None, help="write the full sweep table (every column, every width) as JSON")
+    ap.add_argument("--workload", choices=["spmm", "agnn", "gcn"], default="spmm",
+                    help="spmm: the headline width sweep; agnn: SDDMM -> row softmax -> SpMM attention layers; "
+                         "gcn: GCN / GIN training epochs on the SBM graph")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (no multi-GPU path exists)" % args.gpus,
@@ -64,6 +166,10 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(1)
+    if args.workload == "agnn":
+        return bench_agnn(args)
+    if args.workload == "gcn":
+        return bench_gcn(args)
     from paramspmm_ae_amd import _capi, synth, sweep
     from paramspmm_ae_amd.graph_input import graph_input
 
@@ -92,21 +198,31 @@ def main():
     chosen = {}
     table = {}
     decider = None
-    if args.pick == "decider":
+    pick = args.pick
+    if pick == "auto":
+        from paramspmm_ae_amd.decider import DEFAULT_PICKLE_PATH
+
+        have = all(os.path.exists(os.path.join(DEFAULT_PICKLE_PATH, "rnd_tree_%d.pkl" % d)) for d in range(16, 257, 16))
+        pick = "decider" if have else "sweep"
+    if pick == "decider":
         from paramspmm_ae_amd.decider import SpMMDecider
 
         decider = SpMMDecider()
         decider.gen_model_dict(dims)
+    fixed = None
+    if pick.startswith("fixed:"):
+        _, f_fmt, f_cf, f_bw = pick.split(":")
+        fixed = (int("split" in f_fmt), 2 if f_fmt.startswith("bcsr") else 1, int(f_cf), int(f_bw))
     for d in dims:
-        if args.pick == "sweep" or args.dump:
+        if pick == "sweep" or args.dump:
             ms, gf = sweep.sweep_dim(ops, d, nnz, n, warmup=2, iters=5, X=Xs[d])
             table[d] = {"columns": sweep.column_names(d), "ms": ms.tolist()}
-        if args.pick == "sweep":
+        if pick == "sweep":
             chosen[d] = sweep.decode_column(d, int(np.argmin(ms)))
-        elif args.pick == "decider":
+        elif pick == "decider":
             chosen[d] = tuple(int(v) for v in decider.config_PCSR(graph, d))
         else:
-            chosen[d] = (0, 1, 1, 4)
+            chosen[d] = fixed
     if args.dump:
         with open(args.dump, "w") as f:
             json.dump({"graph": args.graph, "n": n, "nnz": nnz, "formats": F, "table": table}, f)
@@ -143,6 +259,10 @@ def main():
             if rc != 0:
                 _capi.check(rc)
 
+    if args.calibrate_copy:
+        d0 = dims[-1]
+        Ys[d0].copy_(Xs[d0])  # moves 2 * rows * d0 * 4 bytes
+        print("calibration copy: %d bytes read, %d bytes written" % (rows * d0 * 4, rows * d0 * 4), file=sys.stderr)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -166,11 +286,25 @@ def main():
         per_dim.append({"dim": d, "format": fmt, "CF": cf, "blkWarpNum": bw, "ms": round(ms, 5),
                         "gflops": round(2.0 * nnz * d / (ms * 1e-3) / 1e9, 1), "alg_bytes": b_alg,
                         "alg_GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)})
-    dom = max(per_dim, key=lambda r: r["ms"])
-    roofline = {"bound": "hbm", "achieved": dom["alg_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(dom["alg_GBps"] / HBM_PEAK_GBS, 4), "traffic": None,
-                "kernel": "psp_spmm_kernel %s N=%d CF=%d bw=%d" % (dom["format"], dom["dim"], dom["CF"], dom["blkWarpNum"]),
-                "alg_bytes_per_launch": dom["alg_bytes"], "ms_per_launch": dom["ms"],
+    # The dominant kernel: widths that share (vectors per lane, vector width, unroll, format) run the same kernel
+    # symbol, which is what a rocprofv3 kernel trace averages over; take the symbol with the largest share of time.
+    by_symbol = {}
+    for r in per_dim:
+        plan = _capi.spmm_plan(r["dim"], r["CF"], r["blkWarpNum"])
+        sym = "psp_spmm_kernel<%d, %d, %d, %d, %s>" % (plan["coarsen"], plan["vec"], plan["unroll"],
+                                                       2 if r["format"].startswith("bcsr") else 1,
+                                                       "true" if "split" in r["format"] else "false")
+        r["kernel"] = sym
+        by_symbol.setdefault(sym, []).append(r)
+    sym, rows_of = max(by_symbol.items(), key=lambda kv: sum(r["ms"] for r in kv[1]))
+    sym_ms = sum(r["ms"] for r in rows_of)
+    sym_bytes = sum(r["alg_bytes"] for r in rows_of)
+    achieved = sym_bytes / (sym_ms * 1e-3) / 1e9
+    traffic = measured_traffic(args.graph, rows_of)
+    roofline = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
+                "kernel": sym, "widths": [r["dim"] for r in rows_of],
+                "alg_bytes_per_launch": int(sym_bytes / len(rows_of)), "ms_per_launch": round(sym_ms / len(rows_of), 5),
                 "mean_frac_over_widths": round(float(np.mean([r["frac_hbm"] for r in per_dim])), 4)}
 
     out = {
@@ -179,7 +313,7 @@ def main():
         "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: R-MAT 2^20 nodes SpMM width sweep" % args.graph if args.graph == "C2" else args.graph,
-                   "nodes": n, "nnz": nnz, "dims": dims, "pick": args.pick, "setup_s": round(setup_s, 1)},
+                   "nodes": n, "nnz": nnz, "dims": dims, "pick": pick, "setup_s": round(setup_s, 1)},
         "roofline": roofline,
         "sweep": per_dim,
     }

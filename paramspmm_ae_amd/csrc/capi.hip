@@ -103,6 +103,40 @@ int psp_zero_f32(float *p, size_t n, hipStream_t stream)
 }
 
 // ------------------------------------------------------------------------------------------------
+// selective clear for row-split SpMM: one lane per segment (plus one for the rows past the last segment)
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ void psp_clear_rows(float *Y, long long r0, long long r1, int N)
+{
+    for (long long i = r0 * N; i < r1 * N; i++) Y[i] = 0.0f;
+}
+
+__global__ void __launch_bounds__(256)
+psp_split_clear_kernel(const int *__restrict__ rowPtr_split, const int *__restrict__ target_row, float *__restrict__ Y,
+                       int nseg, int N, int nr, int rows_out, int logW)
+{
+    const int s = blockIdx.x * blockDim.x + threadIdx.x;
+    if (s > nseg) return;
+    if (s == nseg) {  // rows after the last targeted row
+        psp_clear_rows(Y, (long long)(target_row[nseg - 1] + 1) * nr, rows_out, N);
+        return;
+    }
+    const int t = target_row[s];
+    const int prev = s > 0 ? target_row[s - 1] : -1;
+    if (t > prev + 1) psp_clear_rows(Y, (long long)(prev + 1) * nr, (long long)t * nr, N);  // rows no segment targets
+    const bool boundary = s > 0 && (s & ((1 << logW) - 1)) == 0 && prev == t;              // row continues across two wavefronts
+    const bool empty = rowPtr_split[s] == rowPtr_split[s + 1];
+    if (boundary || empty) psp_clear_rows(Y, (long long)t * nr, (long long)(t + 1) * nr, N);
+}
+
+int psp_split_clear(const int *rowPtr_split, const int *target_row, float *Y, int nseg, int N, int nr, int rows_out,
+                    int logW, hipStream_t stream)
+{
+    hipLaunchKernelGGL(psp_split_clear_kernel, dim3(psp_ceil_div((long long)nseg + 1, 256)), dim3(256), 0, stream,
+                       rowPtr_split, target_row, Y, nseg, N, nr, rows_out, logW);
+    return psp_check_launch("split clear kernel");
+}
+
+// ------------------------------------------------------------------------------------------------
 // genmask (SDDMM/sddmm_kernel.cu:78-141): one lane per block-row walks its blocks in storage order
 // ------------------------------------------------------------------------------------------------
 __global__ void __launch_bounds__(256)

@@ -57,3 +57,9 @@ int psp_stripe_rows(void);
 
 // zero-fill used instead of hipMemsetAsync (callers may capture these launches in a HIP graph)
 int psp_zero_f32(float *p, size_t n, hipStream_t stream);
+
+// Row-split SpMM: clears exactly the rows of Y the SpMM kernel will not plainly store -- rows whose segments sit
+// in two wavefronts (each wavefront owns 2^logW consecutive segments), rows of empty segments, and rows no segment
+// targets.  nr = matrix rows per target row (2 for 2x1 blocks).
+int psp_split_clear(const int *rowPtr_split, const int *target_row, float *Y, int nseg, int N, int nr, int rows_out,
+                    int logW, hipStream_t stream);

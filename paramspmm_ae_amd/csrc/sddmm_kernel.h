@@ -2,8 +2,8 @@
 // entry p.  Semantics follow SDDMM/sddmm_kernel.cu:917-1287 (the stored values never scale the result; for
 // 2x1 blocks they only decide which of the two entries is computed).
 //
-// A sparse row is owned by L = 2^LOGL lanes; each lane keeps C vectors of V floats of the A row in
-// registers and loads the matching part of the B row, so a group reads L*V*4 contiguous bytes per load.
+// A lane group of L = 2^LOGL lanes works on one sparse row at a time; each lane keeps C vectors of V floats of
+// the A row in registers and loads the matching part of the B row, so a group reads L*V*4 contiguous bytes per load.
 // The per-lane partial dot products are summed across the group with DPP / ds_swizzle butterflies.  The L
 // results of one chunk of L non-zeros are parked one per lane and written with a single coalesced store
 // (the reference stores one float per warp per non-zero).
@@ -30,31 +30,62 @@ template <int LOGL> __device__ __forceinline__ float psp_group_sum(float v)
 }
 
 // val: bcsr -> [nblk,2] block values (gate); csr -> optional per-entry scale (may be null when !SCALE)
+//
+// The walk is the one of the SpMM kernel: a wavefront owns W = 2^logW consecutive segments, their stored entries
+// are divided evenly between the 64/L lane groups, and a group reloads its A row (prefetched one segment ahead)
+// whenever it crosses into another row.  Every stored entry is written exactly once, so `out` needs no clearing.
 template <int LOGL, int C, int V, int U, bool BCSR, bool SPLIT, bool SCALE>
 __global__ void __launch_bounds__(512)
 psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
                  const int *__restrict__ target_row, const float *__restrict__ A, const float *__restrict__ B,
-                 float *__restrict__ out, int nrows, int K, int tiles, int stripe)
+                 float *__restrict__ out, int nseg, int K, int logW, int tiles, int stripe)
 {
     typedef typename psp_vec<V>::type vec_t;
     constexpr int NR = BCSR ? 2 : 1;
     constexpr int L = 1 << LOGL;
+    constexpr int R = PSP_WAVE >> LOGL;
     static_assert(U <= L, "unroll must not exceed the group width");
+    __shared__ int2 s_seg[PSP_MAX_WAVES][PSP_WAVE];  // (end offset, A row) of the wavefront's filled segments
 
     const int tile = psp_xcd_tile(stripe);
     if (tile >= tiles) return;
 
+    const int W = 1 << logW;
     const int lane = threadIdx.x & (PSP_WAVE - 1);
     const int wave = threadIdx.x >> 6;
     const int sub = lane & (L - 1);
+    const int grp = lane >> LOGL;
     const int grp_base = lane - sub;
-    const int row = ((tile * (int)(blockDim.x >> 6) + wave) << (6 - LOGL)) + (lane >> LOGL);
+    const int s0 = (tile * (int)(blockDim.x >> 6) + wave) << logW;
+    if (s0 >= nseg) return;  // wave-uniform
+    const int nvalid = min(W, nseg - s0);
 
-    int lb = 0, hb = 0;
-    if (row < nrows) {
-        lb = rowPtr[row];
-        hb = rowPtr[row + 1];
+    const int P0 = rowPtr[s0];
+    const int P1 = rowPtr[s0 + nvalid];
+    {
+        const bool in = lane < nvalid;
+        const int e = in ? rowPtr[s0 + lane + 1] : P1;
+        const int e_up = __shfl_up(e, 1);  // cross-lane reads stay outside any lane-dependent branch
+        const int b_ = (lane == 0) ? P0 : e_up;
+        const bool filled = in && e != b_;
+        const unsigned long long fmask = __ballot(filled);
+        const int slot = __popcll(fmask & ((1ull << lane) - 1ull));
+        s_seg[wave][lane] = make_int2(P1, -1);
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        if (filled) s_seg[wave][slot] = make_int2(e, SPLIT ? target_row[s0 + lane] : s0 + lane);
     }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const int2 *w_seg = s_seg[wave];
+    if (P0 == P1) return;
+
+    const int q = (P1 - P0 + R - 1) >> (6 - LOGL);
+    int a0 = P0 + grp * q;
+    if (a0 > P1) a0 = P1;
+    const int b0 = min(P1, a0 + q);
+    if (a0 >= b0) return;  // the whole group leaves together; nothing below reads other groups' lanes
 
     int off[C];
     bool live[C];
@@ -65,10 +96,8 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
         off[i] = live[i] ? col : K - V;
     }
 
-    // the A row(s) of this group; dead tail vectors are zero so they add nothing to the dot product
-    float a[NR][C][V];
-    {
-        const int arow = (SPLIT && lb < hb) ? target_row[row] : row;
+    // A row(s) of a segment; dead tail vectors are zero so they add nothing to the dot product
+    auto load_a = [&](int key, float (&dst)[NR][C][V]) {
 #pragma unroll
         for (int r = 0; r < NR; r++)
 #pragma unroll
@@ -79,16 +108,28 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
 #pragma unroll
                     for (int e = 0; e < V; e++) t[e] = 0.0f;
                 }
-                if (lb < hb && live[i]) t = *(const vec_t *)(A + (size_t)(arow * NR + r) * (size_t)K + off[i]);
+                if (live[i]) t = *(const vec_t *)(A + (size_t)(key * NR + r) * (size_t)K + off[i]);
 #pragma unroll
-                for (int e = 0; e < V; e++) a[r][i][e] = psp_elem<V>(t, e);
+                for (int e = 0; e < V; e++) dst[r][i][e] = psp_elem<V>(t, e);
             }
+    };
+
+    int cur = 0;
+    for (int step = W >> 1; step >= 1; step >>= 1)
+        if (w_seg[cur + step - 1].x <= a0) cur += step;
+    int row_end = w_seg[cur].x;
+    int mykey = w_seg[cur].y;
+    float a[NR][C][V], a_nxt[NR][C][V];
+    load_a(mykey, a);
+    {
+        const int nk = cur + 1 < PSP_WAVE ? w_seg[cur + 1].y : -1;
+        load_a(nk >= 0 ? nk : mykey, a_nxt);
     }
 
-    for (int base = lb; base < hb; base += L) {
+    for (int base = a0; base < b0; base += L) {
         const int p = base + sub;
-        const bool ok = p < hb;
-        const int pp = ok ? p : hb - 1;
+        const bool ok = p < b0;
+        const int pp = ok ? p : b0 - 1;
         const int c_cur = colIdx[pp];
         float gate[NR];
         if constexpr (BCSR) {
@@ -102,30 +143,52 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
 #pragma unroll
         for (int r = 0; r < NR; r++) res[r] = 0.0f;
 
-        const int cnt = min(L, hb - base);
-        for (int k = 0; k < cnt; k += U) {
-            int ck[U];
+        const int cnt = min(L, b0 - base);
+        int k = 0;
+        while (k < cnt) {
+            // the current row's entries inside this chunk: positions [k, run_end)
+            const int run_end = min(cnt, row_end - base);
+            for (; k < run_end; k += U) {
+                int ck[U];
 #pragma unroll
-            for (int u = 0; u < U; u++) ck[u] = __builtin_amdgcn_ds_bpermute((grp_base + k + u) << 2, c_cur);
-            vec_t b[U][C];
+                for (int u = 0; u < U; u++) ck[u] = psp_bperm_i(grp_base + min(k + u, L - 1), c_cur);
+                vec_t bv[U][C];
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                const float *br = B + (size_t)ck[u] * (size_t)K;
+                for (int u = 0; u < U; u++) {
+                    const float *br = B + (size_t)ck[u] * (size_t)K;
 #pragma unroll
-                for (int i = 0; i < C; i++) b[u][i] = *(const vec_t *)(br + off[i]);
-            }
-#pragma unroll
-            for (int u = 0; u < U; u++)
-#pragma unroll
-                for (int r = 0; r < NR; r++) {
-                    float part = 0.0f;
-#pragma unroll
-                    for (int i = 0; i < C; i++)
-#pragma unroll
-                        for (int e = 0; e < V; e++) part = __builtin_fmaf(a[r][i][e], psp_elem<V>(b[u][i], e), part);
-                    part = psp_group_sum<LOGL>(part);
-                    if (sub == k + u) res[r] = part;
+                    for (int i = 0; i < C; i++) bv[u][i] = *(const vec_t *)(br + off[i]);
                 }
+#pragma unroll
+                for (int u = 0; u < U; u++)
+#pragma unroll
+                    for (int r = 0; r < NR; r++) {
+                        float part = 0.0f;
+#pragma unroll
+                        for (int i = 0; i < C; i++)
+#pragma unroll
+                            for (int e = 0; e < V; e++) part = __builtin_fmaf(a[r][i][e], psp_elem<V>(bv[u][i], e), part);
+                        part = psp_group_sum<LOGL>(part);
+                        // positions past run_end belong to the next row: their dot product with this A row is dropped
+                        if (sub == k + u && k + u < run_end) res[r] = part;
+                    }
+            }
+            k = run_end;
+            if (base + k == row_end && base + k < b0) {
+                const int2 nx = w_seg[++cur];
+                row_end = nx.x;
+                if (nx.y != mykey) {
+                    mykey = nx.y;
+#pragma unroll
+                    for (int r = 0; r < NR; r++)
+#pragma unroll
+                        for (int i = 0; i < C; i++)
+#pragma unroll
+                            for (int e = 0; e < V; e++) a[r][i][e] = a_nxt[r][i][e];
+                }
+                const int nk = cur + 1 < PSP_WAVE ? w_seg[cur + 1].y : -1;
+                if (nk >= 0 && nk != mykey) load_a(nk, a_nxt);
+            }
         }
         if (ok) {
             if constexpr (BCSR) {
@@ -142,7 +205,7 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
 }
 
 typedef void (*psp_sddmm_kernel_t)(const int *, const int *, const float *, const int *, const float *,
-                                   const float *, float *, int, int, int, int);
+                                   const float *, float *, int, int, int, int, int);
 
 // (LOGL, C, U) triples that exist.  C grows only once the group is 16 lanes wide (DPP-only reduction);
 // beyond 64 vectors the group widens to 32 and 64 lanes.

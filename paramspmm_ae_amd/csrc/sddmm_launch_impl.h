@@ -28,10 +28,16 @@ int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, con
                                  : psp_sddmm_lookup<BCSR, SPLIT, false>(logL, C, V);
     if (!k) return psp_fail(PSP_ERR_ARG, "sddmm: no kernel for logL %d coarsen %d vec %d", logL, C, V);
 
-    const int rows_per_block = blkWarpNum * (PSP_WAVE >> logL);
-    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, rows_per_block), psp_stripe_rows() / rows_per_block);
+    // segments per wavefront: as for SpMM (one per lane group for plain input, 16 for row-split input, fewer for
+    // small matrices)
+    const int logR = 6 - logL;
+    int logW = SPLIT ? (logR > 4 ? logR : 4) : logR;
+    while (logW > 0 && (nrows >> logW) < 4096) logW--;
+    if (logW < logR - 1) logW = logR - 1;
+    const int segs_per_block = blkWarpNum << logW;
+    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block), psp_stripe_rows() / segs_per_block);
     dim3 grid(g.launch, 1, 1), block(blkWarpNum * PSP_WAVE, 1, 1);
     hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, BCSR ? val : scale, target_row, A, B, out, nrows, K,
-                       g.real, g.stripe);
+                       logW, g.real, g.stripe);
     return psp_check_launch("sddmm kernel");
 }

@@ -21,21 +21,8 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
         PSP_REQUIRE(!SPLIT || target_row, "spmm: target_row is null");
     }
 
-    // rows the kernel does not store to must read as zero
-    if (SPLIT) {
-        rc = psp_zero_f32(Y, (size_t)rows_out * N, stream);
-    } else {
-        const size_t covered = (size_t)nrows * NR;
-        rc = psp_zero_f32(Y + covered * N, ((size_t)rows_out - covered) * N, stream);
-    }
-    if (rc != PSP_OK) return rc;
-    if (nrows == 0) return PSP_OK;
-
     int logL = 0;
     while ((1 << logL) < plan.lanes_per_row) logL++;
-    psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll);
-    if (!k) return psp_fail(PSP_ERR_ARG, "spmm: no kernel for coarsen %d vec %d unroll %d", plan.coarsen, plan.vec, plan.unroll);
-
     // Segments per wavefront.  Plain input gets one row per lane group on average: rows that are neighbours in
     // the matrix are then walked at the same time and share their X rows in the L1 / L2, while the even division
     // of the wavefront's entries still levels moderate differences in row length.  Row-split input means the
@@ -49,6 +36,28 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     if (w_env && atoi(w_env) >= 0 && atoi(w_env) <= 6) logW = atoi(w_env);
     while (logW > 0 && (nrows >> logW) < 4096) logW--;
     if (logW < logR - 1) logW = logR - 1;
+
+    // rows the kernel does not store to must read as zero
+    if (SPLIT) {
+        // The kernel stores rows that one wavefront holds alone and adds (atomics) to rows shared by several
+        // wavefronts.  Large outputs are therefore not cleared as a whole: a pass over the segments clears only
+        // the shared rows and the rows without segments.  Small outputs are cheaper to clear outright.
+        size_t clear_min = (size_t)32 << 20;  // floats
+        if (const char *c_env = getenv("PSP_SPLIT_CLEAR_MIN")) clear_min = (size_t)atoll(c_env);  // tuning / test aid
+        if ((size_t)rows_out * N >= clear_min && nrows > 0)
+            rc = psp_split_clear(rowPtr, target_row, Y, nrows, N, NR, rows_out, logW, stream);
+        else
+            rc = psp_zero_f32(Y, (size_t)rows_out * N, stream);
+    } else {
+        const size_t covered = (size_t)nrows * NR;
+        rc = psp_zero_f32(Y + covered * N, ((size_t)rows_out - covered) * N, stream);
+    }
+    if (rc != PSP_OK) return rc;
+    if (nrows == 0) return PSP_OK;
+
+    psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll);
+    if (!k) return psp_fail(PSP_ERR_ARG, "spmm: no kernel for coarsen %d vec %d unroll %d", plan.coarsen, plan.vec, plan.unroll);
+
     int align_pct = 50;
     const char *a_env = getenv("PSP_ALIGN_PCT");  // tuning aid
     if (a_env) align_pct = atoi(a_env);

@@ -220,13 +220,13 @@ def fit_main(args):
         lab = pd.concat([info, pd.DataFrame({"OP_SpMM": y})], axis=1)
         lab.to_csv(os.path.join(args.data, "dim%d_OP_SpMM.csv" % d), index=False)
         best = None
-        for n_est in (30, 50, 80):
+        for n_est in (20, 30, 50, 80):  # the notebook uses 30 / 50 / 80; a larger forest must earn its size
             clf = RandomForestClassifier(n_estimators=n_est, n_jobs=-1, random_state=17)
             clf.fit(X[tr], y[tr])
             pick = clf.predict(X[te])
             norm = TP[te, pick] / TP[te].max(axis=1)  # normalised performance of the pick
             score = (float(np.mean(norm >= 1 / 1.10)), float(norm.mean()))
-            if best is None or score > best[0]:
+            if best is None or score[0] > best[0][0] + 1e-9:
                 best = (score, n_est, clf, pick, norm)
         (within10, mean_norm), n_est, clf, pick, norm = best
         report["per_dim"][d] = {

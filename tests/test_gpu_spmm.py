@@ -127,3 +127,30 @@ def test_spmm_linearity_and_format_agreement_at_scale(oracle):
     # and one width against the oracle at this size
     want = oracle.spmm_csr(rowPtr, colIdx, val, X1[:, :16].contiguous().cpu().numpy())
     assert_close(spmm_capi("csr", F, X1[:, :16].contiguous(), 1, 4), want, what="rmat17 N=16")
+
+
+@pytest.mark.parametrize("fmt", ["csr_split", "bcsr_split"])
+def test_split_selective_clear_path(oracle, fmt, monkeypatch):
+    """Large outputs of the row-split formats are not cleared as a whole: only rows shared by two wavefronts, rows
+    of empty segments and rows without segments are.  Force that path on a small matrix with long rows, empty
+    rows at the start, in the middle and at the end, and a poisoned Y."""
+    from gpu_util import Formats, spmm_capi, spmm_oracle, spmm_abs_scale, assert_close
+
+    monkeypatch.setenv("PSP_SPLIT_CLEAR_MIN", "0")
+    rowPtr, colIdx, val = random_csr(6000, 14, 21, empty_frac=0.3, hub=(3000, 2500), values="uniform")
+    k = np.diff(rowPtr).copy()
+    k[:70] = 0
+    k[-90:] = 0
+    k[1000:1400] = 0
+    keep = np.repeat(k > 0, np.diff(rowPtr))
+    rowPtr = np.concatenate([[0], np.cumsum(k)]).astype(np.int32)
+    colIdx, val = colIdx[keep], val[keep]
+    F = Formats(oracle, rowPtr, colIdx, val, g=8, gb=8)
+    for N in (16, 128):
+        X = np.random.default_rng(N).standard_normal((F.n, N)).astype(np.float32)
+        want = spmm_oracle(oracle, fmt, F, X)
+        scale = spmm_abs_scale(oracle, F, X, want.shape[0])
+        for CF, bw in ((1, 4), (2 if N > 32 else 1, 8)):
+            got = spmm_capi(fmt, F, torch.from_numpy(X).cuda(), CF, bw)
+            torch.cuda.synchronize()
+            assert_close(got, want, what="%s N=%d CF=%d selective clear" % (fmt, N, CF), scale=scale)
