@@ -77,15 +77,27 @@ def bench_agnn(args):
     import ParamSpMM
     from paramspmm_ae_amd import synth
 
-    graph = "C2" if args.graph == "C2" else args.graph
+    from paramspmm_ae_amd.decider import SpMMDecider
+    from paramspmm_ae_amd.graph_input import graph_input
+
+    graph = args.graph
     rowPtr, colIdx, val, n = synth.config_graph(graph)
     nnz = colIdx.size
-    rp, ci, v = (torch.from_numpy(a).cuda() for a in (rowPtr, colIdx, val))
+    g = graph_input(graph, "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val)
+    dec = SpMMDecider()
+    dec.gen_model_dict([32])
+    if_split, _, CF, bw = dec.config_PCSR(g, 32)  # the edge values live in CSR order, so the CSR layouts are used
+    c = g.csr_data
+    rp, ci, v = c.rowPtr.cuda(), c.colIdx.cuda(), c.val.cuda()
+    rps, tr = c.rowPtr_split.cuda(), c.target_row.cuda()
     gen = torch.Generator(device="cuda").manual_seed(7)
     out = {"metric": "AGNN attention layer stack: SDDMM + row softmax + SpMM(N=32), 5 layers", "unit": "ms per 5 layers",
            "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "higher_is_better": False, "scaling": "weak",
            "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-           "config": {"workload": "%s pattern, K in (32, 64), H [n, 32]" % graph, "nodes": n, "nnz": nnz}, "per_K": []}
+           "config": {"workload": "%s pattern, K in (32, 64), H [n, 32]" % graph, "nodes": n, "nnz": nnz,
+                      "format": "csr_split" if if_split else "csr", "CF": CF, "blkWarpNum": bw}, "per_K": []}
     H = torch.randn(n, 32, device="cuda", generator=gen)
     for K in (32, 64):
         X = torch.nn.functional.normalize(torch.randn(n, K, device="cuda", generator=gen), dim=1).contiguous()
@@ -94,9 +106,14 @@ def bench_agnn(args):
         def layers():
             h = H
             for _ in range(5):
-                e = ParamSDDMM.csr_sddmm_scaled(X, Y, rp, ci, v, 8)
-                a = ParamSDDMM.segment_softmax(rp, e)
-                h = ParamSpMM.csr_spmm(h, rp, ci, a, 1, 8)
+                if if_split:
+                    e = ParamSDDMM.csr_split_sddmm_scaled(X, Y, rps, ci, v, tr, bw)
+                    a = ParamSDDMM.segment_softmax(rp, e)
+                    h = ParamSpMM.csr_split_spmm(h, rps, ci, a, tr, CF, bw)
+                else:
+                    e = ParamSDDMM.csr_sddmm_scaled(X, Y, rp, ci, v, bw)
+                    a = ParamSDDMM.segment_softmax(rp, e)
+                    h = ParamSpMM.csr_spmm(h, rp, ci, a, CF, bw)
             return h
 
         for _ in range(args.warmup):

@@ -170,9 +170,12 @@ PSP_EXPORT int psp_genmask(const int *rowPtr_b, const int *rowPtr, const float *
 }
 
 // ------------------------------------------------------------------------------------------------
-// segment softmax: 16 lanes per row, three sweeps over the row (max, sum, write); rows of up to 16
-// entries never re-read memory
+// segment softmax.  Phase 1: 16 lanes per row, three sweeps over the row (max, sum, write); rows of up to 16
+// entries never re-read memory.  Rows longer than PSP_SOFTMAX_LONG entries are left to phase 2, where the whole
+// workgroup (256 lanes) takes them one at a time, so a hub row does not serialise on 16 lanes.
 // ------------------------------------------------------------------------------------------------
+#define PSP_SOFTMAX_LONG 1024
+
 __device__ __forceinline__ float psp_max16(float v)
 {
     v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), 0xB1, 0xF, 0xF, false)));
@@ -185,6 +188,13 @@ __device__ __forceinline__ float psp_max16(float v)
 __global__ void __launch_bounds__(256)
 psp_segment_softmax_kernel(const int *__restrict__ rowPtr, const float *in, float *out, int M)
 {
+    __shared__ int s_long[16];    // rows of this workgroup left to phase 2
+    __shared__ int s_nlong;
+    __shared__ float s_red[4];    // one slot per wavefront
+    const float NEG = -3.402823466e+38f;
+    if (threadIdx.x == 0) s_nlong = 0;
+    __syncthreads();
+
     const int row = (blockIdx.x * blockDim.x + threadIdx.x) >> 4;
     const int sub = threadIdx.x & 15;
     int lb = 0, hb = 0;
@@ -192,20 +202,47 @@ psp_segment_softmax_kernel(const int *__restrict__ rowPtr, const float *in, floa
         lb = rowPtr[row];
         hb = rowPtr[row + 1];
     }
-    if (lb == hb) return;  // whole 16-lane group leaves together
-    const float NEG = -3.402823466e+38f;
-    const float first = (lb + sub < hb) ? in[lb + sub] : NEG;
-    float mx = first;
-    for (int p = lb + 16 + sub; p < hb; p += 16) mx = fmaxf(mx, in[p]);
-    mx = psp_max16(mx);
-    float s = (lb + sub < hb) ? __expf(first - mx) : 0.0f;
-    for (int p = lb + 16 + sub; p < hb; p += 16) s += __expf(in[p] - mx);
-    s = psp_group_sum<4>(s);
-    const float inv = 1.0f / s;
-    // all reads of a chunk happen before its writes, so in == out is fine
-    float e0 = __expf(first - mx) * inv;
-    for (int p = lb + 16 + sub; p < hb; p += 16) out[p] = __expf(in[p] - mx) * inv;
-    if (lb + sub < hb) out[lb + sub] = e0;
+    if (hb - lb > PSP_SOFTMAX_LONG) {
+        if (sub == 0) s_long[atomicAdd(&s_nlong, 1)] = row;
+    } else if (lb < hb) {  // a 16-lane group is uniform here
+        const float first = (lb + sub < hb) ? in[lb + sub] : NEG;
+        float mx = first;
+        for (int p = lb + 16 + sub; p < hb; p += 16) mx = fmaxf(mx, in[p]);
+        mx = psp_max16(mx);
+        float s = (lb + sub < hb) ? __expf(first - mx) : 0.0f;
+        for (int p = lb + 16 + sub; p < hb; p += 16) s += __expf(in[p] - mx);
+        s = psp_group_sum<4>(s);
+        const float inv = 1.0f / s;
+        // all reads of a chunk happen before its writes, so in == out is fine
+        const float e0 = __expf(first - mx) * inv;
+        for (int p = lb + 16 + sub; p < hb; p += 16) out[p] = __expf(in[p] - mx) * inv;
+        if (lb + sub < hb) out[lb + sub] = e0;
+    }
+    __syncthreads();
+
+    const int nlong = s_nlong;  // workgroup-uniform
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = 0; i < nlong; i++) {
+        const int r = s_long[i];
+        const int a = rowPtr[r], b = rowPtr[r + 1];
+        float mx = NEG;
+        for (int p = a + threadIdx.x; p < b; p += 256) mx = fmaxf(mx, in[p]);
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+        if (lane == 0) s_red[wave] = mx;
+        __syncthreads();
+        mx = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+        __syncthreads();
+        float s = 0.0f;
+        for (int p = a + threadIdx.x; p < b; p += 256) s += __expf(in[p] - mx);
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) s += __shfl_xor(s, d);
+        if (lane == 0) s_red[wave] = s;
+        __syncthreads();
+        const float inv = 1.0f / (s_red[0] + s_red[1] + s_red[2] + s_red[3]);
+        __syncthreads();
+        for (int p = a + threadIdx.x; p < b; p += 256) out[p] = __expf(in[p] - mx) * inv;
+    }
 }
 
 PSP_EXPORT int psp_segment_softmax_f32(const int *rowPtr, const float *in, float *out, int M, psp_stream_t stream)

@@ -90,6 +90,12 @@ static Tensor csr_sddmm_scaled(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx,
     return sddmm_new(0, A, B, rowPtr, colIdx, values, nullptr, &values, 1, blkWarpNum);
 }
 
+static Tensor csr_split_sddmm_scaled(Tensor A, Tensor B, Tensor rowPtr_split, Tensor colIdx, Tensor values,
+                                     Tensor target_row, int blkWarpNum)
+{
+    return sddmm_new(1, A, B, rowPtr_split, colIdx, values, &target_row, &values, 1, blkWarpNum);
+}
+
 // ---- *_profile twins (SDDMM/sddmm.cpp:338-661): int GFLOP/s = 2*nnz*K / t -------------------------------
 static int profile_impl(int fmt, const Tensor &A, const Tensor &B, const Tensor &rowPtr, const Tensor &colIdx,
                         const Tensor &values, const Tensor *target_row, long nnz, int CF, int blkWarpNum)
@@ -189,5 +195,6 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("genmask", &genmask, "CSR slot -> flat index into the 2x1 block values");
     // additions of this build
     m.def("csr_sddmm_scaled", &csr_sddmm_scaled, "values[p] * <A[row], B[col]>");
+    m.def("csr_split_sddmm_scaled", &csr_split_sddmm_scaled, "values[p] * <A[row], B[col]> on the row-split format");
     m.def("segment_softmax", &segment_softmax, "softmax over the stored entries of each CSR row");
 }

@@ -95,3 +95,23 @@ def test_segment_softmax_parity(oracle, small):
     # in place
     _capi.check(_capi.lib.psp_segment_softmax_f32(p(F.d["rowPtr"]), p(ed), p(ed), F.n, stream()))
     assert_close(ed, out.cpu().numpy(), rtol=0, atol=0, what="softmax in place")
+
+
+def test_segment_softmax_long_rows(oracle):
+    """Rows above 1024 entries are handled by a whole workgroup; several in one workgroup's 16 rows, plus empty rows."""
+    from paramspmm_ae_amd import _capi
+    from gpu_util import stream, assert_close
+
+    rowPtr, colIdx, val = random_csr(5000, 6, 4, empty_frac=0.3, hub=(17, 4000))
+    k = np.diff(rowPtr).copy()
+    k[18], k[21], k[4999] = 1500, 1025, 2049
+    rowPtr = np.concatenate([[0], np.cumsum(k)]).astype(np.int32)
+    e = (np.random.default_rng(2).standard_normal(rowPtr[-1]) * 5).astype(np.float32)
+    ed = torch.from_numpy(e).cuda()
+    rp = torch.from_numpy(rowPtr).cuda()
+    out = torch.full_like(ed, float("nan"))
+    p = _capi.ptr
+    _capi.check(_capi.lib.psp_segment_softmax_f32(p(rp), p(ed), p(out), rowPtr.size - 1, stream()))
+    assert_close(out, oracle.segment_softmax(rowPtr, e), rtol=1e-5, atol=1e-6, what="softmax long rows")
+    _capi.check(_capi.lib.psp_segment_softmax_f32(p(rp), p(ed), p(ed), rowPtr.size - 1, stream()))
+    assert_close(ed, out.cpu().numpy(), rtol=0, atol=0, what="softmax long rows in place")
