@@ -142,6 +142,15 @@ int psp_sddmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b, const fl
  * ------------------------------------------------------------------------------------------- */
 int psp_segment_softmax_f32(const int *rowPtr, const float *in, float *out, int M, psp_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * DEVICE: C[K1,K2] = A^T * B for tall-skinny row-major A [n,K1] and B [n,K2]; C is overwritten.
+ * Stands in for the weight-gradient product torch::mm(H.t(), AG) of the fused GCN backward
+ * (SpCONV/SpCONV.h:70) when both widths are 16, 32, 48 or 64 (psp_gemm_atb_supported tells); partial products of
+ * row bands are added with fp32 atomics, so the summation order is not fixed.
+ * ------------------------------------------------------------------------------------------- */
+int psp_gemm_atb_supported(int K1, int K2);
+int psp_gemm_atb_f32(const float *A, const float *B, float *C, long long n, int K1, int K2, psp_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

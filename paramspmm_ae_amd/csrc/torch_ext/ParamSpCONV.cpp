@@ -24,6 +24,21 @@ static Tensor aggregate(int fmt, const Tensor &D, const Tensor &rowPtr, const Te
     return Y;
 }
 
+// H^T * AG.  For narrow layers the product is a reduction over ~10^6 rows into a tiny matrix, which the library
+// streams at memory speed; everything else goes to torch::mm.
+static Tensor weight_gradient(const Tensor &H, const Tensor &AG)
+{
+    const bool narrow = H.dim() == 2 && AG.dim() == 2 && H.size(0) == AG.size(0) && H.size(0) >= 16384 &&
+                        H.scalar_type() == torch::kFloat32 && AG.scalar_type() == torch::kFloat32 &&
+                        psp_gemm_atb_supported((int)H.size(1), (int)AG.size(1));
+    if (!narrow) return torch::mm(H.t(), AG);
+    Tensor Hc = H.contiguous(), Gc = AG.contiguous();
+    DeviceGuard guard(Hc.device());
+    Tensor dW = torch::empty({Hc.size(1), Gc.size(1)}, Hc.options());
+    ok(psp_gemm_atb_f32(fp(Hc), fp(Gc), fpw(dW), Hc.size(0), (int)Hc.size(1), (int)Gc.size(1), stream_of(Hc)));
+    return dW;
+}
+
 static Tensor forward_impl(int fmt, const Tensor &H, const Tensor &W, const Tensor &rowPtr, const Tensor &colIdx,
                            const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
 {
@@ -41,7 +56,7 @@ static std::vector<Tensor> backward_impl(int fmt, const Tensor &dY, const Tensor
     // the reference multiplies by A, not A^T (SpCONV/SpCONV.h:67-71): exact for the symmetric matrices its
     // loaders build
     Tensor AG = aggregate(fmt, dY, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
-    return {torch::mm(AG, W.t()), torch::mm(H.t(), AG)};
+    return {torch::mm(AG, W.t()), weight_gradient(H, AG)};
 }
 
 #define PSP_CONV(NAME, FMT)                                                                                       \
@@ -75,6 +90,12 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
     m.def("split_csr", &pspglue::split_csr, "row split on the host");
     m.def("split_csr_par", &pspglue::split_csr_par, "row split on the host with a precomputed segment prefix");
+    // addition of this build: H^T * G for tall-skinny operands (memory-speed kernel for widths 16..64, else torch::mm)
+    m.def("weight_gradient", [](Tensor H, Tensor G) {
+        need_gpu(H, "H");
+        need_gpu(G, "G");
+        return weight_gradient(H, G);
+    }, "H^T * G");
     m.def("csr_spmm_forward", &csr_spmm_forward, "A*(H*W), CSR");
     m.def("csr_spmm_backward", &csr_spmm_backward, "[dH, dW], CSR");
     m.def("csr_split_spmm_forward", &csr_split_spmm_forward, "A*(H*W), row-split CSR");

@@ -86,7 +86,7 @@ class AGNNFunction(torch.autograd.Function):
         d_output = d_output.contiguous()
         d_input_prime = op.AGNN_spmm(edge_attentions, d_output)
         d_input = torch.mm(d_input_prime, weights.t().contiguous())
-        d_weights = torch.mm(X.t().contiguous(), d_input_prime)
+        d_weights = SpCONV.weight_gradient(X, d_input_prime)  # X^T * d_input_prime
         d_attention = op.AGNN_sddmm(d_output)
         if d_attention.dim() != 1:
             d_attention = d_attention.view(-1)[op.mask]  # block layout -> CSR slots
@@ -117,7 +117,7 @@ class GINFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_output):
         X_agg, weights = ctx.saved_tensors
-        d_weights = torch.mm(X_agg.t(), d_output)
+        d_weights = SpCONV.weight_gradient(X_agg, d_output.contiguous())  # X_agg^T * d_output
         d_input = ctx.ParamSpMM.GIN_spmm(torch.mm(d_output, weights.t()).contiguous())
         return d_input, d_weights, None
 

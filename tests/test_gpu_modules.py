@@ -201,3 +201,26 @@ def test_training_driver_runs_gcn_gin_agnn():
         res = GNN.main(["--net", net, "--synthetic", "C1", "--hidden_list", "16", "--num_classes", "16",
                         "--num_features", "32", "--num_epoches", "3", "--config", "0", "2", "1", "4"])
         assert all(ms > 0 for ms in res.values())
+
+
+@pytest.mark.parametrize("K1,K2", [(16, 16), (32, 16), (16, 64), (48, 32), (64, 64)])
+def test_tall_skinny_weight_gradient_product(K1, K2):
+    """psp_gemm_atb_f32 (the H^T * AG of the fused GCN backward) against a float64 product; n is not a multiple
+    of the 64-row tile and the output is poisoned first."""
+    from paramspmm_ae_amd import _capi
+
+    n = 70_001
+    g = torch.Generator(device="cuda").manual_seed(K1 * 100 + K2)
+    A = torch.randn(n, K1, device="cuda", generator=g)
+    B = torch.randn(n, K2, device="cuda", generator=g)
+    C = torch.full((K1, K2), float("nan"), device="cuda")
+    p = _capi.ptr
+    assert _capi.lib.psp_gemm_atb_supported(K1, K2) == 1 and _capi.lib.psp_gemm_atb_supported(K1, 20) == 0
+    _capi.check(_capi.lib.psp_gemm_atb_f32(p(A), p(B), p(C), n, K1, K2, torch.cuda.current_stream().cuda_stream))
+    want = A.double().t() @ B.double()
+    # fp32 accumulation over 70k terms of magnitude ~1: error ~ sqrt(n) * eps * |terms|
+    torch.testing.assert_close(C.double(), want, rtol=1e-4, atol=2e-2)
+    assert _capi.lib.psp_gemm_atb_f32(p(A), p(B), p(C), n, K1, 20, None) == -1
+    _capi.check(_capi.lib.psp_gemm_atb_f32(p(A), p(B), p(C), 0, K1, K2, None))
+    torch.cuda.synchronize()
+    assert bool((C == 0).all())
