@@ -145,7 +145,7 @@ int psp_segment_softmax_f32(const int *rowPtr, const float *in, float *out, int 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: C[K1,K2] = A^T * B for tall-skinny row-major A [n,K1] and B [n,K2]; C is overwritten.
  * Stands in for the weight-gradient product torch::mm(H.t(), AG) of the fused GCN backward
- * (SpCONV/SpCONV.h:70) when both widths are 16, 32, 48 or 64 (psp_gemm_atb_supported tells); partial products of
+ * (SpCONV/SpCONV.h:70) when both widths are multiples of 16 up to 128 (psp_gemm_atb_supported tells); partial products of
  * row bands are added with fp32 atomics, so the summation order is not fixed.
  * ------------------------------------------------------------------------------------------- */
 int psp_gemm_atb_supported(int K1, int K2);

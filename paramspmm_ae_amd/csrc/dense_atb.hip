@@ -1,4 +1,4 @@
-// C[K1,K2] = A^T * B for tall-skinny A [n,K1], B [n,K2] (n ~ 10^6, K1,K2 <= 64): the weight-gradient product
+// C[K1,K2] = A^T * B for tall-skinny A [n,K1], B [n,K2] (n ~ 10^6, K1,K2 multiples of 16 up to 128): the weight-gradient product
 // H^T * (A dY) of the fused GCN layer (SpCONV/SpCONV.h:70 calls torch::mm(H.t(), AG)).  The product is a
 // reduction over n with a tiny output; a general GEMM picks tiles for large outputs and runs it 20-40 times
 // slower than the memory traffic allows.  Here every workgroup streams a contiguous band of rows through LDS
@@ -7,14 +7,13 @@
 #include "psp_common.h"
 #include "spmm_kernel.h"
 
-#define ATB_ROWS 64
-
 template <int K1, int K2>
 __global__ void __launch_bounds__(256)
 psp_atb_kernel(const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, long long n,
                long long rows_per_block)
 {
     constexpr int RM = K1 / 16, RN = K2 / 16;
+    constexpr int ATB_ROWS = (K1 + K2 > 128) ? 32 : 64;  // at most 32 KB of LDS per workgroup
     __shared__ float sA[ATB_ROWS][K1];
     __shared__ float sB[ATB_ROWS][K2];
     const int t = threadIdx.x;
@@ -68,8 +67,8 @@ static psp_atb_kernel_t atb_lookup(int K1, int K2)
 {
 #define ATB_CASE(a, b) \
     if (K1 == a && K2 == b) return psp_atb_kernel<a, b>;
-#define ATB_ROW(a) ATB_CASE(a, 16) ATB_CASE(a, 32) ATB_CASE(a, 48) ATB_CASE(a, 64)
-    ATB_ROW(16) ATB_ROW(32) ATB_ROW(48) ATB_ROW(64)
+#define ATB_ROW(a) ATB_CASE(a, 16) ATB_CASE(a, 32) ATB_CASE(a, 48) ATB_CASE(a, 64) ATB_CASE(a, 80) ATB_CASE(a, 96) ATB_CASE(a, 112) ATB_CASE(a, 128)
+    ATB_ROW(16) ATB_ROW(32) ATB_ROW(48) ATB_ROW(64) ATB_ROW(80) ATB_ROW(96) ATB_ROW(112) ATB_ROW(128)
 #undef ATB_ROW
 #undef ATB_CASE
     return nullptr;
@@ -82,11 +81,12 @@ PSP_EXPORT int psp_gemm_atb_f32(const float *A, const float *B, float *C, long l
 {
     PSP_REQUIRE(n >= 0 && K1 >= 1 && K2 >= 1, "gemm_atb: bad size");
     psp_atb_kernel_t k = atb_lookup(K1, K2);
-    PSP_REQUIRE(k != nullptr, "gemm_atb: K1 and K2 must be 16, 32, 48 or 64 (got %d, %d)", K1, K2);
+    PSP_REQUIRE(k != nullptr, "gemm_atb: K1 and K2 must be multiples of 16 up to 128 (got %d, %d)", K1, K2);
     PSP_REQUIRE(C != nullptr && (n == 0 || (A && B)), "gemm_atb: null pointer");
     int rc = psp_zero_f32(C, (size_t)K1 * K2, (hipStream_t)stream);
     if (rc != PSP_OK || n == 0) return rc;
     // about 8 workgroups per CU, each on a contiguous band of whole 64-row tiles
+    const int ATB_ROWS = 64;
     long long blocks = (n + ATB_ROWS - 1) / ATB_ROWS;
     if (blocks > 2048) blocks = 2048;
     long long rows_per_block = ((n + blocks - 1) / blocks + ATB_ROWS - 1) / ATB_ROWS * ATB_ROWS;

@@ -203,7 +203,7 @@ def test_training_driver_runs_gcn_gin_agnn():
         assert all(ms > 0 for ms in res.values())
 
 
-@pytest.mark.parametrize("K1,K2", [(16, 16), (32, 16), (16, 64), (48, 32), (64, 64)])
+@pytest.mark.parametrize("K1,K2", [(16, 16), (32, 16), (16, 64), (48, 32), (64, 64), (128, 128), (112, 16), (32, 128)])
 def test_tall_skinny_weight_gradient_product(K1, K2):
     """psp_gemm_atb_f32 (the H^T * AG of the fused GCN backward) against a float64 product; n is not a multiple
     of the 64-row tile and the output is poisoned first."""
