@@ -168,6 +168,7 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of X (known size) so a counter run can be calibrated")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-vendor", action="store_true", help="skip the rocSPARSE comparison leg")
     ap.add_argument("--dump", default=None, help="write the full sweep table (every column, every width) as JSON")
     ap.add_argument("--workload", choices=["spmm", "agnn", "gcn"], default="spmm",
                     help="spmm: the headline width sweep; agnn: SDDMM -> row softmax -> SpMM attention layers; "
@@ -334,6 +335,22 @@ def main():
         "roofline": roofline,
         "sweep": per_dim,
     }
+
+    if not args.no_vendor:
+        # vendor library beside it: rocSPARSE CSR SpMM (default algorithm), the counterpart of the cuSPARSE baseline
+        # the reference quotes its speed-ups against (SpMM/Baseline_kernel.cu:24-169)
+        import ParamSpMM
+
+        c = ops[0]
+        v_ms = {}
+        for d in dims:
+            v_ms[d] = ParamSpMM.vendor_spmm_time_ms(0, Xs[d][:n].contiguous() if rows != n else Xs[d], c.rowPtr, c.colIdx, c.val, 1, 3)
+        speedups = [v_ms[r["dim"]] / r["ms"] for r in per_dim]
+        out["vendor_baseline"] = {"library": "rocSPARSE rocsparse_spmm, CSR, rocsparse_spmm_alg_default, fp32",
+                                  "gflops": round(flops_step / (sum(v_ms.values()) * 1e-3) / 1e9, 1),
+                                  "ms_per_width": {str(d): round(v_ms[d], 4) for d in dims},
+                                  "speedup_per_width": {str(r["dim"]): round(s_, 2) for r, s_ in zip(per_dim, speedups)},
+                                  "mean_speedup": round(float(np.mean(speedups)), 2)}
 
     if not args.no_cpu:
         # the reference's CPU path: torch.sparse.mm of the CSR tensor (verification.py:18-46), host cores

@@ -40,6 +40,54 @@ def dynamic_CF_prompter(dim, CF_set=None, warp_size=32, verbose=False):
     return keep
 
 
+class _VendorFormatSpMM(object):
+    """Vendor-library SpMM on a re-formatted copy of the graph's CSR matrix (PCSR.py:45-124)."""
+
+    _compute = _profile = _label = None
+
+    def _convert(self, csr):
+        raise NotImplementedError
+
+    def __init__(self, graph, device="cuda"):
+        from scipy.sparse import csr_matrix
+
+        c = graph.csr_data
+        m = csr_matrix((c.val.numpy(), c.colIdx.numpy(), c.rowPtr.numpy()), shape=(graph.mtx_nodes, graph.mtx_nodes))
+        self.idx_a, self.idx_b, self.val = (torch.from_numpy(a).to(device) for a in self._convert(m))
+        self.mtx_nodes = graph.mtx_nodes
+
+    def _dense_input(self, dim, x):
+        if x is None and dim is None:
+            raise ValueError("at least one of x and dim should be given")
+        return torch.ones(self.mtx_nodes, dim, device="cuda") if dim is not None else x.to("cuda")
+
+    def get_spmm_result(self, dim=None, x=None):
+        return getattr(SpMM, self._compute)(self._dense_input(dim, x), self.idx_a, self.idx_b, self.val).to("cpu")
+
+    def profiling(self, dim=None, x=None, verbose=True):
+        X = self._dense_input(dim, x)
+        throughput = getattr(SpMM, self._profile)(X, self.idx_a, self.idx_b, self.val)
+        if verbose:
+            print("{}-> dim: {} gflops: {:.0f}".format(self._label, X.size(1), throughput))
+        return throughput
+
+
+class coo_spmm(_VendorFormatSpMM):
+    _compute, _profile, _label = "cusparse_compute_coo_alg4", "cusparse_profile_coo_alg4", "coo"
+
+    def _convert(self, csr):
+        coo = csr.tocoo()
+        return coo.row.astype("int32"), coo.col.astype("int32"), coo.data.astype("float32")
+
+
+class csc_spmm(_VendorFormatSpMM):
+    _compute, _profile, _label = "cusparse_compute_csc", "cusparse_profile_csc", "csc"
+
+    def _convert(self, csr):
+        csc = csr.tocsc()
+        return csc.indptr.astype("int32"), csc.indices.astype("int32"), csc.data.astype("float32")
+
+
 # (if_split, blocked) -> operator names in the three modules
 _SPMM = {(False, False): "csr_spmm", (True, False): "csr_split_spmm", (False, True): "bcsr_spmm", (True, True): "bcsr_split_spmm"}
 _SDDMM = {(False, False): "csr_sddmm", (True, False): "csr_split_sddmm", (False, True): "bcsr_sddmm", (True, True): "bcsr_split_sddmm"}
@@ -166,6 +214,29 @@ class pcsr_spmm(object):
 
     def profiling(self, dim=None, x=None, verbose=True):
         return self.cf_warpnum_profiling(self.CF, self.blkWarpNum, dim=dim, x=x, verbose=verbose)
+
+    # ---- vendor baselines on the plain CSR arrays (PCSR.py:581-657); served by rocSPARSE here --------------
+    def _vendor(self, compute, profile, label, dim, x, is_profiling, verbose=True):
+        assert torch.cuda.is_available()
+        if self.if_split or self.vec_size != 1:
+            raise ValueError("cusparse only support vec_size=1 and if_split=False")
+        X = self._dense_input(dim, x)
+        if is_profiling:
+            throughput = getattr(SpMM, profile)(X, self.rowPtr, self.colIdx, self.val)
+            if verbose:
+                print("{}-> dim: {} gflops: {:.0f}".format(label, X.size(1), throughput))
+            return throughput
+        return getattr(SpMM, compute)(X, self.rowPtr, self.colIdx, self.val).to("cpu")
+
+    def cusparse_ref(self, dim=None, x=None, is_profiling=False, verbose=True):
+        return self._vendor("cusparse_compute", "cusparse_profile", "cusparse", dim, x, is_profiling, verbose)
+
+    def cusparse_csr_alg2_ref(self, dim=None, x=None, is_profiling=False, verbose=True):
+        return self._vendor("cusparse_compute_csr_alg2", "cusparse_profile_csr_alg2", "cusparse_csr_alg2", dim, x,
+                            is_profiling, verbose)
+
+    def gespmm_ref(self, dim=None, x=None, is_profiling=False, verbose=True):
+        return self._vendor("gespmm_compute", "gespmm_profile", "gespmm", dim, x, is_profiling, verbose)
 
     def time_ms(self, X, CF=None, blkWarpNum=None, warmup=5, iters=20):
         """Mean milliseconds per SpMM launch (an addition of this build; used by the sweep harness)."""

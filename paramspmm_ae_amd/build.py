@@ -39,7 +39,7 @@ def _ext_command(name):
     ] + inc + [
         src, "-o", out,
         "-L" + LIB, "-lparamsp_hip", "-L" + torch_lib, "-lc10", "-lc10_hip", "-ltorch", "-ltorch_cpu", "-ltorch_hip",
-        "-ltorch_python", "-L/opt/rocm/lib", "-lamdhip64",
+        "-ltorch_python", "-L/opt/rocm/lib", "-lamdhip64", "-lrocsparse",
         "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib, "-Wl,-rpath,/opt/rocm/lib",
     ]
 
@@ -47,11 +47,12 @@ def _ext_command(name):
 def build_extensions(force=False):
     os.makedirs(LIB, exist_ok=True)
     hdr = os.path.join(CSRC, "torch_ext", "glue_common.h")
+    hdr2 = os.path.join(CSRC, "torch_ext", "baseline_rocsparse.h")
     todo = []
     for name in MODULES:
         src = os.path.join(CSRC, "torch_ext", name + ".cpp")
         out = os.path.join(LIB, name + ".so")
-        newest = max(os.path.getmtime(src), os.path.getmtime(hdr), os.path.getmtime(os.path.join(ROOT, "include", "paramsp.h")))
+        newest = max(os.path.getmtime(src), os.path.getmtime(hdr), os.path.getmtime(hdr2), os.path.getmtime(os.path.join(ROOT, "include", "paramsp.h")))
         if force or not os.path.exists(out) or os.path.getmtime(out) < newest:
             todo.append(name)
 

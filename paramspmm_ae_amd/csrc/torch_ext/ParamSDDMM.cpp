@@ -1,6 +1,7 @@
 // Python module `ParamSDDMM`: the binding surface of the reference's SDDMM/sddmm.cpp:675-701, backed by
 // libparamsp_hip.so.
 #include "glue_common.h"
+#include "baseline_rocsparse.h"
 
 using namespace pspglue;
 using torch::Tensor;
@@ -173,8 +174,22 @@ static Tensor vec_sddmm(Tensor, Tensor, Tensor, Tensor, Tensor, int, int) { not_
 static Tensor vec_split_sddmm(Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_split_sddmm"); }
 static int vec_sddmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_sddmm_profile"); }
 static int vec_split_sddmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_split_sddmm_profile"); }
-static void cusparse_sddmm_compute(Tensor, Tensor, Tensor, Tensor, Tensor) { not_built("the cuSPARSE SDDMM comparison baseline"); }
-static int cusparse_sddmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor) { not_built("the cuSPARSE SDDMM comparison baseline"); }
+// vendor baseline under the reference's name (SDDMM/sddmm_baseline_kernel.cu): rocSPARSE SDDMM, written in place
+// into `values`, which is also returned
+static Tensor cusparse_sddmm_compute(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values)
+{
+    DeviceGuard guard(A.device());
+    VendorSDDMM op(A, B, rowPtr, colIdx, values);
+    op.run();
+    return values;
+}
+static int cusparse_sddmm_profile(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values)
+{
+    DeviceGuard guard(A.device());
+    VendorSDDMM op(A, B, rowPtr, colIdx, values);
+    const float ms = time_launches((hipStream_t)stream_of(A), kProfileWarmup, kProfileIters, [&] { op.run(); });
+    return gflops(2.0 * (double)values.size(0) * (double)A.size(1), ms);
+}
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
@@ -190,8 +205,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("bcsr_split_sddmm_profile", &bcsr_split_sddmm_profile, "GFLOP/s of bcsr_split_sddmm");
     m.def("vec_sddmm_profile", &vec_sddmm_profile, "not built");
     m.def("vec_split_sddmm_profile", &vec_split_sddmm_profile, "not built");
-    m.def("cusparse_sddmm_compute", &cusparse_sddmm_compute, "not built");
-    m.def("cusparse_sddmm_profile", &cusparse_sddmm_profile, "not built");
+    m.def("cusparse_sddmm_compute", &cusparse_sddmm_compute, "rocSPARSE SDDMM baseline (in place)");
+    m.def("cusparse_sddmm_profile", &cusparse_sddmm_profile, "GFLOP/s of the rocSPARSE SDDMM baseline");
     m.def("genmask", &genmask, "CSR slot -> flat index into the 2x1 block values");
     // additions of this build
     m.def("csr_sddmm_scaled", &csr_sddmm_scaled, "values[p] * <A[row], B[col]>");

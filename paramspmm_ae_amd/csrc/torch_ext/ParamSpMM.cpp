@@ -1,6 +1,7 @@
 // Python module `ParamSpMM`: the binding surface of the reference's SpMM/SpMM.cpp:891-926, backed by
 // libparamsp_hip.so.  Argument order, tensor requirements and return types follow the reference bindings.
 #include "glue_common.h"
+#include "baseline_rocsparse.h"
 
 using namespace pspglue;
 using torch::Tensor;
@@ -75,10 +76,10 @@ static double spmm_time_ms(int fmt, Tensor input, Tensor rowPtr, Tensor colIdx, 
                                  [&] { spmm_into(fmt, Y, input, rowPtr, colIdx, values, tr, CF, blkWarpNum); });
 }
 
-// ---- generic vec_size x 1 blocks and vendor baselines ---------------------------------------------------
+// ---- generic vec_size x 1 blocks and GE-SpMM ---------------------------------------------------------------
 // The reference instantiates vec_spmm only for vec_size 3 (SpMM/SpMM.cpp:352,406) and its decider never
-// selects it (decider.py:63); the cusparse_* / gespmm_* entries are third-party comparison baselines
-// (SpMM/Baseline_kernel.cu).  The names stay importable; calling them reports what is missing.
+// selects it (decider.py:63); gespmm_* is a third-party kernel copied from dgSPARSE (Baseline_kernel.cu:616-857).
+// The names stay importable; calling them reports what is missing.
 [[noreturn]] static void not_built(const char *what)
 {
     TORCH_CHECK(false, what, " is not part of this build (only the PCSR operators csr/csr_split/bcsr/bcsr_split are)");
@@ -87,8 +88,28 @@ static Tensor vec_spmm(Tensor, Tensor, Tensor, Tensor, int, int) { not_built("ve
 static Tensor vec_split_spmm(Tensor, Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_split_spmm (vec_size 3 blocks)"); }
 static int vec_spmm_profile(Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_spmm_profile"); }
 static int vec_split_spmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_split_spmm_profile"); }
-static Tensor baseline4(Tensor, Tensor, Tensor, Tensor) { not_built("the cuSPARSE / GE-SpMM comparison baseline"); }
-static int baseline4_profile(Tensor, Tensor, Tensor, Tensor) { not_built("the cuSPARSE / GE-SpMM comparison baseline"); }
+static Tensor baseline4(Tensor, Tensor, Tensor, Tensor) { not_built("the GE-SpMM comparison baseline"); }
+static int baseline4_profile(Tensor, Tensor, Tensor, Tensor) { not_built("the GE-SpMM comparison baseline"); }
+
+// ---- vendor library baselines: the reference's cusparse_* names, served by rocSPARSE (baseline_rocsparse.h) ----
+#define PSP_VENDOR(NAME, FMT)                                                                                 \
+    static Tensor cusparse_compute##NAME(Tensor X, Tensor ia, Tensor ib, Tensor v) { return vendor_spmm_compute(FMT, X, ia, ib, v); } \
+    static int cusparse_profile##NAME(Tensor X, Tensor ia, Tensor ib, Tensor v) { return vendor_spmm_profile(FMT, X, ia, ib, v); }
+PSP_VENDOR(, kCsr)
+PSP_VENDOR(_csr_alg2, kCsrAlg2)
+PSP_VENDOR(_coo_alg4, kCooAlg4)
+PSP_VENDOR(_csc, kCsc)
+
+// mean ms per call of the rocSPARSE baseline (format 0 csr, 1 csr load-balanced, 2 coo, 3 csc)
+static double vendor_spmm_time_ms(int format, Tensor X, Tensor ia, Tensor ib, Tensor v, int warmup, int iters)
+{
+    TORCH_CHECK(format >= 0 && format <= 3, "format must be 0..3");
+    TORCH_CHECK(warmup >= 0 && iters >= 1, "warmup >= 0 and iters >= 1 required");
+    DeviceGuard guard(X.device());
+    auto Y = torch::zeros_like(X);
+    VendorSpMM op((VendorFormat)format, X, ia, ib, v, Y);
+    return (double)time_launches((hipStream_t)stream_of(X), warmup, iters, [&] { op.run(); });
+}
 
 static py::dict spmm_plan(int N, int CF, int blkWarpNum)
 {
@@ -121,17 +142,18 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("bcsr_split_spmm_profile", &bcsr_split_spmm_profile, "GFLOP/s of bcsr_split_spmm");
     m.def("vec_spmm_profile", &vec_spmm_profile, "not built");
     m.def("vec_split_spmm_profile", &vec_split_spmm_profile, "not built");
-    m.def("cusparse_compute", &baseline4, "not built");
-    m.def("cusparse_profile", &baseline4_profile, "not built");
-    m.def("cusparse_compute_csr_alg2", &baseline4, "not built");
-    m.def("cusparse_profile_csr_alg2", &baseline4_profile, "not built");
-    m.def("cusparse_compute_coo_alg4", &baseline4, "not built");
-    m.def("cusparse_profile_coo_alg4", &baseline4_profile, "not built");
-    m.def("cusparse_compute_csc", &baseline4, "not built");
-    m.def("cusparse_profile_csc", &baseline4_profile, "not built");
+    m.def("cusparse_compute", &cusparse_compute, "rocSPARSE SpMM baseline");
+    m.def("cusparse_profile", &cusparse_profile, "GFLOP/s of the rocSPARSE SpMM baseline");
+    m.def("cusparse_compute_csr_alg2", &cusparse_compute_csr_alg2, "rocSPARSE SpMM baseline");
+    m.def("cusparse_profile_csr_alg2", &cusparse_profile_csr_alg2, "GFLOP/s of the rocSPARSE SpMM baseline");
+    m.def("cusparse_compute_coo_alg4", &cusparse_compute_coo_alg4, "rocSPARSE SpMM baseline");
+    m.def("cusparse_profile_coo_alg4", &cusparse_profile_coo_alg4, "GFLOP/s of the rocSPARSE SpMM baseline");
+    m.def("cusparse_compute_csc", &cusparse_compute_csc, "rocSPARSE SpMM baseline");
+    m.def("cusparse_profile_csc", &cusparse_profile_csc, "GFLOP/s of the rocSPARSE SpMM baseline");
     m.def("gespmm_compute", &baseline4, "not built");
     m.def("gespmm_profile", &baseline4_profile, "not built");
     // additions of this build
     m.def("spmm_time_ms", &spmm_time_ms, "mean ms per launch: (fmt, X, rowPtr, colIdx, val, target_row|None, CF, bw, warmup, iters)");
+    m.def("vendor_spmm_time_ms", &vendor_spmm_time_ms, "mean ms per rocSPARSE SpMM: (format, X, idx_a, idx_b, val, warmup, iters)");
     m.def("spmm_plan", &spmm_plan, "how (N, CF, blkWarpNum) maps onto the wave64 kernel");
 }

@@ -98,7 +98,7 @@ def test_extension_argument_errors():
     with pytest.raises(RuntimeError, match="float32"):
         ParamSpMM.csr_spmm(x.double(), rp, ci, v.double(), 1, 4)
     with pytest.raises(RuntimeError, match="not part of this build"):
-        ParamSpMM.cusparse_compute(x, rp, ci, v)
+        ParamSpMM.gespmm_compute(x, rp, ci, v)
     with pytest.raises(RuntimeError, match="same number of columns"):
         ParamSDDMM.csr_sddmm(x, torch.zeros(8, 8, device="cuda"), rp, ci, v, 1, 4)
     # bcsr output is padded to an even number of rows
@@ -224,3 +224,32 @@ def test_tall_skinny_weight_gradient_product(K1, K2):
     _capi.check(_capi.lib.psp_gemm_atb_f32(p(A), p(B), p(C), 0, K1, K2, None))
     torch.cuda.synchronize()
     assert bool((C == 0).all())
+
+
+def test_vendor_baselines_agree_with_the_oracle(oracle):
+    """The reference's cusparse_* names are served by rocSPARSE: CSR (default and load-balanced), COO and CSC SpMM,
+    and the in-place SDDMM (values <- dot products, SDDMM/sddmm_baseline_kernel.cu:24-80)."""
+    import ParamSDDMM
+    from paramspmm_ae_amd.PCSR import pcsr_spmm, coo_spmm, csc_spmm
+    from gpu_util import assert_close
+
+    n = 2001
+    g, rowPtr, colIdx, val = sym_graph(n, 5)
+    X = np.random.default_rng(0).standard_normal((n, 48)).astype(np.float32)
+    Xd = torch.from_numpy(X).cuda()
+    want = oracle.spmm_csr(rowPtr, colIdx, val, X)
+    scale = oracle.spmm_csr(rowPtr, colIdx, np.abs(val), np.abs(X))
+    op = pcsr_spmm(g, vec_size=1, if_split=False)
+    assert_close(op.cusparse_ref(x=Xd), want, what="rocsparse csr", scale=scale)
+    assert_close(op.cusparse_csr_alg2_ref(x=Xd), want, what="rocsparse csr merge path", scale=scale)
+    assert_close(coo_spmm(g).get_spmm_result(x=Xd), want, what="rocsparse coo", scale=scale)
+    assert_close(csc_spmm(g).get_spmm_result(x=Xd), want, what="rocsparse csc", scale=scale)
+    assert op.cusparse_ref(dim=32, is_profiling=True, verbose=False) > 0
+    with pytest.raises(ValueError):
+        pcsr_spmm(g, vec_size=2, if_split=False).cusparse_ref(dim=16)
+    A = X / np.linalg.norm(X, axis=1, keepdims=True)
+    Ad = torch.from_numpy(A).cuda()
+    vals = op.val.clone()
+    out = ParamSDDMM.cusparse_sddmm_compute(Ad, Ad, op.rowPtr, op.colIdx, vals)
+    assert out.data_ptr() == vals.data_ptr()  # in place, as in the reference
+    assert_close(vals, oracle.sddmm_csr(rowPtr, colIdx, A, A), rtol=1e-5, atol=1e-6, what="rocsparse sddmm")
