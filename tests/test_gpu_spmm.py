@@ -154,3 +154,31 @@ def test_split_selective_clear_path(oracle, fmt, monkeypatch):
             got = spmm_capi(fmt, F, torch.from_numpy(X).cuda(), CF, bw)
             torch.cuda.synchronize()
             assert_close(got, want, what="%s N=%d CF=%d selective clear" % (fmt, N, CF), scale=scale)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_spmm_local_matrices_both_block_sizes(oracle, fmt):
+    """Banded and community-ordered matrices (the structure the cache-friendly configurations have) at both
+    workgroup sizes and several column tilings."""
+    from gpu_util import Formats, spmm_capi, spmm_oracle, spmm_abs_scale, assert_close
+    from paramspmm_ae_amd import synth
+    from paramspmm_ae_amd.train_decider import banded
+
+    graphs = {
+        "band": banded(20_001, 14, 30, seed=1),
+        "sbm": synth.sbm(12_000, 120, 18, 1.5, seed=2),
+    }
+    for name, (r, c, n) in graphs.items():
+        rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+        F = Formats(oracle, rowPtr, colIdx, val)
+        for N, CF in ((16, 1), (64, 1), (64, 2), (128, 4), (96, 3)):
+            print("case", fmt, name, N, CF, flush=True)
+            X = np.random.default_rng(N).standard_normal((F.n + (F.n & 1), N)).astype(np.float32)
+            want = spmm_oracle(oracle, fmt, F, X)
+            scale = spmm_abs_scale(oracle, F, X, want.shape[0])
+            Xd = torch.from_numpy(X).cuda()
+            got8 = spmm_capi(fmt, F, Xd, CF, 8)
+            got4 = spmm_capi(fmt, F, Xd, CF, 4)
+            torch.cuda.synchronize()
+            assert_close(got8, want, what="%s %s N=%d CF=%d bw=8" % (fmt, name, N, CF), scale=scale)
+            assert_close(got4, want, what="%s %s N=%d CF=%d bw=4" % (fmt, name, N, CF), scale=scale)
