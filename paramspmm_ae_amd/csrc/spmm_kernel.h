@@ -42,7 +42,9 @@ template <int V> __device__ __forceinline__ void psp_store_vec(float *p, const f
 #pragma unroll
         for (int e = 0; e < V; e++) t[e] = a[e];
     }
-    *(typename psp_vec<V>::type *)p = t;
+    // Y is written once and not read again by this kernel: the streaming hint keeps it from displacing rows of X
+    // in the L2 (measured 1-5 % faster; the same hint on colIdx / val loads is slower, other column tiles re-read them)
+    __builtin_nontemporal_store(t, (typename psp_vec<V>::type *)p);
 }
 
 __device__ __forceinline__ int psp_bperm_i(int src_lane, int v) { return __builtin_amdgcn_ds_bpermute(src_lane << 2, v); }
