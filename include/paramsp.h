@@ -73,6 +73,37 @@ int psp_bcsr_build(const int *rowPtr, const int *colIdx, const float *val, int n
                    int *rowPtr_b, int *colIdx_b, float *val_b);
 
 /* ---------------------------------------------------------------------------------------------
+ * DEVICE: PCSR index construction on the GPU, the twins of the host builders above (same outputs, bit for
+ * bit).  The reference builds on the host only (SpMM/SpMM.cpp:15-75, graph_input.py:243-274).  Each builder is
+ * two calls with one read-back of a size in between: offsets (count + exclusive scan), then fill.
+ *   workspace: psp_scan_workspace_ints(n) ints of device memory, n = number of scanned items (nrows for the
+ *              split, (nrows+1)/2 for BCSR);
+ *   status:    one device int the caller has set to 0; the kernels OR psp_build_flag bits into it.  With a
+ *              non-zero status the outputs are not valid (the host builders accept such input).
+ * ------------------------------------------------------------------------------------------- */
+enum psp_build_flag {
+    PSP_BUILD_OVERFLOW = 1,  /* a prefix sum left the int32 range */
+    PSP_BUILD_UNSORTED = 2,  /* a row's column indices are not strictly ascending (BCSR builder only) */
+    PSP_BUILD_BAD_ROWPTR = 4 /* rowPtr decreases */
+};
+int psp_scan_workspace_ints(int n);
+
+/* row_split_offset[nrows+1] = exclusive prefix sum of ceil(nnz_i / g): the array graph_input.py:135 computes
+ * with torch.cumsum; row_split_offset[nrows] is S. */
+int psp_split_csr_offsets_dev(const int *rowPtr, int nrows, int g, int *row_split_offset, int *workspace,
+                              int workspace_ints, int *status, psp_stream_t stream);
+/* fills rowPtr_split[S+1] and target_row[S] like psp_split_csr_par. */
+int psp_split_csr_fill_dev(const int *rowPtr, const int *row_split_offset, int nrows, int g, int S,
+                           int *rowPtr_split, int *target_row, psp_stream_t stream);
+
+/* rowPtr_b[(nrows+1)/2+1]; rowPtr_b[(nrows+1)/2] is nblk.  Input rows must hold strictly ascending columns. */
+int psp_bcsr_offsets_dev(const int *rowPtr, const int *colIdx, int nrows, int *rowPtr_b, int *workspace,
+                         int workspace_ints, int *status, psp_stream_t stream);
+/* fills colIdx_b[nblk] and val_b[nblk*2] in the block order of psp_bcsr_build. */
+int psp_bcsr_fill_dev(const int *rowPtr, const int *colIdx, const float *val, int nrows, const int *rowPtr_b,
+                      int *colIdx_b, float *val_b, psp_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * DEVICE: genmask, SDDMM/sddmm.cpp:663-673 -> sddmm_kernel.cu:78-141.
  * mask[nnz] (int32) is fully written: CSR slot -> flat index into val_b of the same non-zero.
  * rowPtr must hold at least 2*nblkrows entries (+1 when the row count is even).

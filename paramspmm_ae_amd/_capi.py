@@ -45,6 +45,11 @@ SIGNATURES = {
     "psp_split_csr_par": [_vp, _vp, _i, _i, _vp, _vp],
     "psp_bcsr_count": [_vp, _vp, _i, _i],
     "psp_bcsr_build": [_vp, _vp, _vp, _i, _i, _vp, _vp, _vp],
+    "psp_scan_workspace_ints": [_i],
+    "psp_split_csr_offsets_dev": [_vp, _i, _i, _vp, _vp, _i, _vp, _vp],
+    "psp_split_csr_fill_dev": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp],
+    "psp_bcsr_offsets_dev": [_vp, _vp, _i, _vp, _vp, _i, _vp, _vp],
+    "psp_bcsr_fill_dev": [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp],
     "psp_genmask": [_vp, _vp, _vp, _i, _i, _vp, _vp],
     "psp_spmm_csr_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "psp_spmm_csr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],

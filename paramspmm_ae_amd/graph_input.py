@@ -7,6 +7,8 @@ and method names its callers use, graph_input.py:17-430), built differently:
 * the BCSR blocks come from ``psp_bcsr_build`` of libparamsp_hip.so (first-encounter block order, i.e. what
   SciPy's ``tobsr`` yields in graph_input.py:245-256) instead of a SciPy conversion;
 * row splitting goes through ``ParamSpMM.split_csr_par`` as in graph_input.py:135-136;
+* with a GPU present both are built there instead (``device_builder``: same arrays bit for bit, copied back so that
+  the attributes stay CPU tensors as in the reference); ``build_on="host"`` keeps the host builders;
 * ``load_from_csr`` accepts arrays directly, so synthetic graphs never touch a ``.mtx`` file.
 """
 import math
@@ -106,15 +108,21 @@ class csr_data(object):
         self.real_avg_degree = (self.num_edges / self.real_nrow).item()
         self._choose_granularity(manual_granularity, is_avg_granularity)
 
-    def get_split(self, verbose=True):
+    def get_split(self, verbose=True, build_on="auto"):
         if self.split_granularity is None:
             raise ValueError("split_granularity is None, must be init first")
-        import ParamSpMM  # the extension module of this build (lib/ParamSpMM.so)
-
         t0 = time.perf_counter()
-        offsets = torch.zeros(self.row_split_nnz.numel() + 1, dtype=torch.int32)
-        offsets[1:] = self.row_split_nnz.cumsum(dim=0).to(torch.int32)
-        self.rowPtr_split, self.target_row = ParamSpMM.split_csr_par(self.rowPtr, offsets, self.split_granularity)
+        if _use_device(build_on):
+            from . import device_builder
+
+            rs, tr = device_builder.split_csr_device(self.rowPtr.cuda(), self.split_granularity)
+            self.rowPtr_split, self.target_row = rs.cpu(), tr.cpu()
+        else:
+            import ParamSpMM  # the extension module of this build (lib/ParamSpMM.so)
+
+            offsets = torch.zeros(self.row_split_nnz.numel() + 1, dtype=torch.int32)
+            offsets[1:] = self.row_split_nnz.cumsum(dim=0).to(torch.int32)
+            self.rowPtr_split, self.target_row = ParamSpMM.split_csr_par(self.rowPtr, offsets, self.split_granularity)
         if verbose:
             print(
                 "get_split -> split time: (ms): {:.3f} split_gran: {} \n split_ratio: {} avg_nnz: {} split_rows: {}".format(
@@ -143,12 +151,32 @@ class csr_data(object):
         print("= split_ratio: {:.5f}".format(float(self.split_ratio)))
 
 
-def build_bcsr(rowPtr, colIdx, val, ncols=None):
-    """CSR (numpy int32/int32/fp32) -> 2x1 BCSR arrays via libparamsp_hip.so (host code)."""
+def _use_device(build_on):
+    if build_on not in ("auto", "host", "device"):
+        raise ValueError("build_on must be 'auto', 'host' or 'device'")
+    if build_on == "device" and not torch.cuda.is_available():
+        raise RuntimeError("build_on='device' needs a GPU")
+    return build_on == "device" or (build_on == "auto" and torch.cuda.is_available())
+
+
+def build_bcsr(rowPtr, colIdx, val, ncols=None, build_on="host"):
+    """CSR (numpy int32/int32/fp32) -> 2x1 BCSR arrays (numpy) via libparamsp_hip.so: the host builder, or the
+    device builder when ``build_on`` says so and the rows are strictly ascending."""
     rowPtr = np.ascontiguousarray(rowPtr, np.int32)
     colIdx = np.ascontiguousarray(colIdx, np.int32)
     val = np.ascontiguousarray(val, np.float32)
     n = rowPtr.size - 1
+    if ncols is None and _use_device(build_on):
+        from . import device_builder
+
+        try:
+            out = device_builder.build_bcsr_device(
+                torch.from_numpy(rowPtr).cuda(), torch.from_numpy(colIdx).cuda(), torch.from_numpy(val).cuda()
+            )
+            return tuple(t.cpu().numpy() for t in out)
+        except device_builder.NotCanonical:
+            if build_on == "device":
+                raise
     ncols = n + (n & 1) if ncols is None else ncols
     nblk = _capi.check(_capi.lib.psp_bcsr_count(_capi.ptr(rowPtr), _capi.ptr(colIdx), n, ncols))
     rowPtr_b = np.empty((n + 1) // 2 + 1, np.int32)
@@ -214,8 +242,9 @@ class graph_input(object):
         )
 
     def load_from_csr(self, rowPtr, colIdx, val, manual_granularity=None, is_avg_granularity=False, blk_size=2,
-                      if_mask=False):
-        """Build every format from a square CSR matrix given as arrays (column indices sorted per row)."""
+                      if_mask=False, build_on="auto"):
+        """Build every format from a square CSR matrix given as arrays (column indices sorted per row).
+        ``build_on``: "host", "device" or "auto" (the GPU when there is one) for the BCSR and row-split arrays."""
         if blk_size != 2:
             raise ValueError("this build only has 2x1 blocks (blk_size=2)")
         t0 = time.perf_counter()
@@ -230,7 +259,7 @@ class graph_input(object):
         self.csr_data = csr_data(rowPtr, colIdx, val, n, nnz, True)
         self.csr_data.init_info(is_avg_granularity=is_avg_granularity, manual_granularity=manual_granularity)
 
-        rowPtr_b, colIdx_b, val_b = build_bcsr(rowPtr, colIdx, val)
+        rowPtr_b, colIdx_b, val_b = build_bcsr(rowPtr, colIdx, val, build_on=build_on)
         nblk = colIdx_b.size
         # graph_input.py:257-266: the blocked format counts block-rows and blocks (the latter as a float)
         self.bcsr_data = csr_data(rowPtr_b, colIdx_b, val_b, (n + 1) // 2, float(nblk), False)
@@ -252,19 +281,19 @@ class graph_input(object):
         self.loaded_flag = True
         self.reordered_flag = True
         self.bcsr_flag = True
-        self.get_split_csr()
-        self.get_split_bcsr()
+        self.get_split_csr(build_on)
+        self.get_split_bcsr(build_on)
         if self.verbose:
             print("data format all preprocess (ms): {:.3f}".format((time.perf_counter() - t0) * 1e3))
         return self
 
-    def get_split_csr(self):
+    def get_split_csr(self, build_on="auto"):
         self.csr_split_flag = True
-        self.csr_data.get_split(self.verbose)
+        self.csr_data.get_split(self.verbose, build_on)
 
-    def get_split_bcsr(self):
+    def get_split_bcsr(self, build_on="auto"):
         self.bcsr_split_flag = True
-        self.bcsr_data.get_split(self.verbose)
+        self.bcsr_data.get_split(self.verbose, build_on)
 
     # ------------------------------------------------------------------------------------------
     def normalize_adj(self, mtx):
