@@ -155,6 +155,57 @@ def bench_gcn(args):
     print(json.dumps(out))
 
 
+def bench_build(args):
+    """PCSR format construction (2x1 BCSR + both row splits): the host builders against the device builders on the
+    same CSR arrays.  Device times start with the CSR arrays on the GPU and end with the built arrays on the GPU
+    (synchronised); `device_roundtrip_ms` adds the upload of the CSR and the copy of the results back to the host,
+    which is what graph_input.load_from_csr pays to keep its CPU-tensor attributes."""
+    import time
+    import torch
+    from paramspmm_ae_amd import synth, device_builder  # the package puts its lib/ directory on sys.path
+    from paramspmm_ae_amd.graph_input import build_bcsr
+    import ParamSpMM
+
+    rowPtr, colIdx, val, n = synth.config_graph(args.graph)
+    g = 32
+    t0 = time.perf_counter()
+    rb, cb, vb = build_bcsr(rowPtr, colIdx, val, build_on="host")
+    k = np.diff(rowPtr)
+    off = np.zeros(n + 1, np.int32)
+    off[1:] = np.cumsum((k + g - 1) // g)
+    ParamSpMM.split_csr_par(torch.from_numpy(rowPtr), torch.from_numpy(off), g)
+    kb = np.diff(rb)
+    offb = np.zeros(rb.size, np.int32)
+    offb[1:] = np.cumsum((kb + g - 1) // g)
+    ParamSpMM.split_csr_par(torch.from_numpy(rb), torch.from_numpy(offb), g)
+    host_ms = (time.perf_counter() - t0) * 1e3
+
+    def device_once(upload):
+        t0 = time.perf_counter()
+        d = [torch.from_numpy(a).cuda() for a in (rowPtr, colIdx, val)] if upload else dev
+        t1 = time.perf_counter()
+        b = device_builder.build_bcsr_device(*d)
+        s1 = device_builder.split_csr_device(d[0], g)
+        s2 = device_builder.split_csr_device(b[0], g)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        if upload:
+            [t.cpu() for t in (*b, *s1, *s2)]
+        return (t2 - t1) * 1e3, (time.perf_counter() - t0) * 1e3
+
+    dev = [torch.from_numpy(a).cuda() for a in (rowPtr, colIdx, val)]
+    device_once(False)
+    dev_ms = min(device_once(False)[0] for _ in range(max(3, args.steps)))
+    round_ms = min(device_once(True)[1] for _ in range(3))
+    print(json.dumps({"metric": "PCSR construction ms (2x1 BCSR + CSR and BCSR row split, g=32)", "unit": "ms", "n_gpus": 1,
+                      "steps": max(3, args.steps), "warmup": 1, "higher_is_better": False, "scaling": "weak",
+                      "vs_baseline": None, "dtype": "i32", "data": "synthetic",
+                      "config": {"workload": "%s format construction" % args.graph, "nodes": n, "nnz": int(rowPtr[-1])},
+                      "value": round(dev_ms, 3), "ms_per_step": round(dev_ms, 3), "device_ms": round(dev_ms, 3),
+                      "device_roundtrip_ms": round(round_ms, 3), "host_ms": round(host_ms, 3),
+                      "speedup_device": round(host_ms / dev_ms, 1), "speedup_roundtrip": round(host_ms / round_ms, 1)}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -170,9 +221,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-vendor", action="store_true", help="skip the rocSPARSE comparison leg")
     ap.add_argument("--dump", default=None, help="write the full sweep table (every column, every width) as JSON")
-    ap.add_argument("--workload", choices=["spmm", "agnn", "gcn"], default="spmm",
+    ap.add_argument("--workload", choices=["spmm", "agnn", "gcn", "build"], default="spmm",
                     help="spmm: the headline width sweep; agnn: SDDMM -> row softmax -> SpMM attention layers; "
-                         "gcn: GCN / GIN training epochs on the SBM graph")
+                         "gcn: GCN / GIN training epochs on the SBM graph; build: PCSR construction, host against device")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (no multi-GPU path exists)" % args.gpus,
@@ -188,6 +239,8 @@ def main():
         return bench_agnn(args)
     if args.workload == "gcn":
         return bench_gcn(args)
+    if args.workload == "build":
+        return bench_build(args)
     from paramspmm_ae_amd import _capi, synth, sweep
     from paramspmm_ae_amd.graph_input import graph_input
 

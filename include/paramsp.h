@@ -182,6 +182,13 @@ int psp_segment_softmax_f32(const int *rowPtr, const float *in, float *out, int 
 int psp_gemm_atb_supported(int K1, int K2);
 int psp_gemm_atb_f32(const float *A, const float *B, float *C, long long n, int K1, int K2, psp_stream_t stream);
 
+/* ---------------------------------------------------------------------------------------------
+ * DEVICE: comparison baseline, ParamSpMM.gespmm_compute (SpMM/Baseline_kernel.cu:616-788): CSR SpMM with one
+ * wavefront per row and the row's (column, value) pairs cached in LDS.  Y [M,N] is fully written.
+ * ------------------------------------------------------------------------------------------- */
+int psp_baseline_rowcache_spmm_f32(const int *rowPtr, const int *colIdx, const float *val, const float *X,
+                                   float *Y, int M, int N, psp_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -76,10 +76,9 @@ static double spmm_time_ms(int fmt, Tensor input, Tensor rowPtr, Tensor colIdx, 
                                  [&] { spmm_into(fmt, Y, input, rowPtr, colIdx, values, tr, CF, blkWarpNum); });
 }
 
-// ---- generic vec_size x 1 blocks and GE-SpMM ---------------------------------------------------------------
+// ---- generic vec_size x 1 blocks ------------------------------------------------------------------------------
 // The reference instantiates vec_spmm only for vec_size 3 (SpMM/SpMM.cpp:352,406) and its decider never
-// selects it (decider.py:63); gespmm_* is a third-party kernel copied from dgSPARSE (Baseline_kernel.cu:616-857).
-// The names stay importable; calling them reports what is missing.
+// selects it (decider.py:63).  The names stay importable; calling them reports what is missing.
 [[noreturn]] static void not_built(const char *what)
 {
     TORCH_CHECK(false, what, " is not part of this build (only the PCSR operators csr/csr_split/bcsr/bcsr_split are)");
@@ -88,8 +87,35 @@ static Tensor vec_spmm(Tensor, Tensor, Tensor, Tensor, int, int) { not_built("ve
 static Tensor vec_split_spmm(Tensor, Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_split_spmm (vec_size 3 blocks)"); }
 static int vec_spmm_profile(Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_spmm_profile"); }
 static int vec_split_spmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_split_spmm_profile"); }
-static Tensor baseline4(Tensor, Tensor, Tensor, Tensor) { not_built("the GE-SpMM comparison baseline"); }
-static int baseline4_profile(Tensor, Tensor, Tensor, Tensor) { not_built("the GE-SpMM comparison baseline"); }
+
+// ---- row-caching baseline under the reference's gespmm_* names (SpMM/Baseline_kernel.cu:744-857) ----------------
+static void rowcache_into(Tensor &Y, const Tensor &X, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values)
+{
+    ok(psp_baseline_rowcache_spmm_f32(ip(rowPtr), ip(colIdx), fp(values), fp(X), fpw(Y), (int)rowPtr.size(0) - 1,
+                                      (int)X.size(1), stream_of(X)));
+}
+static void check_rowcache_args(const Tensor &X, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values)
+{
+    check_spmm_args(0, X, rowPtr, colIdx, values, nullptr);
+    TORCH_CHECK(rowPtr.size(0) - 1 <= X.size(0), "gespmm: the matrix has more rows than the dense input");
+}
+static Tensor gespmm_compute(Tensor X, Tensor rowPtr, Tensor colIdx, Tensor values)
+{
+    check_rowcache_args(X, rowPtr, colIdx, values);
+    pspglue::DeviceGuard guard(X.device());
+    auto Y = torch::zeros_like(X);
+    rowcache_into(Y, X, rowPtr, colIdx, values);
+    return Y;
+}
+static int gespmm_profile(Tensor X, Tensor rowPtr, Tensor colIdx, Tensor values)
+{
+    check_rowcache_args(X, rowPtr, colIdx, values);
+    pspglue::DeviceGuard guard(X.device());
+    auto Y = torch::zeros_like(X);
+    const float ms = time_launches((hipStream_t)stream_of(X), pspglue::kProfileWarmup, pspglue::kProfileIters,
+                                   [&] { rowcache_into(Y, X, rowPtr, colIdx, values); });
+    return (int)(2.0 * (double)values.size(0) * (double)X.size(1) / ((double)ms * 1e-3) / 1e9);
+}
 
 // ---- vendor library baselines: the reference's cusparse_* names, served by rocSPARSE (baseline_rocsparse.h) ----
 #define PSP_VENDOR(NAME, FMT)                                                                                 \
@@ -150,8 +176,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("cusparse_profile_coo_alg4", &cusparse_profile_coo_alg4, "GFLOP/s of the rocSPARSE SpMM baseline");
     m.def("cusparse_compute_csc", &cusparse_compute_csc, "rocSPARSE SpMM baseline");
     m.def("cusparse_profile_csc", &cusparse_profile_csc, "GFLOP/s of the rocSPARSE SpMM baseline");
-    m.def("gespmm_compute", &baseline4, "not built");
-    m.def("gespmm_profile", &baseline4_profile, "not built");
+    m.def("gespmm_compute", &gespmm_compute, "row-caching CSR SpMM baseline (one wavefront per row)");
+    m.def("gespmm_profile", &gespmm_profile, "GFLOP/s of the row-caching baseline");
     // additions of this build
     m.def("spmm_time_ms", &spmm_time_ms, "mean ms per launch: (fmt, X, rowPtr, colIdx, val, target_row|None, CF, bw, warmup, iters)");
     m.def("vendor_spmm_time_ms", &vendor_spmm_time_ms, "mean ms per rocSPARSE SpMM: (format, X, idx_a, idx_b, val, warmup, iters)");

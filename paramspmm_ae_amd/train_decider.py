@@ -55,15 +55,24 @@ def grid_with_holes(nx, ny, drop, seed):
     return r[keep], c[keep], n
 
 
-def corpus():
-    """Deterministic list of (name, builder) covering power-law, R-MAT, community, mesh and banded structure."""
+def corpus(replicas=2):
+    """Deterministic list of (name, builder) covering power-law, R-MAT, community, mesh and banded structure.
+    Every replica walks the same parameter grid with its own random choices (which grid points are skipped, hub
+    degree, ordering, seeds); deterministic structures (plain stencils) appear once."""
+    items = []
+    for rep in range(replicas):
+        _corpus_replica(items, rep)
+    return items
+
+
+def _corpus_replica(items, rep):
     from . import synth
 
-    items = []
-    rng = np.random.default_rng(2024)
+    rng = np.random.default_rng(2024 + rep)
+    suffix = "" if rep == 0 else "_r%d" % rep
 
     def add(name, fn):
-        items.append((name, fn))
+        items.append((name + suffix, fn))
 
     # Chung-Lu power law
     for n in (10_000, 20_000, 60_000, 200_000, 600_000, 1_500_000):
@@ -102,8 +111,11 @@ def corpus():
                         lambda n=n, size=size, din=din, dout=dout, perm=perm, seed=seed:
                         synth.sbm(n, n // size, din, dout, seed=seed, permute=perm))
     # meshes
-    for nx, ny in ((128, 128), (256, 256), (512, 512), (1024, 1024), (2048, 1024), (2048, 2048), (4096, 1024), (8192, 256),
-                   (100, 100), (300, 700), (1000, 500), (3000, 1000), (64, 4096), (1536, 1536)):
+    stencils = ((128, 128), (256, 256), (512, 512), (1024, 1024), (2048, 1024), (2048, 2048), (4096, 1024), (8192, 256),
+                (100, 100), (300, 700), (1000, 500), (3000, 1000), (64, 4096), (1536, 1536))
+    if rep > 0:  # other aspect ratios and sizes
+        stencils = tuple((int(rng.integers(60, 3000)), int(rng.integers(60, 3000))) for _ in range(len(stencils)))
+    for nx, ny in stencils:
         add("stencil_%dx%d" % (nx, ny), lambda nx=nx, ny=ny: synth.stencil2d(nx, ny))
     for nx, ny, drop in ((512, 512, 0.3), (1024, 1024, 0.25), (2048, 1024, 0.4), (1500, 1500, 0.1), (256, 256, 0.2),
                          (2048, 2048, 0.3), (700, 900, 0.5), (400, 4000, 0.15)):
@@ -116,7 +128,6 @@ def corpus():
                 continue
             seed = int(rng.integers(1 << 30))
             add("band_n%d_k%d_w%d" % (n, k, w), lambda n=n, k=k, w=w, seed=seed: banded(n, k, w, seed))
-    return items
 
 
 # ------------------------------------------------------------------------------------------------------------

@@ -97,14 +97,34 @@ def test_extension_argument_errors():
         ParamSpMM.csr_spmm(x, rp.long(), ci, v, 1, 4)
     with pytest.raises(RuntimeError, match="float32"):
         ParamSpMM.csr_spmm(x.double(), rp, ci, v.double(), 1, 4)
+    assert torch.count_nonzero(ParamSpMM.gespmm_compute(x, rp, ci, v)) == 0
     with pytest.raises(RuntimeError, match="not part of this build"):
-        ParamSpMM.gespmm_compute(x, rp, ci, v)
+        ParamSpMM.vec_spmm(x, rp, ci, v, 1, 4)
     with pytest.raises(RuntimeError, match="same number of columns"):
         ParamSDDMM.csr_sddmm(x, torch.zeros(8, 8, device="cuda"), rp, ci, v, 1, 4)
     # bcsr output is padded to an even number of rows
     xo = torch.zeros(7, 16, device="cuda")
     rpb = torch.zeros(5, dtype=torch.int32, device="cuda")
     assert ParamSpMM.bcsr_spmm(xo, rpb, ci, torch.zeros(0, 2, device="cuda"), 1, 4).shape == (8, 16)
+
+
+@pytest.mark.parametrize("N", [16, 33, 130, 256, 1030])
+def test_row_caching_baseline_matches_oracle(oracle, N):
+    """gespmm_compute: the comparison baseline (one wavefront per row, entries cached in LDS) computes the same
+    product; a hub row longer than the cache and empty rows included."""
+    import ParamSpMM
+    from gpu_util import assert_close
+
+    rowPtr, colIdx, val = random_csr(1501, 7.0, seed=N, empty_frac=0.2, hub=(5, 1300))
+    X = np.random.default_rng(N).standard_normal((1501, N)).astype(np.float32)
+    want = oracle.spmm_csr(rowPtr, colIdx, val, X)
+    scale = oracle.spmm_csr(rowPtr, colIdx, np.abs(val), np.abs(X))
+    got = ParamSpMM.gespmm_compute(torch.from_numpy(X).cuda(), torch.from_numpy(rowPtr).cuda(),
+                                   torch.from_numpy(colIdx).cuda(), torch.from_numpy(val).cuda())
+    assert_close(got, want, what="row-caching baseline N=%d" % N, scale=scale)
+    if N == 16:
+        assert ParamSpMM.gespmm_profile(torch.from_numpy(X).cuda(), torch.from_numpy(rowPtr).cuda(),
+                                        torch.from_numpy(colIdx).cuda(), torch.from_numpy(val).cuda()) > 0
 
 
 def test_spconv_forward_backward(oracle):
