@@ -115,10 +115,11 @@ class pcsr_spmm(object):
         else:
             self.mtx_nodes, self.mtx_edges = graph.mtx_nodes, graph.mtx_edges
             fmt = graph.csr_data if vec_size == 1 else graph.bcsr_data
-            self.rowPtr = (fmt.rowPtr_split if if_split else fmt.rowPtr).to(device)
-            self.colIdx = fmt.colIdx.to(device)
-            self.val = fmt.val.to(device)
-            self.target_row = fmt.target_row.to(device) if if_split else None
+            # one device copy per format, shared by every operator built on this graph
+            self.rowPtr = fmt.on_device("rowPtr_split" if if_split else "rowPtr", device)
+            self.colIdx = fmt.on_device("colIdx", device)
+            self.val = fmt.on_device("val", device)
+            self.target_row = fmt.on_device("target_row", device) if if_split else None
             if vec_size != 1 and getattr(graph, "mask", None) is not None:
                 self.mask = graph.mask.to(device)
         self.vec_size = vec_size

@@ -76,6 +76,26 @@ class csr_data(object):
         self.row_split_nnz = None
         self.rowPtr_split = None
         self.target_row = None
+        self._dev = {}  # (attribute name, device) -> copy of that attribute on the device
+
+    def on_device(self, name, device):
+        """The attribute ``name`` as a tensor on ``device``; uploaded once and kept (the device builders leave
+        their outputs here, so a format built on the GPU is never uploaded again)."""
+        device = torch.device(device)
+        if device.type != "cuda":
+            return getattr(self, name).to(device)
+        if device.index is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        key = (name, device)
+        host = getattr(self, name)
+        t = self._dev.get(key)
+        if t is None or t.shape != host.shape:
+            t = host.to(device)
+            self._dev[key] = t
+        return t
+
+    def _keep_device(self, name, tensor):
+        self._dev[(name, tensor.device)] = tensor
 
     # graph_input.py:48-51
     def split_ratio_comp(self, split_granularity):
@@ -115,8 +135,10 @@ class csr_data(object):
         if _use_device(build_on):
             from . import device_builder
 
-            rs, tr = device_builder.split_csr_device(self.rowPtr.cuda(), self.split_granularity)
+            rs, tr = device_builder.split_csr_device(self.on_device("rowPtr", "cuda"), self.split_granularity)
             self.rowPtr_split, self.target_row = rs.cpu(), tr.cpu()
+            self._keep_device("rowPtr_split", rs)
+            self._keep_device("target_row", tr)
         else:
             import ParamSpMM  # the extension module of this build (lib/ParamSpMM.so)
 
@@ -159,9 +181,10 @@ def _use_device(build_on):
     return build_on == "device" or (build_on == "auto" and torch.cuda.is_available())
 
 
-def build_bcsr(rowPtr, colIdx, val, ncols=None, build_on="host"):
+def build_bcsr(rowPtr, colIdx, val, ncols=None, build_on="host", device_arrays=None):
     """CSR (numpy int32/int32/fp32) -> 2x1 BCSR arrays (numpy) via libparamsp_hip.so: the host builder, or the
-    device builder when ``build_on`` says so and the rows are strictly ascending."""
+    device builder when ``build_on`` says so and the rows are strictly ascending.  ``device_arrays``: the CSR
+    already on the GPU (rowPtr, colIdx, val) to build from; on return it holds the three BCSR tensors on the GPU."""
     rowPtr = np.ascontiguousarray(rowPtr, np.int32)
     colIdx = np.ascontiguousarray(colIdx, np.int32)
     val = np.ascontiguousarray(val, np.float32)
@@ -170,13 +193,16 @@ def build_bcsr(rowPtr, colIdx, val, ncols=None, build_on="host"):
         from . import device_builder
 
         try:
-            out = device_builder.build_bcsr_device(
-                torch.from_numpy(rowPtr).cuda(), torch.from_numpy(colIdx).cuda(), torch.from_numpy(val).cuda()
-            )
+            src = device_arrays if device_arrays else [torch.from_numpy(a).cuda() for a in (rowPtr, colIdx, val)]
+            out = device_builder.build_bcsr_device(*src)
+            if device_arrays is not None:
+                device_arrays[:] = out
             return tuple(t.cpu().numpy() for t in out)
         except device_builder.NotCanonical:
             if build_on == "device":
                 raise
+    if device_arrays is not None:
+        del device_arrays[:]
     ncols = n + (n & 1) if ncols is None else ncols
     nblk = _capi.check(_capi.lib.psp_bcsr_count(_capi.ptr(rowPtr), _capi.ptr(colIdx), n, ncols))
     rowPtr_b = np.empty((n + 1) // 2 + 1, np.int32)
@@ -259,10 +285,15 @@ class graph_input(object):
         self.csr_data = csr_data(rowPtr, colIdx, val, n, nnz, True)
         self.csr_data.init_info(is_avg_granularity=is_avg_granularity, manual_granularity=manual_granularity)
 
-        rowPtr_b, colIdx_b, val_b = build_bcsr(rowPtr, colIdx, val, build_on=build_on)
+        on_gpu = []
+        if _use_device(build_on):
+            on_gpu = [self.csr_data.on_device(k, "cuda") for k in ("rowPtr", "colIdx", "val")]
+        rowPtr_b, colIdx_b, val_b = build_bcsr(rowPtr, colIdx, val, build_on=build_on, device_arrays=on_gpu)
         nblk = colIdx_b.size
         # graph_input.py:257-266: the blocked format counts block-rows and blocks (the latter as a float)
         self.bcsr_data = csr_data(rowPtr_b, colIdx_b, val_b, (n + 1) // 2, float(nblk), False)
+        for k, t in zip(("rowPtr", "colIdx", "val"), on_gpu):
+            self.bcsr_data._keep_device(k, t)
         self.bcsr_data.init_info(is_avg_granularity=is_avg_granularity, manual_granularity=manual_granularity)
         self.pack_rate = nnz / (2 * nblk) if nblk else 0.0
 
@@ -274,7 +305,8 @@ class graph_input(object):
                 raise RuntimeError("if_mask=True runs genmask on the GPU and no GPU is available")
             dev = torch.device("cuda")
             mask = ParamSDDMM.genmask(
-                self.bcsr_data.rowPtr.to(dev), self.csr_data.rowPtr.to(dev), self.bcsr_data.val.to(dev), self.mtx_edges
+                self.bcsr_data.on_device("rowPtr", dev), self.csr_data.on_device("rowPtr", dev),
+                self.bcsr_data.on_device("val", dev), self.mtx_edges
             )
             self.mask = mask.to(torch.int64)
 

@@ -9,8 +9,8 @@ SuiteSparse / OGB collection the reference downloads.
                 every <representation, CF, blkWarpNum> at every width 16..256 -> csv files with the reference's
                 schema: mtx_info.csv, dim<N>.csv (GFLOP/s per column), dim<N>_OP_SpMM.csv (features + arg-max
                 column = class code).
-  fit    (CPU)  80/20 split, one RandomForestClassifier per width -> rnd_tree_<N>.pkl, and a report with the
-                reference's two statistics (test accuracy, mean normalised performance) plus the share of test
+  fit    (CPU)  one RandomForestClassifier per width -> rnd_tree_<N>.pkl, and a 5-fold cross-validated report with
+                the reference's two statistics (accuracy, mean normalised performance) plus the share of
                 matrices whose pick is within 10 % of the best swept configuration.
 
     python -m paramspmm_ae_amd.train_decider sweep --out gpurun_out/decider [--part 0/3]
@@ -213,17 +213,31 @@ def load_training_data(data_dir):
     return info, {d: pd.concat(tps[d], ignore_index=True) for d in DIMS}
 
 
+def _fit_forest(X, TP, near, n_est):
+    """Forest on 'near-best' labels: a matrix contributes one sample for every configuration whose throughput is at
+    least ``near`` times its best one, the samples of a matrix sharing a total weight of 1.  near = 1 is the
+    reference's arg-max label (PCSR.py:815-818); a threshold below 1 keeps timing noise between configurations
+    that are equally good from turning into label noise."""
+    from sklearn.ensemble import RandomForestClassifier
+
+    ok = TP >= near * TP.max(axis=1, keepdims=True)
+    rows, cols = np.nonzero(ok)
+    weight = 1.0 / ok.sum(axis=1)[rows]
+    clf = RandomForestClassifier(n_estimators=n_est, n_jobs=-1, random_state=17)
+    clf.fit(X[rows], cols, sample_weight=weight)
+    return clf
+
+
 def fit_main(args):
     import pandas as pd
-    from sklearn.ensemble import RandomForestClassifier
-    from sklearn.model_selection import train_test_split
+    from sklearn.model_selection import KFold
 
     info, tps = load_training_data(args.data)
     X = info[FEATURES].to_numpy(dtype=np.float64)
     os.makedirs(args.out, exist_ok=True)
-    report = {"matrices": int(len(info)), "per_dim": {}}
-    idx = np.arange(len(info))
-    tr, te = train_test_split(idx, test_size=0.2, random_state=17)
+    report = {"matrices": int(len(info)), "validation": "5-fold cross-validation: every matrix is predicted by a forest "
+              "that has not seen it", "per_dim": {}}
+    folds = list(KFold(5, shuffle=True, random_state=17).split(X))
     for d in DIMS:
         TP = tps[d].to_numpy(dtype=np.float64)
         y = TP.argmax(axis=1)  # class code = column index (PCSR.py:815-818)
@@ -231,27 +245,29 @@ def fit_main(args):
         lab = pd.concat([info, pd.DataFrame({"OP_SpMM": y})], axis=1)
         lab.to_csv(os.path.join(args.data, "dim%d_OP_SpMM.csv" % d), index=False)
         best = None
-        for n_est in (20, 30, 50, 80):  # the notebook uses 30 / 50 / 80; a larger forest must earn its size
-            clf = RandomForestClassifier(n_estimators=n_est, n_jobs=-1, random_state=17)
-            clf.fit(X[tr], y[tr])
-            pick = clf.predict(X[te])
-            norm = TP[te, pick] / TP[te].max(axis=1)  # normalised performance of the pick
-            score = (float(np.mean(norm >= 1 / 1.10)), float(norm.mean()))
-            if best is None or score[0] > best[0][0] + 1e-9:
-                best = (score, n_est, clf, pick, norm)
-        (within10, mean_norm), n_est, clf, pick, norm = best
+        for near in (1.0, 0.97, 0.95):
+            for n_est in (30, 50, 80):  # the sizes the reference's notebook uses
+                pick = np.zeros(len(X), dtype=np.int64)
+                for tr, te in folds:
+                    pick[te] = _fit_forest(X[tr], TP[tr], near, n_est).predict(X[te]).astype(np.int64)
+                norm = TP[np.arange(len(X)), pick] / TP.max(axis=1)  # normalised performance of the pick
+                score = (float(np.mean(norm >= 1 / 1.10)), float(norm.mean()))
+                if best is None or score > best[0]:
+                    best = (score, near, n_est, pick, norm)
+        (within10, mean_norm), near, n_est, pick, norm = best
         report["per_dim"][d] = {
-            "n_estimators": n_est, "classes": int(TP.shape[1]), "test_matrices": int(len(te)),
-            "test_accuracy": float(np.mean(pick == y[te])), "mean_normalised_performance": mean_norm,
-            "share_within_10pct_of_best": within10, "worst_normalised_performance": float(norm.min()),
+            "near_best_threshold": near, "n_estimators": n_est, "classes": int(TP.shape[1]),
+            "validated_matrices": int(len(X)), "accuracy": float(np.mean(pick == y)),
+            "mean_normalised_performance": mean_norm, "share_within_10pct_of_best": within10,
+            "worst_normalised_performance": float(norm.min()),
         }
         # the shipped model is refitted on every matrix
-        final = RandomForestClassifier(n_estimators=n_est, n_jobs=-1, random_state=17).fit(X, y)
+        final = _fit_forest(X, TP, near, n_est)
         final.n_jobs = 1
         with open(os.path.join(args.out, "rnd_tree_%d.pkl" % d), "wb") as f:
             pickle.dump(final, f)
-        print("dim %3d: %2d classes  n_estimators %d  test acc %.3f  mean norm perf %.4f  within 10%%: %.3f  worst %.3f" % (
-            d, TP.shape[1], n_est, report["per_dim"][d]["test_accuracy"], mean_norm, within10, norm.min()), flush=True)
+        print("dim %3d: %2d classes  near %.2f  n_estimators %d  acc %.3f  mean norm perf %.4f  within 10%%: %.3f  worst %.3f" % (
+            d, TP.shape[1], near, n_est, report["per_dim"][d]["accuracy"], mean_norm, within10, norm.min()), flush=True)
     allw = [v["share_within_10pct_of_best"] for v in report["per_dim"].values()]
     report["share_within_10pct_mean"] = float(np.mean(allw))
     report["share_within_10pct_min"] = float(np.min(allw))
