@@ -172,6 +172,11 @@ int psp_sddmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b, const fl
  * the SDDMM -> softmax -> SpMM attention pipeline.  in and out may alias.
  * ------------------------------------------------------------------------------------------- */
 int psp_segment_softmax_f32(const int *rowPtr, const float *in, float *out, int M, psp_stream_t stream);
+/* Same result with the work of rows longer than 128 entries spread over the whole GPU (four launches instead of
+ * one; a hub row otherwise runs on a single workgroup).  nnz = rowPtr[M]; workspace: 2*M floats of device memory,
+ * contents irrelevant on entry.  The sum of a long row is accumulated with fp32 atomics. */
+int psp_segment_softmax_ws_f32(const int *rowPtr, const float *in, float *out, int M, int nnz, float *workspace,
+                               psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: C[K1,K2] = A^T * B for tall-skinny row-major A [n,K1] and B [n,K2]; C is overwritten.

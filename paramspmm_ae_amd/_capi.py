@@ -60,6 +60,7 @@ SIGNATURES = {
     "psp_sddmm_bcsr_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "psp_sddmm_bcsr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "psp_segment_softmax_f32": [_vp, _vp, _vp, _i, _vp],
+    "psp_segment_softmax_ws_f32": [_vp, _vp, _vp, _i, _i, _vp, _vp],
     "psp_baseline_rowcache_spmm_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
     "psp_gemm_atb_supported": [_i, _i],
     "psp_gemm_atb_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _vp],

@@ -170,11 +170,19 @@ PSP_EXPORT int psp_genmask(const int *rowPtr_b, const int *rowPtr, const float *
 }
 
 // ------------------------------------------------------------------------------------------------
-// segment softmax.  Phase 1: 16 lanes per row, three sweeps over the row (max, sum, write); rows of up to 16
-// entries never re-read memory.  Rows longer than PSP_SOFTMAX_LONG entries are left to phase 2, where the whole
-// workgroup (256 lanes) takes them one at a time, so a hub row does not serialise on 16 lanes.
+// segment softmax.  Short rows: 16 lanes per row, three sweeps over the row (max, sum, write); rows of up to 64
+// entries never re-read memory.  Rows longer than PSP_SOFTMAX_LONG (128) entries are handled in one of two ways:
+//   * without workspace (psp_segment_softmax_f32): the workgroup that met the row takes it with all 256 lanes;
+//     a hub row of 10^5 entries then runs on one workgroup -- correct, but it becomes the tail of the launch;
+//   * with workspace (psp_segment_softmax_ws_f32): the short-row kernel only resets the row's (max, sum) pair in
+//     the workspace; three further launches walk the entry array in chunks of PSP_SOFTMAX_CHUNK entries, every
+//     workgroup finding the long rows that cross its chunk and, one wavefront per row, contributing to their max
+//     (atomic max), their sum (atomic add) and finally writing its part of the result -- a hub row spreads over
+//     the whole GPU and rows of a few hundred entries no longer crawl along on 16 lanes.
 // ------------------------------------------------------------------------------------------------
-#define PSP_SOFTMAX_LONG 1024
+#define PSP_SOFTMAX_LONG 128
+#define PSP_SOFTMAX_CHUNK 4096
+#define PSP_SOFTMAX_NEG (-3.402823466e+38f)
 
 __device__ __forceinline__ float psp_max16(float v)
 {
@@ -185,13 +193,37 @@ __device__ __forceinline__ float psp_max16(float v)
     return v;
 }
 
-__global__ void __launch_bounds__(256)
-psp_segment_softmax_kernel(const int *__restrict__ rowPtr, const float *in, float *out, int M)
+// 256-lane reductions through LDS (4 wavefronts); every lane of the workgroup must call them
+__device__ __forceinline__ float psp_block_max(float v, float *s_red)
 {
-    __shared__ int s_long[16];    // rows of this workgroup left to phase 2
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) v = fmaxf(v, __shfl_xor(v, d));
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
+    __syncthreads();
+    return v;
+}
+__device__ __forceinline__ float psp_block_sum(float v, float *s_red)
+{
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) v += __shfl_xor(v, d);
+    if ((threadIdx.x & 63) == 0) s_red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    v = s_red[0] + s_red[1] + s_red[2] + s_red[3];
+    __syncthreads();
+    return v;
+}
+
+// WS: long rows are left to the chunk kernels, only their workspace pair is reset here
+template <bool WS>
+__global__ void __launch_bounds__(256)
+psp_segment_softmax_kernel(const int *__restrict__ rowPtr, const float *in, float *out, int M, float *__restrict__ ws)
+{
+    __shared__ int s_long[16];    // rows of this workgroup left to the long-row loop
     __shared__ int s_nlong;
     __shared__ float s_red[4];    // one slot per wavefront
-    const float NEG = -3.402823466e+38f;
+    const float NEG = PSP_SOFTMAX_NEG;
     if (threadIdx.x == 0) s_nlong = 0;
     __syncthreads();
 
@@ -203,45 +235,118 @@ psp_segment_softmax_kernel(const int *__restrict__ rowPtr, const float *in, floa
         hb = rowPtr[row + 1];
     }
     if (hb - lb > PSP_SOFTMAX_LONG) {
-        if (sub == 0) s_long[atomicAdd(&s_nlong, 1)] = row;
+        if (WS) {
+            if (sub == 0) {
+                ws[2 * (size_t)row] = NEG;
+                ws[2 * (size_t)row + 1] = 0.0f;
+            }
+        } else if (sub == 0) {
+            s_long[atomicAdd(&s_nlong, 1)] = row;
+        }
     } else if (lb < hb) {  // a 16-lane group is uniform here
-        const float first = (lb + sub < hb) ? in[lb + sub] : NEG;
-        float mx = first;
-        for (int p = lb + 16 + sub; p < hb; p += 16) mx = fmaxf(mx, in[p]);
+        // the first 64 entries of the row stay in registers (four independent loads per lane): rows up to that
+        // length are read once; longer ones sweep the rest three times
+        float v[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int p = lb + sub + 16 * j;
+            v[j] = p < hb ? in[p] : NEG;
+        }
+        float mx = fmaxf(fmaxf(v[0], v[1]), fmaxf(v[2], v[3]));
+        for (int p = lb + 64 + sub; p < hb; p += 16) mx = fmaxf(mx, in[p]);
         mx = psp_max16(mx);
-        float s = (lb + sub < hb) ? __expf(first - mx) : 0.0f;
-        for (int p = lb + 16 + sub; p < hb; p += 16) s += __expf(in[p] - mx);
+        float ex[4], s = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            ex[j] = __expf(v[j] - mx);  // exactly 0 for the padding value
+            s += ex[j];
+        }
+        for (int p = lb + 64 + sub; p < hb; p += 16) s += __expf(in[p] - mx);
         s = psp_group_sum<4>(s);
         const float inv = 1.0f / s;
-        // all reads of a chunk happen before its writes, so in == out is fine
-        const float e0 = __expf(first - mx) * inv;
-        for (int p = lb + 16 + sub; p < hb; p += 16) out[p] = __expf(in[p] - mx) * inv;
-        if (lb + sub < hb) out[lb + sub] = e0;
+        // every entry is read and written by the same lane, reads first, so in == out is fine
+        for (int p = lb + 64 + sub; p < hb; p += 16) out[p] = __expf(in[p] - mx) * inv;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int p = lb + sub + 16 * j;
+            if (p < hb) out[p] = ex[j] * inv;
+        }
     }
+    if (WS) return;
     __syncthreads();
 
     const int nlong = s_nlong;  // workgroup-uniform
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     for (int i = 0; i < nlong; i++) {
         const int r = s_long[i];
         const int a = rowPtr[r], b = rowPtr[r + 1];
         float mx = NEG;
         for (int p = a + threadIdx.x; p < b; p += 256) mx = fmaxf(mx, in[p]);
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
-        if (lane == 0) s_red[wave] = mx;
-        __syncthreads();
-        mx = fmaxf(fmaxf(s_red[0], s_red[1]), fmaxf(s_red[2], s_red[3]));
-        __syncthreads();
+        mx = psp_block_max(mx, s_red);
         float s = 0.0f;
         for (int p = a + threadIdx.x; p < b; p += 256) s += __expf(in[p] - mx);
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) s += __shfl_xor(s, d);
-        if (lane == 0) s_red[wave] = s;
-        __syncthreads();
-        const float inv = 1.0f / (s_red[0] + s_red[1] + s_red[2] + s_red[3]);
-        __syncthreads();
+        const float inv = 1.0f / psp_block_sum(s, s_red);
         for (int p = a + threadIdx.x; p < b; p += 256) out[p] = __expf(in[p] - mx) * inv;
+    }
+}
+
+// float maximum through the integer atomics: the order of non-negative floats is that of their bit patterns
+// read as signed integers, the order of negative floats is the reverse of their patterns read as unsigned
+__device__ __forceinline__ void psp_atomic_max_f32(float *addr, float v)
+{
+    if (v >= 0.0f) atomicMax((int *)addr, __float_as_int(v));
+    else atomicMin((unsigned int *)addr, __float_as_uint(v));
+}
+
+// PASS 0: row maxima, 1: sums of exp(x - max), 2: results.  One workgroup per chunk of the entry array.
+template <int PASS>
+__global__ void __launch_bounds__(256)
+psp_softmax_long_kernel(const int *__restrict__ rowPtr, const float *in, float *out, int M, int nnz, float *ws)
+{
+    __shared__ int s_rows[PSP_SOFTMAX_CHUNK / PSP_SOFTMAX_LONG + 4];  // long rows that cross this chunk
+    __shared__ int s_n;
+    const int c0 = blockIdx.x * PSP_SOFTMAX_CHUNK;
+    const int c1 = min(nnz, c0 + PSP_SOFTMAX_CHUNK);
+    if (threadIdx.x == 0) s_n = 0;
+    __syncthreads();
+    // rows that hold entries of [c0, c1): from the first row ending after c0 to the last row starting before c1
+    int lo = 0, hi = M;
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (rowPtr[mid + 1] > c0) hi = mid; else lo = mid + 1;
+    }
+    const int r_first = lo;
+    hi = M;
+    while (lo < hi) {
+        const int mid = (lo + hi) >> 1;
+        if (rowPtr[mid] >= c1) hi = mid; else lo = mid + 1;
+    }
+    const int r_end = lo;  // first row starting at or after c1
+    for (int r = r_first + threadIdx.x; r < r_end; r += 256)
+        if (rowPtr[r + 1] - rowPtr[r] > PSP_SOFTMAX_LONG) s_rows[atomicAdd(&s_n, 1)] = r;
+    __syncthreads();
+    const int n = s_n;  // workgroup-uniform, at most CHUNK/LONG + 2
+    // one wavefront per (row, chunk) intersection
+    const int lane = threadIdx.x & 63;
+    for (int i = threadIdx.x >> 6; i < n; i += 4) {
+        const int r = s_rows[i];
+        const int a = max(rowPtr[r], c0), b = min(rowPtr[r + 1], c1);
+        if (PASS == 0) {
+            float mx = PSP_SOFTMAX_NEG;
+            for (int p = a + lane; p < b; p += 64) mx = fmaxf(mx, in[p]);
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+            if (lane == 0) psp_atomic_max_f32(ws + 2 * (size_t)r, mx);
+        } else if (PASS == 1) {
+            const float mx = ws[2 * (size_t)r];
+            float s = 0.0f;
+            for (int p = a + lane; p < b; p += 64) s += __expf(in[p] - mx);
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) s += __shfl_xor(s, d);
+            if (lane == 0) atomicAdd(ws + 2 * (size_t)r + 1, s);
+        } else {
+            const float mx = ws[2 * (size_t)r], inv = 1.0f / ws[2 * (size_t)r + 1];
+            for (int p = a + lane; p < b; p += 64) out[p] = __expf(in[p] - mx) * inv;
+        }
     }
 }
 
@@ -250,9 +355,25 @@ PSP_EXPORT int psp_segment_softmax_f32(const int *rowPtr, const float *in, float
     PSP_REQUIRE(M >= 0, "segment_softmax: negative row count");
     if (M == 0) return PSP_OK;
     PSP_REQUIRE(rowPtr && in && out, "segment_softmax: null pointer");
-    hipLaunchKernelGGL(psp_segment_softmax_kernel, dim3(psp_ceil_div((long long)M * 16, 256)), dim3(256), 0,
-                       (hipStream_t)stream, rowPtr, in, out, M);
+    hipLaunchKernelGGL(psp_segment_softmax_kernel<false>, dim3(psp_ceil_div((long long)M * 16, 256)), dim3(256), 0,
+                       (hipStream_t)stream, rowPtr, in, out, M, (float *)nullptr);
     return psp_check_launch("segment softmax kernel");
+}
+
+PSP_EXPORT int psp_segment_softmax_ws_f32(const int *rowPtr, const float *in, float *out, int M, int nnz,
+                                          float *workspace, psp_stream_t stream)
+{
+    PSP_REQUIRE(M >= 0 && nnz >= 0, "segment_softmax_ws: negative size");
+    if (M == 0 || nnz == 0) return PSP_OK;
+    PSP_REQUIRE(rowPtr && in && out && workspace, "segment_softmax_ws: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(psp_segment_softmax_kernel<true>, dim3(psp_ceil_div((long long)M * 16, 256)), dim3(256), 0, st,
+                       rowPtr, in, out, M, workspace);
+    const dim3 grid(psp_ceil_div(nnz, PSP_SOFTMAX_CHUNK));
+    hipLaunchKernelGGL(psp_softmax_long_kernel<0>, grid, dim3(256), 0, st, rowPtr, in, out, M, nnz, workspace);
+    hipLaunchKernelGGL(psp_softmax_long_kernel<1>, grid, dim3(256), 0, st, rowPtr, in, out, M, nnz, workspace);
+    hipLaunchKernelGGL(psp_softmax_long_kernel<2>, grid, dim3(256), 0, st, rowPtr, in, out, M, nnz, workspace);
+    return psp_check_launch("segment softmax kernels");
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -161,8 +161,12 @@ static Tensor segment_softmax(Tensor rowPtr, Tensor e)
     same_device(rowPtr, e, "segment_softmax");
     check_rowptr_vs(rowPtr, "rowPtr");
     pspglue::DeviceGuard guard(e.device());
+    TORCH_CHECK(e.numel() <= 0x7fffffffLL, "segment_softmax: more than 2^31-1 entries");
     auto out = torch::empty_like(e);
-    ok(psp_segment_softmax_f32(ip(rowPtr), fp(e), fpw(out), (int)rowPtr.size(0) - 1, stream_of(e)));
+    // the (max, sum) pairs of rows long enough to be spread over several workgroups
+    auto ws = torch::empty({2 * (rowPtr.size(0) - 1)}, e.options());
+    ok(psp_segment_softmax_ws_f32(ip(rowPtr), fp(e), fpw(out), (int)rowPtr.size(0) - 1, (int)e.numel(), fpw(ws),
+                                  stream_of(e)));
     return out;
 }
 

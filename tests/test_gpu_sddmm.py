@@ -98,7 +98,7 @@ def test_segment_softmax_parity(oracle, small):
 
 
 def test_segment_softmax_long_rows(oracle):
-    """Rows above 1024 entries are handled by a whole workgroup; several in one workgroup's 16 rows, plus empty rows."""
+    """Rows above the long-row threshold (128 entries) are handled by a whole workgroup; several in one workgroup's 16 rows, plus empty rows."""
     from paramspmm_ae_amd import _capi
     from gpu_util import stream, assert_close
 
@@ -115,3 +115,37 @@ def test_segment_softmax_long_rows(oracle):
     assert_close(out, oracle.segment_softmax(rowPtr, e), rtol=1e-5, atol=1e-6, what="softmax long rows")
     _capi.check(_capi.lib.psp_segment_softmax_f32(p(rp), p(ed), p(ed), rowPtr.size - 1, stream()))
     assert_close(ed, out.cpu().numpy(), rtol=0, atol=0, what="softmax long rows in place")
+
+
+@pytest.mark.parametrize("all_negative", [False, True])
+def test_segment_softmax_with_workspace_spreads_long_rows(oracle, all_negative):
+    """The workspace variant hands rows above 128 entries to chunk-wise launches (atomic max, atomic sum): rows
+    that cross chunk boundaries, a row of several chunks, long rows next to each other, the last row long, empty
+    rows, and inputs that are all negative (the float maximum goes through integer atomics)."""
+    from paramspmm_ae_amd import _capi
+    from gpu_util import stream, assert_close
+
+    rowPtr, colIdx, val = random_csr(6000, 6, 7, empty_frac=0.3, hub=(17, 5500))
+    k = np.diff(rowPtr).copy()
+    k[18], k[19], k[21], k[3000], k[5999] = 1500, 1025, 20000, 4096, 2049
+    k[100:140] = 129  # forty rows just above the threshold in a row: more than one list entry per wavefront
+    rowPtr = np.concatenate([[0], np.cumsum(k)]).astype(np.int32)
+    nnz = int(rowPtr[-1])
+    e = (np.random.default_rng(3).standard_normal(nnz) * 5).astype(np.float32)
+    if all_negative:
+        e = -np.abs(e) - 1.0
+    ed = torch.from_numpy(e).cuda()
+    rp = torch.from_numpy(rowPtr).cuda()
+    out = torch.full_like(ed, float("nan"))
+    ws = torch.full((2 * (rowPtr.size - 1),), float("nan"), device="cuda")  # contents must not matter
+    p = _capi.ptr
+    want = oracle.segment_softmax(rowPtr, e)
+    _capi.check(_capi.lib.psp_segment_softmax_ws_f32(p(rp), p(ed), p(out), rowPtr.size - 1, nnz, p(ws), stream()))
+    assert_close(out, want, rtol=1e-5, atol=1e-6, what="softmax with workspace")
+    # a second call on the used workspace, in place
+    _capi.check(_capi.lib.psp_segment_softmax_ws_f32(p(rp), p(ed), p(ed), rowPtr.size - 1, nnz, p(ws), stream()))
+    assert_close(ed, want, rtol=1e-5, atol=1e-6, what="softmax with workspace, in place")
+    # through the module
+    import ParamSDDMM
+    got = ParamSDDMM.segment_softmax(rp, torch.from_numpy(e).cuda())
+    assert_close(got, want, rtol=1e-5, atol=1e-6, what="ParamSDDMM.segment_softmax")
