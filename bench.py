@@ -146,10 +146,14 @@ def bench_gcn(args):
     graphs = [args.graph] if args.graph in ("C5", "C5p", "C1") else ["C5", "C5p"]
     for g in graphs:
         for net in ("GCN", "GIN"):
-            res = GNN.main(["--net", net, "--synthetic", g, "--hidden_list", "16", "32", "128", "--num_classes", "16",
-                            "--num_features", "32", "--num_epoches", str(args.steps)])
+            argv = ["--net", net, "--synthetic", g, "--hidden_list", "16", "32", "128", "--num_classes", "16",
+                    "--num_features", "32", "--num_epoches", str(args.steps)]
+            res = GNN.main(argv)
+            # the same epochs with the training step recorded once in a HIP graph and replayed
+            res_graph = GNN.main(argv + ["--hip_graph"])
             for (name, hidden), ms in res.items():
-                out["epochs"].append({"graph": name, "net": net, "hidden": hidden, "ms_per_epoch": round(ms, 3)})
+                out["epochs"].append({"graph": name, "net": net, "hidden": hidden, "ms_per_epoch": round(ms, 3),
+                                      "ms_per_epoch_hip_graph": round(res_graph[(name, hidden)], 3)})
     out["value"] = out["epochs"][0]["ms_per_epoch"]
     out["ms_per_step"] = out["value"]
     print(json.dumps(out))
