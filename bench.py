@@ -134,6 +134,76 @@ def bench_agnn(args):
     print(json.dumps(out))
 
 
+def bench_sddmm(args):
+    """SDDMM out[p] = <A[row(p)], B[col(p)]> over the stored pattern (reference semantics: unscaled), widths
+    K = 16..128, all four formats at both workgroup sizes; the best per width is reported with its algorithmic
+    bytes (row pointers + column indices + A + B + the output) against the HBM peak, next to rocSPARSE's SDDMM."""
+    import torch
+
+    import paramspmm_ae_amd  # noqa: F401
+    import ParamSDDMM
+    from paramspmm_ae_amd import synth
+    from paramspmm_ae_amd.graph_input import graph_input
+
+    rowPtr, colIdx, val, n = synth.config_graph(args.graph)
+    nnz = colIdx.size
+    g = graph_input(args.graph, "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val)
+    c, b = g.csr_data, g.bcsr_data
+    dev = "cuda"
+    C = {k: c.on_device(k, dev) for k in ("rowPtr", "colIdx", "val", "rowPtr_split", "target_row")}
+    Bf = {k: b.on_device(k, dev) for k in ("rowPtr", "colIdx", "val", "rowPtr_split", "target_row")}
+    nblk = Bf["colIdx"].numel()
+    rows = (n + 1) // 2 * 2
+    gen = torch.Generator(device="cuda").manual_seed(7)
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    per_K = []
+    for K in (16, 32, 64, 128):
+        A = torch.randn(rows, K, device=dev, generator=gen)
+        Bm = torch.randn(rows, K, device=dev, generator=gen)
+        cands = {}
+        for bw in (4, 8):
+            cands[("csr", bw)] = lambda bw=bw: ParamSDDMM.csr_sddmm(A, Bm, C["rowPtr"], C["colIdx"], C["val"], 1, bw)
+            cands[("csr_split", bw)] = lambda bw=bw: ParamSDDMM.csr_split_sddmm(A, Bm, C["rowPtr_split"], C["colIdx"], C["val"], C["target_row"], 1, bw)
+            cands[("bcsr", bw)] = lambda bw=bw: ParamSDDMM.bcsr_sddmm(A, Bm, Bf["rowPtr"], Bf["colIdx"], Bf["val"], 1, bw)
+            cands[("bcsr_split", bw)] = lambda bw=bw: ParamSDDMM.bcsr_split_sddmm(A, Bm, Bf["rowPtr_split"], Bf["colIdx"], Bf["val"], Bf["target_row"], 1, bw)
+        times = {k: timed(f) for k, f in cands.items()}
+        (fmt, bw), ms = min(times.items(), key=lambda kv: kv[1])
+        if fmt.startswith("bcsr"):
+            alg = 4 * (Bf["rowPtr_split" if "split" in fmt else "rowPtr"].numel()) + 12 * nblk + 8 * n * K + 8 * nblk
+        else:
+            alg = 4 * (C["rowPtr_split" if "split" in fmt else "rowPtr"].numel()) + 4 * nnz + 8 * n * K + 4 * nnz
+        if "split" in fmt:
+            alg += 4 * (Bf if fmt.startswith("bcsr") else C)["target_row"].numel()
+        vals = C["val"].clone()
+        vendor_ms = timed(lambda: ParamSDDMM.cusparse_sddmm_compute(A[:n].contiguous() if rows != n else A,
+                                                                    Bm[:n].contiguous() if rows != n else Bm,
+                                                                    C["rowPtr"], C["colIdx"], vals)) if not args.no_vendor else None
+        per_K.append({"K": K, "format": fmt, "blkWarpNum": bw, "ms": round(ms, 5), "gflops": round(2.0 * nnz * K / ms / 1e6, 1),
+                      "alg_bytes": int(alg), "alg_GBps": round(alg / ms / 1e6, 1), "frac_hbm": round(alg / ms / 1e6 / HBM_PEAK_GBS, 4),
+                      "all_ms": {"%s/%d" % k: round(v, 5) for k, v in times.items()},
+                      "rocsparse_ms": None if vendor_ms is None else round(vendor_ms, 5)})
+    total_ms = sum(r["ms"] for r in per_K)
+    value = sum(2.0 * nnz * r["K"] for r in per_K) / total_ms / 1e6
+    print(json.dumps({"metric": "SDDMM GFLOP/s (2*nnz*K) over K = 16..128", "value": round(value, 1), "unit": "GFLOP/s",
+                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(total_ms, 4),
+                      "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": "%s SDDMM width sweep" % args.graph, "nodes": n, "nnz": nnz}, "per_K": per_K}))
+
+
 def bench_gcn(args):
     """GCN and GIN training epochs (BASELINE.json configs[4]): 5 layers, hidden 16 / 32 / 128, 16 classes, random
     features and weights, forward + backward + Adam, on the 1M-node stochastic block model in community order
@@ -225,9 +295,10 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-vendor", action="store_true", help="skip the rocSPARSE comparison leg")
     ap.add_argument("--dump", default=None, help="write the full sweep table (every column, every width) as JSON")
-    ap.add_argument("--workload", choices=["spmm", "agnn", "gcn", "build"], default="spmm",
+    ap.add_argument("--workload", choices=["spmm", "agnn", "gcn", "build", "sddmm"], default="spmm",
                     help="spmm: the headline width sweep; agnn: SDDMM -> row softmax -> SpMM attention layers; "
-                         "gcn: GCN / GIN training epochs on the SBM graph; build: PCSR construction, host against device")
+                         "gcn: GCN / GIN training epochs on the SBM graph; build: PCSR construction, host against device; "
+                         "sddmm: SDDMM width sweep over the four formats")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (no multi-GPU path exists)" % args.gpus,
@@ -245,6 +316,8 @@ def main():
         return bench_gcn(args)
     if args.workload == "build":
         return bench_build(args)
+    if args.workload == "sddmm":
+        return bench_sddmm(args)
     from paramspmm_ae_amd import _capi, synth, sweep
     from paramspmm_ae_amd.graph_input import graph_input
 

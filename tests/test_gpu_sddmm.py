@@ -149,3 +149,38 @@ def test_segment_softmax_with_workspace_spreads_long_rows(oracle, all_negative):
     import ParamSDDMM
     got = ParamSDDMM.segment_softmax(rp, torch.from_numpy(e).cuda())
     assert_close(got, want, rtol=1e-5, atol=1e-6, what="ParamSDDMM.segment_softmax")
+
+
+def test_full_size_headline_graph_properties(oracle):
+    """SDDMM on the benchmark's R-MAT 2^20 pattern: A = B = ones gives K on every stored entry; with A = B the
+    result is symmetric on the symmetric pattern (entry (i,j) equals entry (j,i)); the split format agrees with the
+    plain one bit for bit (every entry is one lane group's own dot product); the blocked result holds the same
+    numbers at the positions the mask names."""
+    from gpu_util import Formats, sddmm_capi
+    from paramspmm_ae_amd import synth, _capi
+
+    rowPtr, colIdx, val, n = synth.config_graph("C2")
+    F = Formats(oracle, rowPtr, colIdx, val)
+    K = 32
+    ones = torch.ones(n, K, device="cuda")
+    assert torch.all(sddmm_capi("csr_split", F, ones, ones, 8) == K)
+    A = torch.randn(n, K, device="cuda", generator=torch.Generator(device="cuda").manual_seed(9))
+    e = sddmm_capi("csr", F, A, A, 4)
+    e_split = sddmm_capi("csr_split", F, A, A, 8)
+    assert torch.equal(e, e_split)
+    # transpose position of every entry: sort (col, row) pairs; the pattern is symmetric, so it is a permutation
+    rows = np.repeat(np.arange(n, dtype=np.int64), np.diff(rowPtr))
+    order = np.lexsort((rows, colIdx.astype(np.int64)))  # entries ordered by (col, row) = transposed CSR order
+    eh = e.cpu().numpy()
+    assert np.array_equal(eh[order], eh), "e(i,j) must equal e(j,i) when A = B"
+    # blocked format through the mask
+    mask = torch.empty(F.nnz, dtype=torch.int32, device="cuda")
+    p = _capi.ptr
+    _capi.check(_capi.lib.psp_genmask(p(F.d["rpb"]), p(F.d["rowPtr"]), p(F.d["vb"]), F.rpb.size - 1, F.nnz, p(mask),
+                                      torch.cuda.current_stream().cuda_stream))
+    eb = sddmm_capi("bcsr", F, A, A, 4).reshape(-1)
+    got = eb[mask.long()].cpu().numpy()
+    # the mask lists a row's entries in block order: compare per row as multisets
+    a_sorted = eh[np.lexsort((eh, rows))]
+    b_sorted = got[np.lexsort((got, rows))]
+    assert np.array_equal(a_sorted, b_sorted)

@@ -182,3 +182,30 @@ def test_spmm_local_matrices_both_block_sizes(oracle, fmt):
             torch.cuda.synchronize()
             assert_close(got8, want, what="%s %s N=%d CF=%d bw=8" % (fmt, name, N, CF), scale=scale)
             assert_close(got4, want, what="%s %s N=%d CF=%d bw=4" % (fmt, name, N, CF), scale=scale)
+
+
+def test_full_size_headline_graph_properties(oracle):
+    """The benchmark's own graph (R-MAT 2^20, 17.9 M entries, hub rows of tens of thousands of entries) at width
+    64: X = ones gives the row sums of A (computed on the host in float64), the four formats agree in every
+    decider-relevant configuration, and A(X1 + X2) = A X1 + A X2."""
+    from gpu_util import Formats, spmm_capi, assert_close
+    from paramspmm_ae_amd import synth
+
+    rowPtr, colIdx, val, n = synth.config_graph("C2")
+    F = Formats(oracle, rowPtr, colIdx, val)
+    rowsum = np.add.reduceat(val.astype(np.float64), rowPtr[:-1].astype(np.int64))
+    rowsum[np.diff(rowPtr) == 0] = 0.0
+    ones = torch.ones(n, 64, device="cuda")
+    for fmt in FMTS:
+        y = spmm_capi(fmt, F, ones, 1, 8)[:n]
+        assert_close(y, np.repeat(rowsum[:, None], 64, axis=1).astype(np.float32), rtol=2e-5, atol=1e-6, what=fmt + " row sums")
+    g = torch.Generator(device="cuda").manual_seed(3)
+    X1 = torch.randn(n, 64, device="cuda", generator=g)
+    X2 = torch.randn(n, 64, device="cuda", generator=g)
+    base = spmm_capi("csr", F, X1, 1, 4)
+    scale = spmm_capi("csr", F, X1.abs(), 1, 4).cpu().numpy()
+    for fmt, CF, bw in (("csr_split", 1, 4), ("csr_split", 2, 8), ("bcsr", 1, 4), ("bcsr_split", 2, 4), ("csr", 2, 8)):
+        assert_close(spmm_capi(fmt, F, X1, CF, bw)[:n], base.cpu().numpy(), what="%s CF=%d bw=%d" % (fmt, CF, bw), scale=scale)
+    lin = spmm_capi("csr_split", F, X1 + X2, 1, 8)
+    both = spmm_capi("csr_split", F, X1, 1, 8) + spmm_capi("csr_split", F, X2, 1, 8)
+    assert_close(lin, both.cpu().numpy(), rtol=1e-4, atol=1e-5, what="linearity at full size")
