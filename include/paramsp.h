@@ -84,7 +84,9 @@ int psp_bcsr_build(const int *rowPtr, const int *colIdx, const float *val, int n
 enum psp_build_flag {
     PSP_BUILD_OVERFLOW = 1,  /* a prefix sum left the int32 range */
     PSP_BUILD_UNSORTED = 2,  /* a row's column indices are not strictly ascending (BCSR builder only) */
-    PSP_BUILD_BAD_ROWPTR = 4 /* rowPtr decreases */
+    PSP_BUILD_BAD_ROWPTR = 4, /* rowPtr decreases, does not start at 0 or does not end at nnz */
+    PSP_BUILD_BAD_COLUMN = 8, /* a column index lies outside [0, ncols)        (psp_check_index_dev only) */
+    PSP_BUILD_BAD_TARGET = 16 /* target_row decreases or leaves [0, target_rows) (psp_check_index_dev only) */
 };
 int psp_scan_workspace_ints(int n);
 
@@ -102,6 +104,14 @@ int psp_bcsr_offsets_dev(const int *rowPtr, const int *colIdx, int nrows, int *r
 /* fills colIdx_b[nblk] and val_b[nblk*2] in the block order of psp_bcsr_build. */
 int psp_bcsr_fill_dev(const int *rowPtr, const int *colIdx, const float *val, int nrows, const int *rowPtr_b,
                       int *colIdx_b, float *val_b, psp_stream_t stream);
+
+/* Validation of index arrays of unknown origin, any of the four formats: rowPtr[M+1] (or rowPtr_split[S+1]) starts at
+ * 0, does not decrease and ends at nnz; every colIdx is inside [0, ncols); target_row (NULL for the plain formats)
+ * does not decrease and stays inside [0, target_rows).  The SpMM / SDDMM kernels trust their inputs, as the
+ * reference's do (no check anywhere in SpMM/SpMM.cpp): an index outside X makes them read outside the buffer.  ORs
+ * psp_build_flag bits into *status (set to 0 by the caller). */
+int psp_check_index_dev(const int *rowPtr, const int *colIdx, const int *target_row, int M, int nnz, int ncols,
+                        int target_rows, int *status, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: genmask, SDDMM/sddmm.cpp:663-673 -> sddmm_kernel.cu:78-141.

@@ -112,6 +112,13 @@ class pcsr_spmm(object):
             self.mtx_nodes, self.mtx_edges = mtx_nodes, mtx_edges
             self.rowPtr, self.colIdx, self.val = rowPtr.to(device), colIdx.to(device), val.to(device)
             self.target_row = None if target_row is None else target_row.to(device)
+            if torch.device(device).type == "cuda":
+                # arrays of unknown origin: the kernels trust their indices, so look at them once
+                from . import device_builder
+
+                rows = (mtx_nodes + vec_size - 1) // vec_size
+                device_builder.check_index(self.rowPtr, self.colIdx, rows * vec_size, self.target_row, rows,
+                                           what="pcsr_spmm index arrays")
         else:
             self.mtx_nodes, self.mtx_edges = graph.mtx_nodes, graph.mtx_edges
             fmt = graph.csr_data if vec_size == 1 else graph.bcsr_data

@@ -50,6 +50,7 @@ SIGNATURES = {
     "psp_split_csr_fill_dev": [_vp, _vp, _i, _i, _i, _vp, _vp, _vp],
     "psp_bcsr_offsets_dev": [_vp, _vp, _i, _vp, _vp, _i, _vp, _vp],
     "psp_bcsr_fill_dev": [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp],
+    "psp_check_index_dev": [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp],
     "psp_genmask": [_vp, _vp, _vp, _i, _i, _vp, _vp],
     "psp_spmm_csr_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "psp_spmm_csr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],

@@ -258,3 +258,42 @@ PSP_EXPORT int psp_bcsr_fill_dev(const int *rowPtr, const int *colIdx, const flo
                        nrows, nbr, (int *)nullptr, rowPtr_b, colIdx_b, val_b, (int *)nullptr);
     return psp_check_launch("bcsr fill kernel");
 }
+
+// ---- index validation ---------------------------------------------------------------------------------------------
+// The SpMM / SDDMM kernels trust their index arrays, as the reference's kernels do: a column index outside X makes
+// them read outside the buffer.  This pass lets a caller check arrays of unknown origin once, on the device.
+__global__ void check_index_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
+                                   const int *__restrict__ target_row, int M, int nnz, int ncols, int target_rows,
+                                   int *__restrict__ status)
+{
+    const long long stride = (long long)gridDim.x * blockDim.x;
+    const long long t = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    int bad = 0;
+    if (t == 0 && (rowPtr[0] != 0 || rowPtr[M] != nnz)) bad |= PSP_BUILD_BAD_ROWPTR;
+    for (long long i = t; i < M; i += stride) {
+        const int a = rowPtr[i], b = rowPtr[i + 1];
+        if (a > b || a < 0 || b > nnz) bad |= PSP_BUILD_BAD_ROWPTR;
+        if (target_row) {
+            const int r = target_row[i];
+            if (r < 0 || r >= target_rows || (i > 0 && target_row[i - 1] > r)) bad |= PSP_BUILD_BAD_TARGET;
+        }
+    }
+    for (long long p = t; p < nnz; p += stride) {
+        const int c = colIdx[p];
+        if (c < 0 || c >= ncols) bad |= PSP_BUILD_BAD_COLUMN;
+    }
+    if (bad) atomicOr(status, bad);
+}
+
+PSP_EXPORT int psp_check_index_dev(const int *rowPtr, const int *colIdx, const int *target_row, int M, int nnz, int ncols,
+                                   int target_rows, int *status, psp_stream_t stream)
+{
+    PSP_REQUIRE(rowPtr && status && M >= 0 && nnz >= 0 && ncols >= 0, "check_index_dev: bad input");
+    PSP_REQUIRE(colIdx || nnz == 0, "check_index_dev: colIdx is null");
+    const long long work = (long long)M > nnz ? M : nnz;
+    int blocks = psp_ceil_div(work > 0 ? work : 1, 256);
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(check_index_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, rowPtr, colIdx, target_row, M, nnz,
+                       ncols, target_rows, status);
+    return psp_check_launch("index check kernel");
+}

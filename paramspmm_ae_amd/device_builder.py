@@ -22,7 +22,11 @@ def _stream():
 def _check_status(status, what):
     flags = int(status.item())  # synchronises with the builder kernels
     if flags & 4:
-        raise ValueError("%s: rowPtr decreases" % what)
+        raise ValueError("%s: rowPtr decreases, does not start at 0 or does not end at the entry count" % what)
+    if flags & 8:
+        raise ValueError("%s: a column index lies outside the matrix" % what)
+    if flags & 16:
+        raise ValueError("%s: target_row decreases or names a row outside the matrix" % what)
     if flags & 1:
         raise OverflowError("%s: more than 2^31-1 output entries" % what)
     if flags & 2:
@@ -33,6 +37,29 @@ def _dev_i32(t):
     if not (t.is_cuda and t.dtype == torch.int32 and t.is_contiguous()):
         raise ValueError("expected a contiguous int32 CUDA tensor")
     return t
+
+
+def check_index(rowPtr, colIdx, ncols, target_row=None, target_rows=0, what="index arrays"):
+    """Raises ValueError when the arrays (on the GPU) would make the kernels read or write outside their buffers."""
+    rowPtr, colIdx = _dev_i32(rowPtr), _dev_i32(colIdx)
+    if target_row is not None:
+        target_row = _dev_i32(target_row)
+    with torch.cuda.device(rowPtr.device):
+        status = torch.zeros(1, dtype=torch.int32, device=rowPtr.device)
+        _capi.check(_capi.lib.psp_check_index_dev(_capi.ptr(rowPtr), _capi.ptr(colIdx) if colIdx.numel() else None,
+                                                  _capi.ptr(target_row), rowPtr.numel() - 1, colIdx.numel(), int(ncols),
+                                                  int(target_rows), _capi.ptr(status), _stream()))
+        _check_status(status, what)
+
+
+def to_host(*tensors):
+    """Device tensors -> host tensors through page-locked memory (several times the rate of a pageable copy; the
+    host copies stay page-locked, which also speeds up any later upload)."""
+    out = [torch.empty(t.shape, dtype=t.dtype, pin_memory=True) for t in tensors]
+    for h, t in zip(out, tensors):
+        h.copy_(t, non_blocking=True)
+    torch.cuda.synchronize()
+    return out
 
 
 def split_csr_device(rowPtr, g):

@@ -136,7 +136,7 @@ class csr_data(object):
             from . import device_builder
 
             rs, tr = device_builder.split_csr_device(self.on_device("rowPtr", "cuda"), self.split_granularity)
-            self.rowPtr_split, self.target_row = rs.cpu(), tr.cpu()
+            self.rowPtr_split, self.target_row = device_builder.to_host(rs, tr)
             self._keep_device("rowPtr_split", rs)
             self._keep_device("target_row", tr)
         else:
@@ -197,7 +197,7 @@ def build_bcsr(rowPtr, colIdx, val, ncols=None, build_on="host", device_arrays=N
             out = device_builder.build_bcsr_device(*src)
             if device_arrays is not None:
                 device_arrays[:] = out
-            return tuple(t.cpu().numpy() for t in out)
+            return tuple(t.numpy() for t in device_builder.to_host(*out))
         except device_builder.NotCanonical:
             if build_on == "device":
                 raise
@@ -287,7 +287,11 @@ class graph_input(object):
 
         on_gpu = []
         if _use_device(build_on):
+            from . import device_builder
+
             on_gpu = [self.csr_data.on_device(k, "cuda") for k in ("rowPtr", "colIdx", "val")]
+            # the host builder rejects column indices outside the matrix; so does this path
+            device_builder.check_index(on_gpu[0], on_gpu[1], n + (n & 1), what="load_from_csr")
         rowPtr_b, colIdx_b, val_b = build_bcsr(rowPtr, colIdx, val, build_on=build_on, device_arrays=on_gpu)
         nblk = colIdx_b.size
         # graph_input.py:257-266: the blocked format counts block-rows and blocks (the latter as a float)

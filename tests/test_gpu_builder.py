@@ -148,3 +148,42 @@ def test_graph_input_same_on_host_and_device():
             assert a.dtype == b.dtype and a.shape == b.shape and torch.equal(a, b), (fmt, name)
     assert torch.equal(h.mask, d.mask)
     assert np.array_equal(h.get_info(), d.get_info())
+
+
+def test_index_check_reports_what_would_fault():
+    """psp_check_index_dev: arrays that would make the SpMM / SDDMM kernels leave their buffers are reported."""
+    from paramspmm_ae_amd import device_builder
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+
+    rowPtr, colIdx, val = random_csr(3000, 5.0, 1, empty_frac=0.2)
+    n = rowPtr.size - 1
+    device_builder.check_index(dev(rowPtr), dev(colIdx), n)  # fine
+    bad = colIdx.copy()
+    bad[bad.size // 2] = n
+    with pytest.raises(ValueError, match="column index"):
+        device_builder.check_index(dev(rowPtr), dev(bad), n)
+    bad[bad.size // 2] = -1
+    with pytest.raises(ValueError, match="column index"):
+        device_builder.check_index(dev(rowPtr), dev(bad), n)
+    rp = rowPtr.copy()
+    rp[10] = rp[11] + 1
+    with pytest.raises(ValueError, match="rowPtr"):
+        device_builder.check_index(dev(rp), dev(colIdx), n)
+    rp = rowPtr.copy()
+    rp[-1] -= 1
+    with pytest.raises(ValueError, match="rowPtr"):
+        device_builder.check_index(dev(rp), dev(colIdx), n)
+    rs, tr = split_dev(rowPtr, 4)
+    device_builder.check_index(dev(rs), dev(colIdx), n, dev(tr), n)
+    tr_bad = tr.copy()
+    tr_bad[5], tr_bad[6] = tr_bad[6] + 1, tr_bad[5]
+    with pytest.raises(ValueError, match="target_row"):
+        device_builder.check_index(dev(rs), dev(colIdx), n, dev(tr_bad), n)
+    # the facade checks arrays it is handed directly
+    with pytest.raises(ValueError, match="column index"):
+        pcsr_spmm(None, 1, False, mtx_nodes=n, mtx_edges=colIdx.size, rowPtr=torch.from_numpy(rowPtr),
+                  colIdx=torch.from_numpy(np.where(np.arange(colIdx.size) == 7, n + 5, colIdx).astype(np.int32)),
+                  val=torch.from_numpy(val))
+    op = pcsr_spmm(None, 1, False, mtx_nodes=n, mtx_edges=colIdx.size, rowPtr=torch.from_numpy(rowPtr),
+                   colIdx=torch.from_numpy(colIdx), val=torch.from_numpy(val))
+    assert op.colIdx.is_cuda
