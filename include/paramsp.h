@@ -198,6 +198,18 @@ int psp_gemm_atb_supported(int K1, int K2);
 int psp_gemm_atb_f32(const float *A, const float *B, float *C, long long n, int K1, int K2, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * DEVICE: mean negative log-likelihood, the loss of the reference's training step (F.nll_loss(model(), labels),
+ * GNN.py:131-146), forward and backward.  logp is [n, C] row-major log-probabilities, labels are int64; rows whose
+ * label is outside [0, C) do not count.  loss: one float.  stats: two floats of device memory that the forward
+ * call fills (sum, count) and the backward call reads.  grad_loss: one float on the device (the incoming
+ * gradient); grad_logp [n, C] is overwritten.  The sum is accumulated with fp32 atomics.
+ * ------------------------------------------------------------------------------------------- */
+int psp_nll_loss_mean_f32(const float *logp, const long long *labels, long long n, int C, float *loss, float *stats,
+                          psp_stream_t stream);
+int psp_nll_loss_mean_backward_f32(const long long *labels, const float *grad_loss, const float *stats, long long n,
+                                   int C, float *grad_logp, psp_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * DEVICE: comparison baseline, ParamSpMM.gespmm_compute (SpMM/Baseline_kernel.cu:616-788): CSR SpMM with one
  * wavefront per row and the row's (column, value) pairs cached in LDS.  Y [M,N] is fully written.
  * ------------------------------------------------------------------------------------------- */

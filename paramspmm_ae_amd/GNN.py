@@ -17,7 +17,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .decider import SpMMDecider, DEFAULT_PICKLE_PATH
-from .gnn_conv import AGNNConv, GCNConv, GINConv
+from .gnn_conv import AGNNConv, GCNConv, GINConv, nll_loss_mean
 from .graph_input import graph_input
 from .PCSR import pcsr_spmm
 
@@ -93,13 +93,13 @@ def capture_training_step(model, labels, optimizer, warmup=3):
     with torch.cuda.stream(side):
         for _ in range(warmup):
             optimizer.zero_grad(set_to_none=True)
-            F.nll_loss(model(), labels).backward()
+            nll_loss_mean(model(), labels).backward()
             optimizer.step()
     torch.cuda.current_stream().wait_stream(side)
     optimizer.zero_grad(set_to_none=True)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        loss = F.nll_loss(model(), labels)
+        loss = nll_loss_mean(model(), labels)
         loss.backward()
         optimizer.step()
     return graph, loss
@@ -113,7 +113,7 @@ def train_profiling(model, labels, num_epoches, verbose=False, progress=False, h
     def epoch():
         model.train()
         optimizer.zero_grad()
-        loss = F.nll_loss(model(), labels)
+        loss = nll_loss_mean(model(), labels)
         loss.backward()
         optimizer.step()
         return loss

@@ -59,6 +59,43 @@ static std::vector<Tensor> backward_impl(int fmt, const Tensor &dY, const Tensor
     return {torch::mm(AG, W.t()), weight_gradient(H, AG)};
 }
 
+// ---- mean NLL loss of the training step (an addition of this build; F.nll_loss in GNN.py:131-146) ----------
+static void check_loss_args(const Tensor &logp, const Tensor &labels)
+{
+    need_gpu(logp, "log-probabilities");
+    need_gpu(labels, "labels");
+    TORCH_CHECK(logp.dim() == 2 && logp.scalar_type() == torch::kFloat32 && logp.is_contiguous(),
+                "nll_loss_mean: log-probabilities must be a contiguous float32 [n, C] tensor");
+    TORCH_CHECK(labels.dim() == 1 && labels.scalar_type() == torch::kInt64 && labels.is_contiguous() &&
+                    labels.size(0) == logp.size(0),
+                "nll_loss_mean: labels must be a contiguous int64 tensor with one entry per row");
+    TORCH_CHECK(logp.device() == labels.device(), "nll_loss_mean: tensors on different devices");
+}
+// returns [loss (0-dim), stats (2 floats: sum, count) for the backward call]
+static std::vector<Tensor> nll_loss_mean(Tensor logp, Tensor labels)
+{
+    check_loss_args(logp, labels);
+    DeviceGuard guard(logp.device());
+    Tensor loss = torch::empty({}, logp.options()), stats = torch::empty({2}, logp.options());
+    ok(psp_nll_loss_mean_f32(fp(logp), (const long long *)labels.data_ptr<int64_t>(), logp.size(0), (int)logp.size(1),
+                             loss.data_ptr<float>(), stats.data_ptr<float>(), stream_of(logp)));
+    return {loss, stats};
+}
+static Tensor nll_loss_mean_backward(Tensor labels, Tensor grad_loss, Tensor stats, long n, long C)
+{
+    need_gpu(labels, "labels");
+    need_gpu(grad_loss, "grad_loss");
+    need_gpu(stats, "stats");
+    TORCH_CHECK(labels.scalar_type() == torch::kInt64 && labels.is_contiguous() && labels.numel() == n, "bad labels");
+    TORCH_CHECK(grad_loss.scalar_type() == torch::kFloat32 && grad_loss.numel() == 1, "grad_loss must hold one float");
+    TORCH_CHECK(stats.scalar_type() == torch::kFloat32 && stats.numel() == 2 && stats.is_contiguous(), "bad stats");
+    DeviceGuard guard(labels.device());
+    Tensor grad = torch::empty({n, C}, stats.options());
+    ok(psp_nll_loss_mean_backward_f32((const long long *)labels.data_ptr<int64_t>(), grad_loss.data_ptr<float>(),
+                                      stats.data_ptr<float>(), n, (int)C, fpw(grad), stream_of(labels)));
+    return grad;
+}
+
 #define PSP_CONV(NAME, FMT)                                                                                       \
     static Tensor NAME##_forward(Tensor H, Tensor W, Tensor rowPtr, Tensor colIdx, Tensor values, int CF, int bw)  \
     {                                                                                                             \
@@ -96,6 +133,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
         need_gpu(G, "G");
         return weight_gradient(H, G);
     }, "H^T * G");
+    m.def("nll_loss_mean", &nll_loss_mean, "[loss, stats] of the mean negative log-likelihood (log-probabilities, int64 labels)");
+    m.def("nll_loss_mean_backward", &nll_loss_mean_backward, "gradient w.r.t. the log-probabilities: (labels, grad_loss, stats, n, C)");
     m.def("csr_spmm_forward", &csr_spmm_forward, "A*(H*W), CSR");
     m.def("csr_spmm_backward", &csr_spmm_backward, "[dH, dW], CSR");
     m.def("csr_split_spmm_forward", &csr_split_spmm_forward, "A*(H*W), row-split CSR");

@@ -24,6 +24,32 @@ def _conv_name(op):
     return _CONV[(bool(op.if_split), op.vec_size != 1)]
 
 
+class _NllLossMean(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logp, labels):
+        loss, stats = SpCONV.nll_loss_mean(logp, labels)
+        ctx.save_for_backward(labels, stats)
+        ctx.shape = tuple(logp.shape)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        labels, stats = ctx.saved_tensors
+        return SpCONV.nll_loss_mean_backward(labels, grad_loss.contiguous(), stats, ctx.shape[0], ctx.shape[1]), None
+
+
+def nll_loss_mean(logp, labels):
+    """``F.nll_loss(logp, labels)`` (mean over the rows, the loss of the reference's training step, GNN.py:131-146)
+    through the library's kernels.  PyTorch reduces the whole batch in one workgroup -- 1.7 ms per step forward plus
+    backward on 10^6 nodes -- where these kernels take some tens of microseconds.  Rows whose label is outside
+    [0, C) do not count, as with PyTorch's ignore_index.  Anything but contiguous float32 CUDA log-probabilities with
+    int64 labels goes to PyTorch."""
+    if (logp.is_cuda and logp.dtype == torch.float32 and logp.dim() == 2 and labels.dtype == torch.int64
+            and labels.dim() == 1):
+        return _NllLossMean.apply(logp.contiguous(), labels.contiguous())
+    return torch.nn.functional.nll_loss(logp, labels)
+
+
 class GCNFunction(torch.autograd.Function):
     """forward A(HW); backward dH = (A dY) W^T, dW = H^T (A dY) -- A is symmetric (gnn_conv.py:13-107)."""
 

@@ -303,7 +303,7 @@ def test_training_step_in_hip_graph_matches_eager(monkeypatch, net, config):
     for step in range(7):
         model_e.train()
         opt_e.zero_grad(set_to_none=True)
-        loss = F.nll_loss(model_e(), g.y)
+        loss = GNN.nll_loss_mean(model_e(), g.y)
         loss.backward()
         opt_e.step()
         if step >= 3:
@@ -322,3 +322,25 @@ def test_training_step_in_hip_graph_matches_eager(monkeypatch, net, config):
         (junk @ junk).sum().item()
     for pe, pg in zip(model_e.parameters(), model_g.parameters()):
         torch.testing.assert_close(pg, pe, rtol=0, atol=5e-3)
+
+
+@pytest.mark.parametrize("n,C", [(1, 1), (1000, 16), (100_003, 7), (1_000_000, 16), (4097, 32)])
+def test_nll_loss_mean_matches_torch(n, C):
+    """The library's mean NLL loss (forward value and gradient) against torch's on the same log-probabilities,
+    including labels outside [0, C), which do not count (-100 is PyTorch's ignore_index)."""
+    import torch.nn.functional as F
+    from paramspmm_ae_amd.gnn_conv import nll_loss_mean
+
+    g = torch.Generator(device="cuda").manual_seed(n + C)
+    logits = torch.randn(n, C, device="cuda", generator=g)
+    labels = torch.randint(0, C, (n,), device="cuda", generator=g)
+    if n > 10:
+        labels[::7] = -100
+    a = F.log_softmax(logits, dim=1).detach().requires_grad_(True)
+    b = a.detach().clone().requires_grad_(True)
+    la = nll_loss_mean(a, labels)
+    lb = F.nll_loss(b, labels)
+    torch.testing.assert_close(la, lb, rtol=2e-5, atol=1e-6)
+    (la * 3.0).backward()
+    (lb * 3.0).backward()
+    torch.testing.assert_close(a.grad, b.grad, rtol=1e-6, atol=0)
