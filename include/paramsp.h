@@ -198,6 +198,16 @@ int psp_gemm_atb_supported(int K1, int K2);
 int psp_gemm_atb_f32(const float *A, const float *B, float *C, long long n, int K1, int K2, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * DEVICE: Y[n,K2] = X[n,K1] * W (transW = 0, W is [K1,K2] row-major) or X * W^T (transW != 0, W is [K2,K1]) for
+ * tall-skinny X and a small weight matrix: torch::mm(H, W) and torch::mm(AG, W.t()) of the fused GCN layer
+ * (SpCONV/SpCONV.h:43-71).  Supported widths: K2 in {16, 32}, K1 in {16, 32, 48, 64} (and 128 with K2 = 16);
+ * psp_gemm_xw_supported tells.  Y is overwritten; X and Y 16-byte aligned.  Deterministic (one lane per row).
+ * ------------------------------------------------------------------------------------------- */
+int psp_gemm_xw_supported(int K1, int K2);
+int psp_gemm_xw_f32(const float *X, const float *W, float *Y, long long n, int K1, int K2, int transW,
+                    psp_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * DEVICE: mean negative log-likelihood, the loss of the reference's training step (F.nll_loss(model(), labels),
  * GNN.py:131-146), forward and backward.  logp is [n, C] row-major log-probabilities, labels are int64; rows whose
  * label is outside [0, C) do not count.  loss: one float.  stats: two floats of device memory that the forward

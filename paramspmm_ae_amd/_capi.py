@@ -65,6 +65,8 @@ SIGNATURES = {
     "psp_baseline_rowcache_spmm_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
     "psp_nll_loss_mean_f32": [_vp, _vp, ctypes.c_longlong, _i, _vp, _vp, _vp],
     "psp_nll_loss_mean_backward_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _vp, _vp],
+    "psp_gemm_xw_supported": [_i, _i],
+    "psp_gemm_xw_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _i, _vp],
     "psp_gemm_atb_supported": [_i, _i],
     "psp_gemm_atb_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _vp],
 }

@@ -39,12 +39,29 @@ static Tensor weight_gradient(const Tensor &H, const Tensor &AG)
     return dW;
 }
 
+// X * W (or X * W^T): the library's one-lane-per-row kernel for narrow layers on many rows, torch::mm otherwise
+static Tensor dense_xw(const Tensor &X, const Tensor &W, bool transW)
+{
+    const long K1 = X.dim() == 2 ? X.size(1) : -1;
+    const bool shapes = X.dim() == 2 && W.dim() == 2 && W.size(transW ? 1 : 0) == K1;
+    const long K2 = shapes ? W.size(transW ? 0 : 1) : -1;
+    const bool narrow = shapes && X.size(0) >= 16384 && X.scalar_type() == torch::kFloat32 &&
+                        W.scalar_type() == torch::kFloat32 && X.is_cuda() && W.is_cuda() &&
+                        psp_gemm_xw_supported((int)K1, (int)K2);
+    if (!narrow) return torch::mm(X, transW ? W.t() : W);
+    Tensor Xc = X.contiguous(), Wc = W.contiguous();
+    DeviceGuard guard(Xc.device());
+    Tensor Y = torch::empty({Xc.size(0), K2}, Xc.options());
+    ok(psp_gemm_xw_f32(fp(Xc), fp(Wc), fpw(Y), Xc.size(0), (int)K1, (int)K2, transW ? 1 : 0, stream_of(Xc)));
+    return Y;
+}
+
 static Tensor forward_impl(int fmt, const Tensor &H, const Tensor &W, const Tensor &rowPtr, const Tensor &colIdx,
                            const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
 {
     need_gpu(H, "input");
     need_gpu(W, "weight");
-    return aggregate(fmt, torch::mm(H, W), rowPtr, colIdx, values, target_row, CF, blkWarpNum);
+    return aggregate(fmt, dense_xw(H, W, false), rowPtr, colIdx, values, target_row, CF, blkWarpNum);
 }
 
 static std::vector<Tensor> backward_impl(int fmt, const Tensor &dY, const Tensor &H, const Tensor &W, const Tensor &rowPtr,
@@ -56,7 +73,7 @@ static std::vector<Tensor> backward_impl(int fmt, const Tensor &dY, const Tensor
     // the reference multiplies by A, not A^T (SpCONV/SpCONV.h:67-71): exact for the symmetric matrices its
     // loaders build
     Tensor AG = aggregate(fmt, dY, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
-    return {torch::mm(AG, W.t()), weight_gradient(H, AG)};
+    return {dense_xw(AG, W, true), weight_gradient(H, AG)};
 }
 
 // ---- mean NLL loss of the training step (an addition of this build; F.nll_loss in GNN.py:131-146) ----------
@@ -133,6 +150,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
         need_gpu(G, "G");
         return weight_gradient(H, G);
     }, "H^T * G");
+    m.def("dense_xw", [](Tensor X, Tensor W, bool transW) {
+        need_gpu(X, "X");
+        need_gpu(W, "W");
+        return dense_xw(X, W, transW);
+    }, "X * W (transW false) or X * W^T for tall-skinny X: (X, W, transW)");
     m.def("nll_loss_mean", &nll_loss_mean, "[loss, stats] of the mean negative log-likelihood (log-probabilities, int64 labels)");
     m.def("nll_loss_mean_backward", &nll_loss_mean_backward, "gradient w.r.t. the log-probabilities: (labels, grad_loss, stats, n, C)");
     m.def("csr_spmm_forward", &csr_spmm_forward, "A*(H*W), CSR");

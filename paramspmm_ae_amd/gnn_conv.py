@@ -95,7 +95,7 @@ class AGNNFunction(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, X, weights, attention_w, ParamSpMM, colIdx):
-        X_prime = torch.mm(X, weights)
+        X_prime = SpCONV.dense_xw(X, weights, False)
         edge_feature = ParamSpMM.AGNN_sddmm(X_prime)
         # csr: [nnz] ; 2x1 blocks: [nblk, 2] -- a single head scales both the same way
         edge_attentions = (edge_feature * attention_w.reshape(())).contiguous()
@@ -111,7 +111,7 @@ class AGNNFunction(torch.autograd.Function):
         X, weights, edge_attentions = ctx.saved_tensors
         d_output = d_output.contiguous()
         d_input_prime = op.AGNN_spmm(edge_attentions, d_output)
-        d_input = torch.mm(d_input_prime, weights.t().contiguous())
+        d_input = SpCONV.dense_xw(d_input_prime, weights, True)
         d_weights = SpCONV.weight_gradient(X, d_input_prime)  # X^T * d_input_prime
         d_attention = op.AGNN_sddmm(d_output)
         if d_attention.dim() != 1:
@@ -138,13 +138,13 @@ class GINFunction(torch.autograd.Function):
         X_agg = ParamSpMM.GIN_spmm(X)
         ctx.save_for_backward(X_agg, weight)
         ctx.ParamSpMM = ParamSpMM
-        return torch.mm(X_agg, weight)
+        return SpCONV.dense_xw(X_agg, weight, False)
 
     @staticmethod
     def backward(ctx, d_output):
         X_agg, weights = ctx.saved_tensors
         d_weights = SpCONV.weight_gradient(X_agg, d_output.contiguous())  # X_agg^T * d_output
-        d_input = ctx.ParamSpMM.GIN_spmm(torch.mm(d_output, weights.t()).contiguous())
+        d_input = ctx.ParamSpMM.GIN_spmm(SpCONV.dense_xw(d_output, weights, True))
         return d_input, d_weights, None
 
 

@@ -344,3 +344,27 @@ def test_nll_loss_mean_matches_torch(n, C):
     (la * 3.0).backward()
     (lb * 3.0).backward()
     torch.testing.assert_close(a.grad, b.grad, rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("K1,K2", [(16, 16), (32, 16), (48, 16), (64, 16), (128, 16), (16, 32), (32, 32), (48, 32), (64, 32),
+                                   (24, 16), (128, 128)])
+def test_dense_xw_matches_torch(K1, K2):
+    """X*W and X*W^T of the layers through the one-lane-per-row kernel (supported widths) or torch::mm (the last two
+    shapes), against a float64 product; a row count that is not a multiple of the workgroup size."""
+    import ParamSpCONV
+
+    n = 100_003
+    g = torch.Generator(device="cuda").manual_seed(K1 * 1000 + K2)
+    X = torch.randn(n, K1, device="cuda", generator=g)
+    W = torch.randn(K1, K2, device="cuda", generator=g)
+    want = (X.double() @ W.double())
+    scale = (X.abs().double() @ W.abs().double())
+    got = ParamSpCONV.dense_xw(X, W, False)
+    assert got.shape == (n, K2)
+    assert torch.all((got.double() - want).abs() <= 1e-5 * scale + 1e-6)
+    Wt = W.t().contiguous()  # [K2, K1]
+    got_t = ParamSpCONV.dense_xw(X, Wt, True)
+    assert torch.all((got_t.double() - want).abs() <= 1e-5 * scale + 1e-6)
+    # few rows: torch::mm path, same answer
+    small = ParamSpCONV.dense_xw(X[:100].contiguous(), W, False)
+    assert torch.all((small.double() - want[:100]).abs() <= 1e-5 * scale[:100] + 1e-6)
