@@ -12,7 +12,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libparamsp_hip.so")
 
 if not os.path.exists(LIB_PATH):
     raise ImportError(
-        "libparamsp_hip.so is not built: run `make -C %s` (or script/build_param.sh) first" % os.path.join(_HERE, "csrc")
+        "libparamsp_hip.so is not built: run `make -C %s` (or paramspmm_ae_amd/build_param.sh) first" % os.path.join(_HERE, "csrc")
     )
 
 lib = ctypes.CDLL(LIB_PATH)

@@ -1,6 +1,6 @@
 """Builds the native parts in-tree: libparamsp_hip.so (hipcc, gfx950) and the three PyTorch extension
 modules ParamSpMM / ParamSDDMM / ParamSpCONV (g++, linked against the library).  Everything lands in
-paramspmm_ae_amd/lib/.  Run as `python -m paramspmm_ae_amd.build` or through script/build_param.sh.
+paramspmm_ae_amd/lib/.  Run as `python -m paramspmm_ae_amd.build` or through paramspmm_ae_amd/build_param.sh.
 """
 import os
 import subprocess
