@@ -139,6 +139,20 @@ int psp_spmm_csr_split_f32(const int *rowPtr_split, const int *colIdx, const flo
                            const int *target_row, const float *X, float *Y, int S, int N, int rows_out,
                            int CF, int blkWarpNum, psp_stream_t stream);
 
+/* Softmax-weighted SpMM on the CSR layouts (no counterpart in the reference: the attention pipeline SDDMM ->
+ * softmax -> SpMM in two kernels instead of three passes):
+ *   Y[i] = sum_j w_ij X[j] / sum_j w_ij,  w_ij = exp(e_ij - row_max[i]),
+ * e in CSR entry order, row_max[i] >= every e_ij of row i (psp_sddmm_*_rowmax_f32 delivers the maximum).  Rows without
+ * entries give zeros.  N % 4 == 0 and CF <= 4.  The split variant needs row_sum: rows_out floats of device
+ * workspace (contents irrelevant on entry); rows shared by several wavefronts are accumulated with fp32 atomics and
+ * normalised by a second launch. */
+int psp_spmm_csr_softmax_f32(const int *rowPtr, const int *colIdx, const float *e, const float *row_max,
+                             const float *X, float *Y, int M, int N, int rows_out, int CF, int blkWarpNum,
+                             psp_stream_t stream);
+int psp_spmm_csr_split_softmax_f32(const int *rowPtr_split, const int *colIdx, const float *e, const int *target_row,
+                                   const float *row_max, float *row_sum, const float *X, float *Y, int S, int N,
+                                   int rows_out, int CF, int blkWarpNum, psp_stream_t stream);
+
 /* ParamSpMM.bcsr_spmm, SpMM/SpMM.cpp:209-271 -> SpMM_kernel.cu:273-343, 1362-1493.
  * Mb block-rows; val_b is [nblk,2]; rows_out >= 2*Mb.  A zero block entry contributes nothing. */
 int psp_spmm_bcsr_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *X,
@@ -165,6 +179,15 @@ int psp_sddmm_csr_f32(const int *rowPtr, const int *colIdx, const float *A, cons
 int psp_sddmm_csr_split_f32(const int *rowPtr_split, const int *colIdx, const int *target_row,
                             const float *A, const float *B, const float *scale, float *out, int S, int K,
                             int blkWarpNum, psp_stream_t stream);
+
+/* The two CSR variants with the largest result of every row delivered as well: row_max[rows] (overwritten; rows
+ * without entries keep the lowest float).  No counterpart in the reference; feeds psp_spmm_*_softmax_f32. */
+int psp_sddmm_csr_rowmax_f32(const int *rowPtr, const int *colIdx, const float *A, const float *B,
+                             const float *scale, float *out, float *row_max, int M, int K, int blkWarpNum,
+                             psp_stream_t stream);
+int psp_sddmm_csr_split_rowmax_f32(const int *rowPtr_split, const int *colIdx, const int *target_row,
+                                   const float *A, const float *B, const float *scale, float *out, float *row_max,
+                                   int S, int rows, int K, int blkWarpNum, psp_stream_t stream);
 
 /* ParamSDDMM.bcsr_sddmm, SDDMM/sddmm.cpp:122-172 -> sddmm_kernel.cu:248-300, 1059-1176.
  * out is [nblk,2]; entries whose block value is zero are written as zero.  A needs 2*Mb rows. */

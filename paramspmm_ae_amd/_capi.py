@@ -58,6 +58,10 @@ SIGNATURES = {
     "psp_spmm_bcsr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "psp_sddmm_csr_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "psp_sddmm_csr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "psp_sddmm_csr_rowmax_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "psp_sddmm_csr_split_rowmax_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "psp_spmm_csr_softmax_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "psp_spmm_csr_split_softmax_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "psp_sddmm_bcsr_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "psp_sddmm_bcsr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "psp_segment_softmax_f32": [_vp, _vp, _vp, _i, _vp],

@@ -102,6 +102,39 @@ int psp_zero_f32(float *p, size_t n, hipStream_t stream)
     return psp_check_launch("zero fill");
 }
 
+__global__ void __launch_bounds__(256) psp_fill_kernel(float *__restrict__ p, size_t n, float value)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = value;
+}
+
+int psp_fill_f32(float *p, size_t n, float value, hipStream_t stream)
+{
+    if (n == 0) return PSP_OK;
+    const int blocks = (int)std::min<size_t>((n + 255) / 256, 256 * 32);
+    hipLaunchKernelGGL(psp_fill_kernel, dim3(blocks), dim3(256), 0, stream, p, n, value);
+    return psp_check_launch("fill");
+}
+
+__global__ void __launch_bounds__(256) psp_row_scale_kernel(float *__restrict__ Y, const float *__restrict__ s, int rows, int N)
+{
+    // 16 lanes per row: almost every row has s == 0 and costs one load
+    const long long g = ((long long)blockIdx.x * blockDim.x + threadIdx.x) >> 4;
+    const int sub = threadIdx.x & 15;
+    if (g >= rows) return;
+    const float w = s[g];
+    if (w == 0.0f) return;
+    const float inv = 1.0f / w;
+    float *yr = Y + g * N;
+    for (int c = sub; c < N; c += 16) yr[c] *= inv;
+}
+
+int psp_row_scale(float *Y, const float *s, int rows, int N, hipStream_t stream)
+{
+    if (rows == 0 || N == 0) return PSP_OK;
+    hipLaunchKernelGGL(psp_row_scale_kernel, dim3(psp_ceil_div((long long)rows * 16, 256)), dim3(256), 0, stream, Y, s, rows, N);
+    return psp_check_launch("row scale");
+}
+
 // ------------------------------------------------------------------------------------------------
 // selective clear for row-split SpMM: one lane per segment (plus one for the rows past the last segment)
 // ------------------------------------------------------------------------------------------------
@@ -287,14 +320,6 @@ psp_segment_softmax_kernel(const int *__restrict__ rowPtr, const float *in, floa
         const float inv = 1.0f / psp_block_sum(s, s_red);
         for (int p = a + threadIdx.x; p < b; p += 256) out[p] = __expf(in[p] - mx) * inv;
     }
-}
-
-// float maximum through the integer atomics: the order of non-negative floats is that of their bit patterns
-// read as signed integers, the order of negative floats is the reverse of their patterns read as unsigned
-__device__ __forceinline__ void psp_atomic_max_f32(float *addr, float v)
-{
-    if (v >= 0.0f) atomicMax((int *)addr, __float_as_int(v));
-    else atomicMin((unsigned int *)addr, __float_as_uint(v));
 }
 
 // PASS 0: row maxima, 1: sums of exp(x - max), 2: results.  One workgroup per chunk of the entry array.
@@ -510,7 +535,16 @@ PSP_EXPORT int psp_spmm_csr_f32(const int *rowPtr, const int *colIdx, const floa
                                 int M, int N, int rows_out, int CF, int blkWarpNum, psp_stream_t stream)
 {
     return psp_spmm_launch<1, false>(rowPtr, colIdx, val, nullptr, X, Y, M, N, rows_out, CF, blkWarpNum,
-                                         (hipStream_t)stream);
+                                         (hipStream_t)stream, nullptr, nullptr);
+}
+
+PSP_EXPORT int psp_spmm_csr_softmax_f32(const int *rowPtr, const int *colIdx, const float *e, const float *row_max,
+                                        const float *X, float *Y, int M, int N, int rows_out, int CF, int blkWarpNum,
+                                        psp_stream_t stream)
+{
+    PSP_REQUIRE(row_max || M == 0, "spmm softmax: row_max is null");
+    return psp_spmm_launch<1, false>(rowPtr, colIdx, e, nullptr, X, Y, M, N, rows_out, CF, blkWarpNum,
+                                     (hipStream_t)stream, row_max, nullptr);
 }
 
 PSP_EXPORT int psp_spmm_csr_split_f32(const int *rowPtr_split, const int *colIdx, const float *val,
@@ -518,14 +552,24 @@ PSP_EXPORT int psp_spmm_csr_split_f32(const int *rowPtr_split, const int *colIdx
                                       int CF, int blkWarpNum, psp_stream_t stream)
 {
     return psp_spmm_launch<1, true>(rowPtr_split, colIdx, val, target_row, X, Y, S, N, rows_out, CF, blkWarpNum,
-                                        (hipStream_t)stream);
+                                        (hipStream_t)stream, nullptr, nullptr);
+}
+
+PSP_EXPORT int psp_spmm_csr_split_softmax_f32(const int *rowPtr_split, const int *colIdx, const float *e,
+                                              const int *target_row, const float *row_max, float *row_sum,
+                                              const float *X, float *Y, int S, int N, int rows_out, int CF,
+                                              int blkWarpNum, psp_stream_t stream)
+{
+    PSP_REQUIRE(row_max || S == 0, "spmm softmax: row_max is null");
+    return psp_spmm_launch<1, true>(rowPtr_split, colIdx, e, target_row, X, Y, S, N, rows_out, CF, blkWarpNum,
+                                    (hipStream_t)stream, row_max, row_sum);
 }
 
 PSP_EXPORT int psp_spmm_bcsr_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *X,
                                  float *Y, int Mb, int N, int rows_out, int CF, int blkWarpNum, psp_stream_t stream)
 {
     return psp_spmm_launch<2, false>(rowPtr_b, colIdx_b, val_b, nullptr, X, Y, Mb, N, rows_out, CF, blkWarpNum,
-                                        (hipStream_t)stream);
+                                        (hipStream_t)stream, nullptr, nullptr);
 }
 
 PSP_EXPORT int psp_spmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b,
@@ -533,14 +577,25 @@ PSP_EXPORT int psp_spmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b
                                        int rows_out, int CF, int blkWarpNum, psp_stream_t stream)
 {
     return psp_spmm_launch<2, true>(rowPtr_bs, colIdx_b, val_b, target_row, X, Y, Sb, N, rows_out, CF, blkWarpNum,
-                                       (hipStream_t)stream);
+                                       (hipStream_t)stream, nullptr, nullptr);
 }
 
 PSP_EXPORT int psp_sddmm_csr_f32(const int *rowPtr, const int *colIdx, const float *A, const float *B,
                                  const float *scale, float *out, int M, int K, int blkWarpNum, psp_stream_t stream)
 {
     return psp_sddmm_launch<false, false>(rowPtr, colIdx, nullptr, nullptr, A, B, scale, out, M, K, blkWarpNum,
-                                          (hipStream_t)stream);
+                                          (hipStream_t)stream, nullptr);
+}
+
+PSP_EXPORT int psp_sddmm_csr_rowmax_f32(const int *rowPtr, const int *colIdx, const float *A, const float *B,
+                                        const float *scale, float *out, float *row_max, int M, int K, int blkWarpNum,
+                                        psp_stream_t stream)
+{
+    PSP_REQUIRE(M >= 0 && (row_max || M == 0), "sddmm rowmax: row_max is null");
+    int rc = psp_fill_f32(row_max, (size_t)M, PSP_F32_LOWEST, (hipStream_t)stream);
+    if (rc != PSP_OK) return rc;
+    return psp_sddmm_launch<false, false>(rowPtr, colIdx, nullptr, nullptr, A, B, scale, out, M, K, blkWarpNum,
+                                          (hipStream_t)stream, row_max);
 }
 
 PSP_EXPORT int psp_sddmm_csr_split_f32(const int *rowPtr_split, const int *colIdx, const int *target_row,
@@ -548,14 +603,26 @@ PSP_EXPORT int psp_sddmm_csr_split_f32(const int *rowPtr_split, const int *colId
                                        int K, int blkWarpNum, psp_stream_t stream)
 {
     return psp_sddmm_launch<false, true>(rowPtr_split, colIdx, nullptr, target_row, A, B, scale, out, S, K,
-                                         blkWarpNum, (hipStream_t)stream);
+                                         blkWarpNum, (hipStream_t)stream, nullptr);
+}
+
+PSP_EXPORT int psp_sddmm_csr_split_rowmax_f32(const int *rowPtr_split, const int *colIdx, const int *target_row,
+                                              const float *A, const float *B, const float *scale, float *out,
+                                              float *row_max, int S, int rows, int K, int blkWarpNum,
+                                              psp_stream_t stream)
+{
+    PSP_REQUIRE(rows >= 0 && (row_max || rows == 0), "sddmm rowmax: row_max is null");
+    int rc = psp_fill_f32(row_max, (size_t)rows, PSP_F32_LOWEST, (hipStream_t)stream);
+    if (rc != PSP_OK) return rc;
+    return psp_sddmm_launch<false, true>(rowPtr_split, colIdx, nullptr, target_row, A, B, scale, out, S, K,
+                                         blkWarpNum, (hipStream_t)stream, row_max);
 }
 
 PSP_EXPORT int psp_sddmm_bcsr_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *A,
                                   const float *B, float *out, int Mb, int K, int blkWarpNum, psp_stream_t stream)
 {
     return psp_sddmm_launch<true, false>(rowPtr_b, colIdx_b, val_b, nullptr, A, B, nullptr, out, Mb, K, blkWarpNum,
-                                         (hipStream_t)stream);
+                                         (hipStream_t)stream, nullptr);
 }
 
 PSP_EXPORT int psp_sddmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b,
@@ -563,5 +630,5 @@ PSP_EXPORT int psp_sddmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_
                                         int K, int blkWarpNum, psp_stream_t stream)
 {
     return psp_sddmm_launch<true, true>(rowPtr_bs, colIdx_b, val_b, target_row, A, B, nullptr, out, Sb, K,
-                                        blkWarpNum, (hipStream_t)stream);
+                                        blkWarpNum, (hipStream_t)stream, nullptr);
 }

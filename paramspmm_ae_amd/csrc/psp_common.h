@@ -57,6 +57,24 @@ int psp_stripe_rows(void);
 
 // zero-fill used instead of hipMemsetAsync (callers may capture these launches in a HIP graph)
 int psp_zero_f32(float *p, size_t n, hipStream_t stream);
+// the same for an arbitrary value
+int psp_fill_f32(float *p, size_t n, float value, hipStream_t stream);
+
+// Y[r, :] /= s[r] for every row with s[r] != 0 (rows of the softmax-weighted row-split SpMM that several
+// wavefronts accumulated without normalising)
+int psp_row_scale(float *Y, const float *s, int rows, int N, hipStream_t stream);
+
+#define PSP_F32_LOWEST (-3.402823466e+38f)
+
+#ifdef __HIPCC__
+// float maximum through the integer atomics: the order of non-negative floats is that of their bit patterns read
+// as signed integers, the order of negative floats is the reverse of their patterns read as unsigned
+__device__ __forceinline__ void psp_atomic_max_f32(float *addr, float v)
+{
+    if (v >= 0.0f) atomicMax((int *)addr, __float_as_int(v));
+    else atomicMin((unsigned int *)addr, __float_as_uint(v));
+}
+#endif
 
 // Row-split SpMM: clears exactly the rows of Y the SpMM kernel will not plainly store -- rows whose segments sit
 // in two wavefronts (each wavefront owns 2^logW consecutive segments), rows of empty segments, and rows no segment

@@ -29,16 +29,34 @@ template <int LOGL> __device__ __forceinline__ float psp_group_sum(float v)
     return v;
 }
 
+// Maximum over aligned groups of 2^LOGL lanes (all lanes of the group active); every lane receives it.
+template <int LOGL> __device__ __forceinline__ float psp_group_max(float v)
+{
+#define PSP_DPP_MAX(CTRL) v = fmaxf(v, __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(v), __float_as_int(v), CTRL, 0xF, 0xF, false)))
+    if constexpr (LOGL >= 1) PSP_DPP_MAX(0xB1);
+    if constexpr (LOGL >= 2) PSP_DPP_MAX(0x4E);
+    if constexpr (LOGL >= 3) PSP_DPP_MAX(0x141);
+    if constexpr (LOGL >= 4) PSP_DPP_MAX(0x140);
+#undef PSP_DPP_MAX
+    if constexpr (LOGL >= 5) v = fmaxf(v, __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(v), 0x401F)));
+    if constexpr (LOGL >= 6) v = fmaxf(v, __int_as_float(__builtin_amdgcn_ds_bpermute((int)((threadIdx.x ^ 32) & 63) << 2, __float_as_int(v))));
+    return v;
+}
+
 // val: bcsr -> [nblk,2] block values (gate); csr -> optional per-entry scale (may be null when !SCALE)
 //
 // The walk is the one of the SpMM kernel: a wavefront owns W = 2^logW consecutive segments, their stored entries
 // are divided evenly between the 64/L lane groups, and a group reloads its A row (prefetched one segment ahead)
 // whenever it crosses into another row.  Every stored entry is written exactly once, so `out` needs no clearing.
+//
+// row_max (CSR layouts, may be null): the largest result of every row is also raised into row_max[row] (atomic
+// max, once per lane group and row; the caller has filled the array with the lowest float).  The attention
+// pipeline's softmax-weighted SpMM takes its reference maxima from there instead of sweeping the entries again.
 template <int LOGL, int C, int V, int U, bool BCSR, bool SPLIT, bool SCALE>
 __global__ void __launch_bounds__(512)
 psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
                  const int *__restrict__ target_row, const float *__restrict__ A, const float *__restrict__ B,
-                 float *__restrict__ out, int nseg, int K, int logW, int tiles, int stripe)
+                 float *__restrict__ out, int nseg, int K, int logW, int tiles, int stripe, float *__restrict__ row_max)
 {
     typedef typename psp_vec<V>::type vec_t;
     constexpr int NR = BCSR ? 2 : 1;
@@ -126,6 +144,14 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
         load_a(nk >= 0 ? nk : mykey, a_nxt);
     }
 
+    float lmax = PSP_F32_LOWEST;  // largest result among this lane's entries of the current row
+    auto emit_row_max = [&](int key) {
+        const float m = psp_group_max<LOGL>(lmax);
+        if (sub == 0 && m > PSP_F32_LOWEST) psp_atomic_max_f32(row_max + key, m);
+        lmax = PSP_F32_LOWEST;
+    };
+    const bool want_max = !BCSR && row_max != nullptr;  // uniform
+
     for (int base = a0; base < b0; base += L) {
         const int p = base + sub;
         const bool ok = p < b0;
@@ -170,7 +196,10 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
                             for (int e = 0; e < V; e++) part = __builtin_fmaf(a[r][i][e], psp_elem<V>(bv[u][i], e), part);
                         part = psp_group_sum<LOGL>(part);
                         // positions past run_end belong to the next row: their dot product with this A row is dropped
-                        if (sub == k + u && k + u < run_end) res[r] = part;
+                        if (sub == k + u && k + u < run_end) {
+                            res[r] = part;
+                            if (!BCSR && want_max) lmax = fmaxf(lmax, SCALE ? part * gate[0] : part);
+                        }
                     }
             }
             k = run_end;
@@ -178,6 +207,7 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
                 const int2 nx = w_seg[++cur];
                 row_end = nx.x;
                 if (nx.y != mykey) {
+                    if (want_max) emit_row_max(mykey);  // the group is converged here: the condition is group-uniform
                     mykey = nx.y;
 #pragma unroll
                     for (int r = 0; r < NR; r++)
@@ -202,10 +232,11 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
             }
         }
     }
+    if (want_max) emit_row_max(mykey);
 }
 
 typedef void (*psp_sddmm_kernel_t)(const int *, const int *, const float *, const int *, const float *,
-                                   const float *, float *, int, int, int, int, int);
+                                   const float *, float *, int, int, int, int, int, float *);
 
 // (LOGL, C, U) triples that exist.  C grows only once the group is 16 lanes wide (DPP-only reduction);
 // beyond 64 vectors the group widens to 32 and 64 lanes.
@@ -230,4 +261,4 @@ static psp_sddmm_kernel_t psp_sddmm_lookup(int logL, int C, int V)
 template <bool BCSR, bool SPLIT>
 int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
                      const float *A, const float *B, const float *scale, float *out, int nrows, int K,
-                     int blkWarpNum, hipStream_t stream);
+                     int blkWarpNum, hipStream_t stream, float *row_max);

@@ -5,7 +5,7 @@
 template <bool BCSR, bool SPLIT>
 int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
                      const float *A, const float *B, const float *scale, float *out, int nrows, int K,
-                     int blkWarpNum, hipStream_t stream)
+                     int blkWarpNum, hipStream_t stream, float *row_max)
 {
     PSP_REQUIRE(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8");
     PSP_REQUIRE(nrows >= 0 && K >= 1, "sddmm: bad size (rows %d, K %d)", nrows, K);
@@ -14,6 +14,7 @@ int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, con
     PSP_REQUIRE(!SPLIT || target_row, "sddmm: target_row is null");
     PSP_REQUIRE(!BCSR || val, "sddmm: block values are null");
     PSP_REQUIRE(!(BCSR && scale), "sddmm: scale is only supported for csr formats");
+    PSP_REQUIRE(!(BCSR && row_max), "sddmm: row maxima are only supported for csr formats");
 
     const int V = (K % 4 == 0) ? 4 : (K % 2 == 0) ? 2 : 1;
     const int nvec = K / V;
@@ -38,6 +39,6 @@ int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, con
     const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block), psp_stripe_rows() / segs_per_block);
     dim3 grid(g.launch, 1, 1), block(blkWarpNum * PSP_WAVE, 1, 1);
     hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, BCSR ? val : scale, target_row, A, B, out, nrows, K,
-                       logW, g.real, g.stripe);
+                       logW, g.real, g.stripe, row_max);
     return psp_check_launch("sddmm kernel");
 }

@@ -56,14 +56,23 @@ __device__ __forceinline__ float psp_bperm_f(int src_lane, float v)
 #define PSP_MAX_WAVES 8  // blkWarpNum is 4 or 8
 
 // NR: rows per stored entry (1 = CSR, 2 = 2x1 BCSR).  SPLIT: segments carry an explicit output row.
-template <int C, int V, int U, int NR, bool SPLIT>
+// SM (CSR layouts): the stored values are attention scores e; the product is taken with softmax weights,
+//   Y[i] = sum_j exp(e_ij - m_i) X[j] / sum_j exp(e_ij - m_i),   m_i = row_max[i] (any upper bound of the row works,
+// the SDDMM kernel delivers the exact maximum).  The weights are formed on the fly, their sum travels with the
+// partial sums like one more column, and a row is divided by it when it is written.  A row that several wavefronts
+// share is accumulated unnormalised (atomics) together with its weight sum in row_sum; psp_row_scale_kernel divides
+// such rows afterwards.  This replaces the separate softmax pass over the entries.
+template <int C, int V, int U, int NR, bool SPLIT, bool SM>
 __global__ void __launch_bounds__(512)
 psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
                 const int *__restrict__ target_row, const float *__restrict__ X, float *__restrict__ Y,
-                int nseg, int N, int logL, int logW, int tiles, int stripe, int align_pct)
+                int nseg, int N, int logL, int logW, int tiles, int stripe, int align_pct,
+                const float *__restrict__ row_max, float *__restrict__ row_sum)
 {
+    static_assert(!SM || NR == 1, "softmax weights exist for the CSR layouts only");
     typedef typename psp_vec<V>::type vec_t;
     __shared__ int2 s_seg[PSP_MAX_WAVES][PSP_WAVE];  // (end offset, output row) of the wavefront's segments
+    __shared__ float s_m[SM ? PSP_MAX_WAVES : 1][SM ? PSP_WAVE : 1];  // SM: reference maximum of each segment's row
 
     const int tile = psp_xcd_tile(stripe);
     if (tile >= tiles) return;
@@ -94,7 +103,11 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         s_seg[wave][lane] = make_int2(P1, -1);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        if (filled) s_seg[wave][slot] = make_int2(e, SPLIT ? target_row[s0 + lane] : s0 + lane);
+        if (filled) {
+            const int key = SPLIT ? target_row[s0 + lane] : s0 + lane;
+            s_seg[wave][slot] = make_int2(e, key);
+            if constexpr (SM) s_m[wave][slot] = row_max[key];
+        }
         if constexpr (!SPLIT) {
             // rows without entries are never visited below: write their zeros here, one row per lane group
             unsigned long long empties = __ballot(in && e == b_);
@@ -183,9 +196,21 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         for (int i = 0; i < C; i++)
 #pragma unroll
             for (int e = 0; e < V; e++) acc[r][i][e] = head[r][i][e] = 0.0f;
+    float acc_l = 0.0f, head_l = 0.0f, m_cur = 0.0f;  // SM: weight sum of the running row / stashed head, row maximum
 
     // out: a finished row goes to Y; `shared` = other wavefronts add to the same row (row-split formats)
     auto write_out = [&](int key, bool shared) {
+        if constexpr (SM) {
+            if (!SPLIT || !shared) {
+                const float inv = 1.0f / acc_l;  // the row's largest entry alone contributes exp(0) = 1
+#pragma unroll
+                for (int i = 0; i < C; i++)
+#pragma unroll
+                    for (int e = 0; e < V; e++) acc[0][i][e] *= inv;
+            } else if (sub == 0 && blockIdx.y == 0) {
+                unsafeAtomicAdd(row_sum + key, acc_l);  // one column tile reports the weight sum
+            }
+        }
 #pragma unroll
         for (int r = 0; r < NR; r++) {
             float *yr = Y + (size_t)(key * NR + r) * (size_t)N;
@@ -215,6 +240,7 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         const int2 sg = w_seg[cur];
         row_end = sg.x;
         mykey = sg.y;
+        if constexpr (SM) m_cur = s_m[wave][cur];
         const int seg_begin = cur == 0 ? P0 : w_seg[cur - 1].x;
         head_valid = a > seg_begin;
         if constexpr (SPLIT) {
@@ -257,6 +283,7 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
             const int src = grp_base + min(k + u, L - 1);                                           \
             ck[u] = psp_bperm_i(src, c_cur);                                                        \
             _Pragma("unroll") for (int r = 0; r < NR; r++) vk[u][r] = psp_bperm_f(src, v_cur[r]);   \
+            if constexpr (SM) vk[u][0] = __expf(vk[u][0] - m_cur);                                  \
         }                                                                                           \
         vec_t x[U][C];                                                                              \
         _Pragma("unroll") for (int u = 0; u < U; u++)                                               \
@@ -267,6 +294,7 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         _Pragma("unroll") for (int u = 0; u < U; u++)                                               \
         {                                                                                           \
             if (!(GUARDED) || k + u < run_end) {                                                    \
+                if constexpr (SM) acc_l += vk[u][0];                                                \
                 _Pragma("unroll") for (int r = 0; r < NR; r++)                                      \
                 {                                                                                   \
                     /* 2x1 blocks: a zero entry is skipped (SpMM_kernel.cu:1399,1405) */            \
@@ -309,6 +337,7 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
                             for (int i = 0; i < C; i++)
 #pragma unroll
                                 for (int e = 0; e < V; e++) head[r][i][e] = acc[r][i][e];
+                        head_l = acc_l;
                         flags = F_HEAD | F_CLOSED;
                     } else {
                         write_out(mykey, first_run && ext_head);
@@ -319,8 +348,10 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
                         for (int i = 0; i < C; i++)
 #pragma unroll
                             for (int e = 0; e < V; e++) acc[r][i][e] = 0.0f;
+                    acc_l = 0.0f;
                     first_run = false;
                     mykey = nkey;
+                    if constexpr (SM) m_cur = s_m[wave][cur];
                 }
             }
         }
@@ -349,6 +380,7 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
                     for (int i = 0; i < C; i++)
 #pragma unroll
                         for (int e = 0; e < V; e++) head[r][i][e] = acc[r][i][e];
+                head_l = acc_l;
                 flags = F_HEAD;
             } else {
                 has_tail = true;
@@ -361,6 +393,7 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
                 for (int i = 0; i < C; i++)
 #pragma unroll
                     for (int e = 0; e < V; e++) head[r][i][e] = acc[r][i][e];
+            head_l = acc_l;
             flags = F_HEAD | F_CLOSED | (ext_tail ? F_SHARED : 0);
         } else {
             write_out(mykey, (first_run && ext_head) || ext_tail);
@@ -374,6 +407,10 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         const int src_c = src & (PSP_WAVE - 1);
         const int hf_any = psp_bperm_i(src_c, flags);  // executed by every lane, then masked
         const int hf = (src < PSP_WAVE) ? hf_any : 0;
+        if constexpr (SM) {
+            const float hl = psp_bperm_f(src_c, head_l);
+            if (has_tail && (hf & F_HEAD)) acc_l += hl;
+        }
 #pragma unroll
         for (int r = 0; r < NR; r++)
 #pragma unroll
@@ -398,16 +435,23 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     M_(5, 1) M_(6, 1) M_(7, 1) M_(8, 1)
 
 typedef void (*psp_spmm_kernel_t)(const int *, const int *, const float *, const int *, const float *, float *,
-                                  int, int, int, int, int, int, int);
+                                  int, int, int, int, int, int, int, const float *, float *);
 
+// softmax-weighted variants exist for CSR layouts, float4 columns and up to 4 vectors per lane
 template <int NR, bool SPLIT>
-static psp_spmm_kernel_t psp_spmm_lookup(int C, int V, int U)
+static psp_spmm_kernel_t psp_spmm_lookup(int C, int V, int U, bool softmax)
 {
 #define PSP_CASE(C_, U_)                                                        \
     if (C == C_ && U == U_) {                                                   \
-        if (V == 4) return psp_spmm_kernel<C_, 4, U_, NR, SPLIT>;               \
-        if (V == 2) return psp_spmm_kernel<C_, 2, U_, NR, SPLIT>;               \
-        return psp_spmm_kernel<C_, 1, U_, NR, SPLIT>;                           \
+        if (softmax) {                                                          \
+            if constexpr (NR == 1 && C_ <= 4) {                                 \
+                if (V == 4) return psp_spmm_kernel<C_, 4, U_, 1, SPLIT, true>;  \
+            }                                                                   \
+            return nullptr;                                                     \
+        }                                                                       \
+        if (V == 4) return psp_spmm_kernel<C_, 4, U_, NR, SPLIT, false>;        \
+        if (V == 2) return psp_spmm_kernel<C_, 2, U_, NR, SPLIT, false>;        \
+        return psp_spmm_kernel<C_, 1, U_, NR, SPLIT, false>;                    \
     }
     PSP_SPMM_FOR_EACH_CU(PSP_CASE)
 #undef PSP_CASE
@@ -418,4 +462,4 @@ static psp_spmm_kernel_t psp_spmm_lookup(int C, int V, int U)
 template <int NR, bool SPLIT>
 int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
                     const float *X, float *Y, int nrows, int N, int rows_out, int CF, int blkWarpNum,
-                    hipStream_t stream);
+                    hipStream_t stream, const float *row_max, float *row_sum);

@@ -6,7 +6,7 @@
 template <int NR, bool SPLIT>
 int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
                     const float *X, float *Y, int nrows, int N, int rows_out, int CF, int blkWarpNum,
-                    hipStream_t stream)
+                    hipStream_t stream, const float *row_max, float *row_sum)
 {
     psp_spmm_plan plan;
     int rc = psp_spmm_plan_for(N, CF, blkWarpNum, &plan);
@@ -54,9 +54,17 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     }
     if (rc != PSP_OK) return rc;
     if (nrows == 0) return PSP_OK;
+    const bool softmax = row_max != nullptr;
+    if (softmax && SPLIT) {
+        PSP_REQUIRE(row_sum, "spmm softmax: row_sum workspace is null");
+        rc = psp_zero_f32(row_sum, (size_t)rows_out, stream);
+        if (rc != PSP_OK) return rc;
+    }
 
-    psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll);
-    if (!k) return psp_fail(PSP_ERR_ARG, "spmm: no kernel for coarsen %d vec %d unroll %d", plan.coarsen, plan.vec, plan.unroll);
+    psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll, softmax);
+    if (!k)
+        return psp_fail(PSP_ERR_ARG, "spmm%s: no kernel for coarsen %d vec %d unroll %d%s", softmax ? " softmax" : "", plan.coarsen,
+                        plan.vec, plan.unroll, softmax ? " (needs N % 4 == 0 and CF <= 4)" : "");
 
     int align_pct = 50;
     const char *a_env = getenv("PSP_ALIGN_PCT");  // tuning aid
@@ -64,6 +72,8 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     const int segs_per_block = plan.waves_per_block << logW;
     const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block), psp_stripe_rows() / segs_per_block);
     dim3 grid(g.launch, plan.col_tiles, 1), block(plan.waves_per_block * PSP_WAVE, 1, 1);
-    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.stripe, align_pct);
-    return psp_check_launch("spmm kernel");
+    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.stripe, align_pct, row_max, row_sum);
+    rc = psp_check_launch("spmm kernel");
+    if (rc != PSP_OK || !(softmax && SPLIT)) return rc;
+    return psp_row_scale(Y, row_sum, rows_out, N, stream);  // rows that several wavefronts added to
 }

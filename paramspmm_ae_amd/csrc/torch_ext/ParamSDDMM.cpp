@@ -97,6 +97,40 @@ static Tensor csr_split_sddmm_scaled(Tensor A, Tensor B, Tensor rowPtr_split, Te
     return sddmm_new(1, A, B, rowPtr_split, colIdx, values, &target_row, &values, 1, blkWarpNum);
 }
 
+// The scaled scores together with the largest score of every row (fed to ParamSpMM.*_spmm_softmax, which then needs
+// no separate softmax pass).  rows: number of matrix rows (the row-split format does not say).
+static std::vector<Tensor> sddmm_scaled_rowmax(int fmt, const Tensor &A, const Tensor &B, const Tensor &rowPtr,
+                                               const Tensor &colIdx, const Tensor &values, const Tensor *target_row,
+                                               long rows, int blkWarpNum)
+{
+    check_sddmm_args(fmt, A, B, rowPtr, colIdx, values, target_row, 1, blkWarpNum);
+    TORCH_CHECK(rows >= 0 && rows <= 0x7fffffffL, "rows out of range");
+    pspglue::DeviceGuard guard(A.device());
+    auto out = torch::empty_like(values);
+    auto row_max = torch::empty({rows}, values.options());
+    const int nseg = (int)rowPtr.size(0) - 1, K = (int)A.size(1);
+    psp_stream_t s = stream_of(A);
+    if (fmt == 0) {
+        TORCH_CHECK(rows == nseg, "rows must equal the number of CSR rows");
+        ok(psp_sddmm_csr_rowmax_f32(ip(rowPtr), ip(colIdx), fp(A), fp(B), fp(values), fpw(out), fpw(row_max), nseg, K,
+                                    blkWarpNum, s));
+    } else {
+        ok(psp_sddmm_csr_split_rowmax_f32(ip(rowPtr), ip(colIdx), ip(*target_row), fp(A), fp(B), fp(values), fpw(out),
+                                          fpw(row_max), nseg, (int)rows, K, blkWarpNum, s));
+    }
+    return {out, row_max};
+}
+static std::vector<Tensor> csr_sddmm_scaled_rowmax(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values,
+                                                   int blkWarpNum)
+{
+    return sddmm_scaled_rowmax(0, A, B, rowPtr, colIdx, values, nullptr, rowPtr.size(0) - 1, blkWarpNum);
+}
+static std::vector<Tensor> csr_split_sddmm_scaled_rowmax(Tensor A, Tensor B, Tensor rowPtr_split, Tensor colIdx,
+                                                         Tensor values, Tensor target_row, long rows, int blkWarpNum)
+{
+    return sddmm_scaled_rowmax(1, A, B, rowPtr_split, colIdx, values, &target_row, rows, blkWarpNum);
+}
+
 // ---- *_profile twins (SDDMM/sddmm.cpp:338-661): int GFLOP/s = 2*nnz*K / t -------------------------------
 static int profile_impl(int fmt, const Tensor &A, const Tensor &B, const Tensor &rowPtr, const Tensor &colIdx,
                         const Tensor &values, const Tensor *target_row, long nnz, int CF, int blkWarpNum)
@@ -215,5 +249,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     // additions of this build
     m.def("csr_sddmm_scaled", &csr_sddmm_scaled, "values[p] * <A[row], B[col]>");
     m.def("csr_split_sddmm_scaled", &csr_split_sddmm_scaled, "values[p] * <A[row], B[col]> on the row-split format");
+    m.def("csr_sddmm_scaled_rowmax", &csr_sddmm_scaled_rowmax, "[values[p] * <A[row], B[col]>, largest score of every row]");
+    m.def("csr_split_sddmm_scaled_rowmax", &csr_split_sddmm_scaled_rowmax,
+          "the same on the row-split format: (A, B, rowPtr_split, colIdx, values, target_row, rows, blkWarpNum)");
     m.def("segment_softmax", &segment_softmax, "softmax over the stored entries of each CSR row");
 }

@@ -26,6 +26,42 @@ static Tensor bcsr_split_spmm(Tensor input, Tensor rowPtr_bcsr_split, Tensor col
     return spmm_new(3, input, rowPtr_bcsr_split, colIdx, values, &target_row, CF, blkWarpNum);
 }
 
+// ---- softmax-weighted SpMM (an addition of this build): Y = softmax_rows(e) * X without a separate softmax pass.
+// e: scores in CSR order, row_max: an upper bound of every row's scores (ParamSDDMM.*_sddmm_scaled_rowmax delivers
+// the maximum).
+static Tensor spmm_softmax(int fmt, const Tensor &X, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &e,
+                           const Tensor &row_max, const Tensor *target_row, int CF, int blkWarpNum)
+{
+    check_spmm_args(fmt, X, rowPtr, colIdx, e, target_row);
+    need_gpu(row_max, "row_max");
+    need_f32(row_max, "row_max", 1);
+    TORCH_CHECK(row_max.size(0) >= X.size(0) || fmt == 0, "row_max must hold one value per matrix row");
+    TORCH_CHECK(X.size(1) % 4 == 0 && CF <= 4, "softmax-weighted SpMM needs a width that is a multiple of 4 and CF <= 4");
+    pspglue::DeviceGuard guard(X.device());
+    auto Y = torch::empty_like(X);
+    const int nseg = (int)rowPtr.size(0) - 1, N = (int)X.size(1), rows_out = (int)Y.size(0);
+    if (N == 0 || rows_out == 0) return Y;
+    if (fmt == 0) {
+        TORCH_CHECK(row_max.size(0) >= nseg, "row_max must hold one value per matrix row");
+        ok(psp_spmm_csr_softmax_f32(ip(rowPtr), ip(colIdx), fp(e), fp(row_max), fp(X), fpw(Y), nseg, N, rows_out, CF,
+                                    blkWarpNum, stream_of(X)));
+    } else {
+        auto row_sum = torch::empty({(long)rows_out}, X.options());
+        ok(psp_spmm_csr_split_softmax_f32(ip(rowPtr), ip(colIdx), fp(e), ip(*target_row), fp(row_max), fpw(row_sum), fp(X),
+                                          fpw(Y), nseg, N, rows_out, CF, blkWarpNum, stream_of(X)));
+    }
+    return Y;
+}
+static Tensor csr_spmm_softmax(Tensor X, Tensor rowPtr, Tensor colIdx, Tensor e, Tensor row_max, int CF, int blkWarpNum)
+{
+    return spmm_softmax(0, X, rowPtr, colIdx, e, row_max, nullptr, CF, blkWarpNum);
+}
+static Tensor csr_split_spmm_softmax(Tensor X, Tensor rowPtr_split, Tensor colIdx, Tensor e, Tensor row_max,
+                                     Tensor target_row, int CF, int blkWarpNum)
+{
+    return spmm_softmax(1, X, rowPtr_split, colIdx, e, row_max, &target_row, CF, blkWarpNum);
+}
+
 // ---- *_profile twins (SpMM/SpMM.cpp:482-889): mean of 200 launches, int GFLOP/s = 2*nnz*N / t ----------
 static int profile_impl(int fmt, const Tensor &X, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values,
                         const Tensor *target_row, long nnz, int CF, int blkWarpNum)
@@ -179,6 +215,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("gespmm_compute", &gespmm_compute, "row-caching CSR SpMM baseline (one wavefront per row)");
     m.def("gespmm_profile", &gespmm_profile, "GFLOP/s of the row-caching baseline");
     // additions of this build
+    m.def("csr_spmm_softmax", &csr_spmm_softmax, "softmax_rows(e) * X: (X, rowPtr, colIdx, e, row_max, CF, blkWarpNum)");
+    m.def("csr_split_spmm_softmax", &csr_split_spmm_softmax,
+          "the same on the row-split format: (X, rowPtr_split, colIdx, e, row_max, target_row, CF, blkWarpNum)");
     m.def("spmm_time_ms", &spmm_time_ms, "mean ms per launch: (fmt, X, rowPtr, colIdx, val, target_row|None, CF, bw, warmup, iters)");
     m.def("vendor_spmm_time_ms", &vendor_spmm_time_ms, "mean ms per rocSPARSE SpMM: (format, X, idx_a, idx_b, val, warmup, iters)");
     m.def("spmm_plan", &spmm_plan, "how (N, CF, blkWarpNum) maps onto the wave64 kernel");

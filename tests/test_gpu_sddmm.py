@@ -184,3 +184,85 @@ def test_full_size_headline_graph_properties(oracle):
     a_sorted = eh[np.lexsort((eh, rows))]
     b_sorted = got[np.lexsort((got, rows))]
     assert np.array_equal(a_sorted, b_sorted)
+
+
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("N,CF,bw", [(32, 1, 8), (16, 1, 4), (64, 2, 4), (128, 4, 8), (96, 3, 4)])
+def test_fused_attention_pipeline_matches_oracle(oracle, split, N, CF, bw):
+    """Scaled SDDMM with row maxima, then the softmax-weighted SpMM, against the oracle's three separate steps
+    (scaled scores -> segment softmax -> SpMM).  Hub row cut over many wavefronts, empty rows, rows shorter than a
+    lane group, scores spread widely (standard normal inputs of width 24, not normalised)."""
+    from paramspmm_ae_amd import _capi
+    from gpu_util import Formats, assert_close, dev, stream
+
+    rowPtr, colIdx, val = random_csr(3001, 9, 21, empty_frac=0.15, hub=(11, 2600), values="uniform")
+    F = Formats(oracle, rowPtr, colIdx, val)
+    n, K = F.n, 24
+    rng = np.random.default_rng(N)
+    A = rng.standard_normal((n, K)).astype(np.float32)
+    B = rng.standard_normal((n, K)).astype(np.float32)
+    H = rng.standard_normal((n, N)).astype(np.float32)
+    e_want = oracle.sddmm_csr(rowPtr, colIdx, A, B) * val
+    w_want = oracle.segment_softmax(rowPtr, e_want)
+    y_want = oracle.spmm_csr(rowPtr, colIdx, w_want, H)
+    scale = oracle.spmm_csr(rowPtr, colIdx, w_want, np.abs(H))
+    m_want = np.full(n, -3.402823466e+38, np.float32)
+    rows = np.repeat(np.arange(n), np.diff(rowPtr))
+    np.maximum.at(m_want, rows, e_want)
+
+    L, p = _capi.lib, _capi.ptr
+    Ad, Bd, Hd = dev(A), dev(B), dev(H)
+    e = torch.full((F.nnz,), float("nan"), device="cuda")
+    m = torch.full((n,), float("nan"), device="cuda")
+    Y = torch.full((n, N), float("nan"), device="cuda")
+    d = F.d
+    if split:
+        _capi.check(L.psp_sddmm_csr_split_rowmax_f32(p(d["rps"]), p(d["colIdx"]), p(d["tr"]), p(Ad), p(Bd), p(d["val"]), p(e),
+                                                     p(m), F.tr.size, n, K, bw, stream()))
+        row_sum = torch.full((n,), float("nan"), device="cuda")
+        _capi.check(L.psp_spmm_csr_split_softmax_f32(p(d["rps"]), p(d["colIdx"]), p(e), p(d["tr"]), p(m), p(row_sum), p(Hd),
+                                                     p(Y), F.tr.size, N, n, CF, bw, stream()))
+    else:
+        _capi.check(L.psp_sddmm_csr_rowmax_f32(p(d["rowPtr"]), p(d["colIdx"]), p(Ad), p(Bd), p(d["val"]), p(e), p(m), n, K,
+                                               bw, stream()))
+        _capi.check(L.psp_spmm_csr_softmax_f32(p(d["rowPtr"]), p(d["colIdx"]), p(e), p(m), p(Hd), p(Y), n, N, n, CF, bw,
+                                               stream()))
+    torch.cuda.synchronize()
+    # the inputs are not normalised: a dot product may cancel, so the relative term is taken against sum |a||b|
+    e_scale = oracle.sddmm_csr(rowPtr, colIdx, np.abs(A), np.abs(B)) * np.abs(val)
+    assert_close(e, e_want, rtol=1e-5, atol=1e-6, what="scores", scale=e_scale)
+    # the row maximum is one of the scores: compare with the device's own scores exactly, with the oracle's loosely
+    m_dev = np.full(n, -3.402823466e+38, np.float32)
+    np.maximum.at(m_dev, rows, e.cpu().numpy())
+    assert np.array_equal(m.cpu().numpy(), m_dev)
+    assert_close(m, m_want, rtol=1e-4, atol=1e-5, what="row maxima")
+    # the weights inherit the rounding of the scores (|d exp(e)| = exp(e) |de|, scores of magnitude up to ~10)
+    assert_close(Y, y_want, rtol=1e-4, atol=1e-5, what="softmax-weighted product", scale=scale)
+
+
+def test_fused_attention_modules_match_unfused():
+    """ParamSDDMM.*_scaled_rowmax + ParamSpMM.*_spmm_softmax against scaled SDDMM -> segment_softmax -> SpMM on an
+    R-MAT graph (2^16 nodes), both layouts."""
+    import ParamSDDMM
+    import ParamSpMM
+    from paramspmm_ae_amd import synth
+    from paramspmm_ae_amd.graph_input import graph_input
+
+    r, c, n = synth.rmat(16, 8 << 16, seed=3)
+    rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+    g = graph_input("t", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val)
+    cd = g.csr_data
+    rp, ci, v, rps, tr = (cd.on_device(k, "cuda") for k in ("rowPtr", "colIdx", "val", "rowPtr_split", "target_row"))
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    X = torch.nn.functional.normalize(torch.randn(n, 32, device="cuda", generator=gen), dim=1).contiguous()
+    H = torch.randn(n, 32, device="cuda", generator=gen)
+    a = ParamSDDMM.segment_softmax(rp, ParamSDDMM.csr_sddmm_scaled(X, X, rp, ci, v, 8))
+    want = ParamSpMM.csr_spmm(H, rp, ci, a, 1, 8)
+    e, m = ParamSDDMM.csr_sddmm_scaled_rowmax(X, X, rp, ci, v, 8)
+    got = ParamSpMM.csr_spmm_softmax(H, rp, ci, e, m, 1, 8)
+    torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-6)
+    e, m = ParamSDDMM.csr_split_sddmm_scaled_rowmax(X, X, rps, ci, v, tr, n, 8)
+    got = ParamSpMM.csr_split_spmm_softmax(H, rps, ci, e, m, tr, 1, 8)
+    torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-6)
