@@ -456,7 +456,7 @@ def main():
     by_symbol = {}
     for r in per_dim:
         plan = _capi.spmm_plan(r["dim"], r["CF"], r["blkWarpNum"])
-        sym = "psp_spmm_kernel<%d, %d, %d, %d, %s>" % (plan["coarsen"], plan["vec"], plan["unroll"],
+        sym = "psp_spmm_kernel<%d, %d, %d, %d, %s, false>" % (plan["coarsen"], plan["vec"], plan["unroll"],
                                                        2 if r["format"].startswith("bcsr") else 1,
                                                        "true" if "split" in r["format"] else "false")
         r["kernel"] = sym
