@@ -222,17 +222,17 @@ def bench_sddmm(args):
 
 
 def bench_gcn(args):
-    """GCN and GIN training epochs (BASELINE.json configs[4]): 5 layers, hidden 16 / 32 / 128, 16 classes, random
+    """GCN, GIN and AGNN training epochs (BASELINE.json configs[4]): 5 layers, hidden 16 / 32 / 128, 16 classes, random
     features and weights, forward + backward + Adam, on the 1M-node stochastic block model in community order
     (C5) and randomly permuted (C5p).  --steps is the number of timed epochs (the reference times 200)."""
     from paramspmm_ae_amd import GNN
 
-    out = {"metric": "GCN / GIN epoch ms (5 layers, fwd+bwd+Adam), SBM 1M nodes", "unit": "ms per epoch", "n_gpus": 1,
+    out = {"metric": "GCN / GIN / AGNN epoch ms (5 layers, fwd+bwd+Adam), SBM 1M nodes", "unit": "ms per epoch", "n_gpus": 1,
            "steps": args.steps, "warmup": 1, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
            "dtype": "f32", "data": "synthetic", "config": {"workload": "C5 / C5p, hidden 16 32 128, 16 classes"}, "epochs": []}
     graphs = [args.graph] if args.graph in ("C5", "C5p", "C1") else ["C5", "C5p"]
     for g in graphs:
-        for net in ("GCN", "GIN"):
+        for net in ("GCN", "GIN", "AGNN"):
             argv = ["--net", net, "--synthetic", g, "--hidden_list", "16", "32", "128", "--num_classes", "16",
                     "--num_features", "32", "--num_epoches", str(args.steps)]
             res = GNN.main(argv)
