@@ -152,19 +152,32 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
     };
     const bool want_max = !BCSR && row_max != nullptr;  // uniform
 
+    // lane `sub` of the group picks up entry base+sub (column index and, where the format has one, its value); the
+    // next chunk's are requested before the current chunk is worked on
+    auto fetch = [&](int base, int &c_out, float (&g_out)[NR]) {
+        const int q = base + sub;
+        const int qq = q < b0 ? q : b0 - 1;
+        c_out = colIdx[qq];
+        if constexpr (BCSR) {
+            const psp_f32x2 t = ((const psp_f32x2 *)val)[qq];
+            g_out[0] = t[0];
+            g_out[1] = t[1];
+        } else {
+            g_out[0] = SCALE ? val[qq] : 1.0f;
+        }
+    };
+    int c_cur;
+    float gate[NR];
+    fetch(a0, c_cur, gate);
+
     for (int base = a0; base < b0; base += L) {
         const int p = base + sub;
         const bool ok = p < b0;
-        const int pp = ok ? p : b0 - 1;
-        const int c_cur = colIdx[pp];
-        float gate[NR];
-        if constexpr (BCSR) {
-            const psp_f32x2 t = ((const psp_f32x2 *)val)[pp];
-            gate[0] = t[0];
-            gate[1] = t[1];
-        } else {
-            gate[0] = SCALE ? val[pp] : 1.0f;
-        }
+        int c_nxt = 0;
+        float gate_nxt[NR];
+#pragma unroll
+        for (int r = 0; r < NR; r++) gate_nxt[r] = 0.0f;
+        if (base + L < b0) fetch(base + L, c_nxt, gate_nxt);
         float res[NR];
 #pragma unroll
         for (int r = 0; r < NR; r++) res[r] = 0.0f;
@@ -231,6 +244,9 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
                 out[p] = SCALE ? res[0] * gate[0] : res[0];
             }
         }
+        c_cur = c_nxt;
+#pragma unroll
+        for (int r = 0; r < NR; r++) gate[r] = gate_nxt[r];
     }
     if (want_max) emit_row_max(mykey);
 }
