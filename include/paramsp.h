@@ -72,6 +72,12 @@ int psp_bcsr_count(const int *rowPtr, const int *colIdx, int nrows, int ncols);
 int psp_bcsr_build(const int *rowPtr, const int *colIdx, const float *val, int nrows, int ncols,
                    int *rowPtr_b, int *colIdx_b, float *val_b);
 
+/* Blocks of R x 1 for any R in 1..8 (graph_input.py:243-266 with blk_size = R; the reference has kernels for R = 3
+ * besides 2): same block order as above, val_b is [nblk, R], rowPtr_b has ceil(nrows/R)+1 entries. */
+int psp_vbsr_count(const int *rowPtr, const int *colIdx, int nrows, int ncols, int R);
+int psp_vbsr_build(const int *rowPtr, const int *colIdx, const float *val, int nrows, int ncols, int R,
+                   int *rowPtr_b, int *colIdx_b, float *val_b);
+
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: PCSR index construction on the GPU, the twins of the host builders above (same outputs, bit for
  * bit).  The reference builds on the host only (SpMM/SpMM.cpp:15-75, graph_input.py:243-274).  Each builder is
@@ -163,6 +169,15 @@ int psp_spmm_bcsr_f32(const int *rowPtr_b, const int *colIdx_b, const float *val
 int psp_spmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b,
                             const int *target_row, const float *X, float *Y, int Sb, int N, int rows_out,
                             int CF, int blkWarpNum, psp_stream_t stream);
+
+/* ParamSpMM.vec_spmm / vec_split_spmm, SpMM/SpMM.cpp:339-480 -> SpMM_kernel.cu:420-562, 1653-1972: blocks of
+ * vec_size x 1 (val_b is [nblk, vec_size]); the reference instantiates vec_size 3 only, this library 3 and, through the
+ * 2x1 kernels, 2.  rows_out >= vec_size * Mb.  CF 7 and 8 with vec_size 3 exceed the register file and run slowly. */
+int psp_spmm_vec_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *X, float *Y, int Mb,
+                     int N, int rows_out, int vec_size, int CF, int blkWarpNum, psp_stream_t stream);
+int psp_spmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b, const int *target_row,
+                           const float *X, float *Y, int Sb, int N, int rows_out, int vec_size, int CF,
+                           int blkWarpNum, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: SDDMM  out[p] = <A[row(p),:], B[col(p),:]>, fp32, NOT scaled by the stored values (the reference

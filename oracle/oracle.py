@@ -44,6 +44,7 @@ def lib():
         _lib.orc_split_csr.restype = ctypes.c_int
         _lib.orc_split_csr_par.restype = ctypes.c_int
         _lib.orc_bcsr_build.restype = ctypes.c_int
+        _lib.orc_vbsr_build.restype = ctypes.c_int
     return _lib
 
 
@@ -101,6 +102,34 @@ def bcsr_build(rowPtr, colIdx, val, ncols=None):
     vb = np.empty((nblk, 2), np.float32)
     lib().orc_bcsr_build(_pi(rowPtr), _pi(colIdx), _pf(val), n, int(ncols), _pi(rpb), _pi(cib), _pf(vb))
     return rpb, cib, vb
+
+
+def vbsr_build(rowPtr, colIdx, val, R, ncols=None):
+    """graph_input.py:243-266 with blk_size = R -> (rowPtr_b, colIdx_b, val_b[nblk,R]) in SciPy tobsr((R,1)) order."""
+    rowPtr, colIdx, val = _i32(rowPtr), _i32(colIdx), _f32(val)
+    n = rowPtr.size - 1
+    if ncols is None:
+        ncols = max(n, int(colIdx.max()) + 1 if colIdx.size else 0)
+    nblk = lib().orc_vbsr_build(_pi(rowPtr), _pi(colIdx), _pf(val), n, int(ncols), int(R), None, None, None)
+    rpb = np.empty((n + R - 1) // R + 1, np.int32)
+    cib = np.empty(nblk, np.int32)
+    vb = np.empty((nblk, R), np.float32)
+    lib().orc_vbsr_build(_pi(rowPtr), _pi(colIdx), _pf(val), n, int(ncols), int(R), _pi(rpb), _pi(cib), _pf(vb))
+    return rpb, cib, vb
+
+
+def spmm_vec(rowPtr_b, colIdx_b, val_b, X, target_row=None, rows_out=None):
+    """SpMM/SpMM_kernel.cu:1653-1972: R x 1 blocks (R = val_b.shape[1]); row-split when target_row is given."""
+    rowPtr_b, colIdx_b, val_b, X = _i32(rowPtr_b), _i32(colIdx_b), _f32(val_b), _f32(X)
+    R = val_b.shape[1]
+    S = rowPtr_b.size - 1
+    nbr = S if target_row is None else (int(np.max(target_row)) + 1 if S else 0)
+    if rows_out is None:
+        rows_out = max(R * nbr, (X.shape[0] + R - 1) // R * R)
+    Y = np.empty((rows_out, X.shape[1]), np.float32)
+    tr = None if target_row is None else _pi(_i32(target_row))
+    lib().orc_spmm_vec(_pi(rowPtr_b), _pi(colIdx_b), _pf(val_b), tr, _pf(X), _pf(Y), S, X.shape[1], rows_out, R)
+    return Y
 
 
 def genmask(rowPtr_b, rowPtr, val_b, nnz):

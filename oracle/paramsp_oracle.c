@@ -18,9 +18,14 @@
  *   orc_bcsr_build        scipy.sparse csr.tobsr((2,1)) (the routine the
  *                         reference itself calls), the hand case
  *                         rows {0:[1,5],1:[0,5,7]}, pubmed block counts
+ *   orc_vbsr_build        scipy.sparse csr.tobsr((R,1)) for R = 3, 4; equals
+ *                         orc_bcsr_build for R = 2
  *   orc_genmask           brute force + permutation-within-row invariant
  *   orc_spmm_*            torch.sparse.mm on CPU (the reference's own
  *                         checker), fp64 dense product, X = ones -> row sums
+ *   orc_spmm_vec          equals orc_spmm_bcsr(_split) for R = 2; for R = 3 the
+ *                         CSR product of the same matrix (entry by entry the
+ *                         same FMA chain), fp64 dense product
  *   orc_sddmm_*           fp64 gathered dot products, A = B = ones -> K
  *   orc_segment_softmax   closed form in fp64 (no reference counterpart)
  */
@@ -101,6 +106,42 @@ ORC_API int orc_bcsr_build(const int *rowPtr, const int *colIdx, const float *va
                     nblk++;
                 }
                 if (colIdx_b) val_b[2 * (size_t)slot[c] + k] += val[p];
+            }
+        }
+        if (rowPtr_b) rowPtr_b[t + 1] = nblk;
+    }
+    free(slot);
+    return nblk;
+}
+
+/* Blocks of R x 1 for any R (graph_input.py:243-266 with blk_size = R; the reference instantiates its kernels for
+ * R = 3 besides the 2 x 1 case above).  Same first-encounter block order: SciPy's csr_tobsr walks the R rows of a
+ * block-row in turn and opens a block at the first entry of a column.  val_b is [nblk, R].                        */
+ORC_API int orc_vbsr_build(const int *rowPtr, const int *colIdx, const float *val,
+                           int nrows, int ncols, int R,
+                           int *rowPtr_b, int *colIdx_b, float *val_b)
+{
+    int nbr = (nrows + R - 1) / R;
+    int *slot = (int *)malloc(sizeof(int) * (size_t)(ncols > 0 ? ncols : 1));
+    for (int c = 0; c < ncols; c++) slot[c] = -1;
+    int nblk = 0;
+    if (rowPtr_b) rowPtr_b[0] = 0;
+    for (int t = 0; t < nbr; t++) {
+        int first = nblk;
+        for (int k = 0; k < R; k++) {
+            int r = R * t + k;
+            if (r >= nrows) break;
+            for (int p = rowPtr[r]; p < rowPtr[r + 1]; p++) {
+                int c = colIdx[p];
+                if (slot[c] < first) {
+                    slot[c] = nblk;
+                    if (colIdx_b) {
+                        colIdx_b[nblk] = c;
+                        for (int q = 0; q < R; q++) val_b[(size_t)R * nblk + q] = 0.0f;
+                    }
+                    nblk++;
+                }
+                if (colIdx_b) val_b[(size_t)R * slot[c] + k] += val[p];
             }
         }
         if (rowPtr_b) rowPtr_b[t + 1] = nblk;
@@ -201,6 +242,27 @@ ORC_API void orc_spmm_bcsr_split(const int *rowPtr_bs, const int *colIdx_b, cons
             Y[(size_t)(2 * t) * N + c] += r0;
             Y[(size_t)(2 * t + 1) * N + c] += r1;
         }
+    }
+}
+
+/* SpMM/SpMM_kernel.cu:1653-1770 (vec_spmm) and 1772-1972 (vec_split_spmm): R x 1 blocks, the 2 x 1 rule for
+ * every one of the R entries of a block (a zero entry adds nothing, 1693-1699).  target_row = NULL: plain format
+ * (segment s is block-row s).  rows_out >= R * (number of block-rows).                                             */
+ORC_API void orc_spmm_vec(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const int *target_row,
+                          const float *X, float *Y, int S, int N, int rows_out, int R)
+{
+    memset(Y, 0, sizeof(float) * (size_t)rows_out * N);
+    for (int s = 0; s < S; s++) {
+        int t = target_row ? target_row[s] : s;
+        for (int c = 0; c < N; c++)
+            for (int q = 0; q < R; q++) {
+                float r = 0.0f;
+                for (int p = rowPtr_b[s]; p < rowPtr_b[s + 1]; p++) {
+                    float v = val_b[(size_t)R * p + q];
+                    if (v != 0.0f) r = fmaf(v, X[(size_t)colIdx_b[p] * N + c], r);
+                }
+                Y[(size_t)(R * t + q) * N + c] += r;
+            }
     }
 }
 

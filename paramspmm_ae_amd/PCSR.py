@@ -96,8 +96,8 @@ _SDDMM = {(False, False): "csr_sddmm", (True, False): "csr_split_sddmm", (False,
 class pcsr_spmm(object):
     def __init__(self, graph, vec_size, if_split, mtx_nodes=None, mtx_edges=None, rowPtr=None, colIdx=None,
                  val=None, target_row=None, CF=1, blkWarpNum=4, device="cuda"):
-        if vec_size not in (1, 2):
-            raise ValueError("this build has vec_size 1 (CSR) and 2 (2x1 BCSR)")
+        if vec_size not in (1, 2, 3):
+            raise ValueError("this build has vec_size 1 (CSR), 2 (2x1 BCSR) and 3 (3x1 blocks, SpMM only)")
         if_split = bool(if_split)
         self.mask = None
         if graph is None:
@@ -122,6 +122,8 @@ class pcsr_spmm(object):
         else:
             self.mtx_nodes, self.mtx_edges = graph.mtx_nodes, graph.mtx_edges
             fmt = graph.csr_data if vec_size == 1 else graph.bcsr_data
+            if vec_size != 1 and getattr(graph, "blk_size", 2) != vec_size:
+                raise ValueError("the graph was loaded with blk_size %d, not %d" % (getattr(graph, "blk_size", 2), vec_size))
             # one device copy per format, shared by every operator built on this graph
             self.rowPtr = fmt.on_device("rowPtr_split" if if_split else "rowPtr", device)
             self.colIdx = fmt.on_device("colIdx", device)
@@ -139,6 +141,12 @@ class pcsr_spmm(object):
     def _key(self):
         return (self.if_split, self.vec_size != 1)
 
+    def _spmm_name(self):
+        # vec_size 3 goes to the generic-block operators (PCSR.py:227-239)
+        if self.vec_size == 3:
+            return "vec_split_spmm" if self.if_split else "vec_spmm"
+        return _SPMM[self._key()]
+
     def _sparse_args(self, val=None):
         args = [self.rowPtr, self.colIdx, self.val if val is None else val]
         if self.if_split:
@@ -146,7 +154,7 @@ class pcsr_spmm(object):
         return args
 
     def _spmm(self, X, val=None, CF=None, blkWarpNum=None):
-        fn = getattr(SpMM, _SPMM[self._key()])
+        fn = getattr(SpMM, self._spmm_name())
         return fn(X, *self._sparse_args(val), self.CF if CF is None else CF,
                   self.blkWarpNum if blkWarpNum is None else blkWarpNum)
 
@@ -176,6 +184,9 @@ class pcsr_spmm(object):
 
     # ---- SDDMM ------------------------------------------------------------------------------
     def _sddmm(self, A, B, blkWarpNum):
+        if self.vec_size == 3:
+            raise NotImplementedError("SDDMM on 3x1 blocks is not part of this build (the reference's vec_sddmm "
+                                      "kernels are never exercised and index their shared memory wrongly)")
         fn = getattr(SDDMM, _SDDMM[self._key()])
         CF = (A.size(1) + 31) // 32
         return fn(A, B, *self._sparse_args(), CF, blkWarpNum)
@@ -196,12 +207,16 @@ class pcsr_spmm(object):
     def forward(self, H, w):
         if H is None or w is None:
             raise ValueError("H and w should be given")
+        if self.vec_size == 3:
+            raise NotImplementedError("the fused GCN operators exist for vec_size 1 and 2 (SpCONV/SpCONV.cpp:498-511)")
         fn = getattr(SpCONV, _SPMM[self._key()] + "_forward")
         return fn(H, w, *self._sparse_args(), self.CF, self.blkWarpNum)
 
     def backward(self, d_output, H, w):
         if d_output is None or H is None:
             raise ValueError("d_output and H should be given")
+        if self.vec_size == 3:
+            raise NotImplementedError("the fused GCN operators exist for vec_size 1 and 2 (SpCONV/SpCONV.cpp:498-511)")
         fn = getattr(SpCONV, _SPMM[self._key()] + "_backward")
         d_input, d_weight = fn(d_output, H, w, *self._sparse_args(), self.CF, self.blkWarpNum)
         return d_input, d_weight
@@ -211,7 +226,7 @@ class pcsr_spmm(object):
         """GFLOP/s (int) of this variant with an explicit (CF, blkWarpNum) (PCSR.py:433-505)."""
         assert torch.cuda.is_available()
         X = self._dense_input(dim, x)
-        fn = getattr(SpMM, _SPMM[self._key()] + "_profile")
+        fn = getattr(SpMM, self._spmm_name() + "_profile")
         args = self._sparse_args()
         if self.vec_size != 1:
             args.append(self.mtx_edges)  # blocked twins take the true nnz before CF
@@ -248,6 +263,8 @@ class pcsr_spmm(object):
 
     def time_ms(self, X, CF=None, blkWarpNum=None, warmup=5, iters=20):
         """Mean milliseconds per SpMM launch (an addition of this build; used by the sweep harness)."""
+        if self.vec_size == 3:
+            raise NotImplementedError("time_ms covers the four decider formats; use cf_warpnum_profiling for 3x1 blocks")
         fmt = (1 if self.if_split else 0) + (2 if self.vec_size != 1 else 0)
         return SpMM.spmm_time_ms(fmt, X, self.rowPtr, self.colIdx, self.val, self.target_row,
                                  self.CF if CF is None else CF, self.blkWarpNum if blkWarpNum is None else blkWarpNum,

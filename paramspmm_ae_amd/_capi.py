@@ -51,6 +51,10 @@ SIGNATURES = {
     "psp_bcsr_offsets_dev": [_vp, _vp, _i, _vp, _vp, _i, _vp, _vp],
     "psp_bcsr_fill_dev": [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp],
     "psp_check_index_dev": [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp],
+    "psp_vbsr_count": [_vp, _vp, _i, _i, _i],
+    "psp_vbsr_build": [_vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp],
+    "psp_spmm_vec_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "psp_spmm_vec_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "psp_genmask": [_vp, _vp, _vp, _i, _i, _vp, _vp],
     "psp_spmm_csr_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "psp_spmm_csr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],

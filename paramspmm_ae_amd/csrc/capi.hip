@@ -476,31 +476,30 @@ PSP_EXPORT int psp_split_csr_par(const int *rowPtr, const int *row_split_offset,
 // host: BCSR 2x1 in first-encounter block order (what SciPy's tobsr produces, graph_input.py:245-256)
 // ------------------------------------------------------------------------------------------------
 static int bcsr_walk(const int *rowPtr, const int *colIdx, const float *val, int nrows, int ncols,
-                     int *rowPtr_b, int *colIdx_b, float *val_b)
+                     int *rowPtr_b, int *colIdx_b, float *val_b, int R = 2)
 {
-    const int nbr = (nrows + 1) / 2;
+    const int nbr = (nrows + R - 1) / R;
     std::vector<int> slot((size_t)std::max(ncols, 1), -1);
     long long nblk = 0;
     if (rowPtr_b) rowPtr_b[0] = 0;
     for (int t = 0; t < nbr; t++) {
         const long long first = nblk;
-        for (int k = 0; k < 2; k++) {
-            const int r = 2 * t + k;
+        for (int k = 0; k < R; k++) {
+            const int r = R * t + k;
             if (r >= nrows) break;
             for (int p = rowPtr[r]; p < rowPtr[r + 1]; p++) {
                 const int c = colIdx[p];
                 if (c < 0 || c >= ncols) return psp_fail(PSP_ERR_ARG, "bcsr: column %d out of range at entry %d", c, p);
                 if (slot[c] < first) {
-                    if (nblk >= 0x7fffffffLL) return psp_fail(PSP_ERR_RANGE, "bcsr: block count overflows int32");
+                    if (nblk >= 0x7fffffffLL / R) return psp_fail(PSP_ERR_RANGE, "bcsr: block count overflows int32");
                     slot[c] = (int)nblk;
                     if (colIdx_b) {
                         colIdx_b[nblk] = c;
-                        val_b[2 * nblk] = 0.0f;
-                        val_b[2 * nblk + 1] = 0.0f;
+                        for (int q = 0; q < R; q++) val_b[(size_t)R * nblk + q] = 0.0f;
                     }
                     nblk++;
                 }
-                if (colIdx_b) val_b[2 * (size_t)slot[c] + k] += val[p];
+                if (colIdx_b) val_b[(size_t)R * slot[c] + k] += val[p];
             }
         }
         if (rowPtr_b) rowPtr_b[t + 1] = (int)nblk;
@@ -526,6 +525,28 @@ PSP_EXPORT int psp_bcsr_build(const int *rowPtr, const int *colIdx, const float 
         return 0;
     }
     return bcsr_walk(rowPtr, colIdx, val, nrows, ncols, rowPtr_b, colIdx_b, val_b);
+}
+
+PSP_EXPORT int psp_vbsr_count(const int *rowPtr, const int *colIdx, int nrows, int ncols, int R)
+{
+    PSP_REQUIRE(rowPtr && nrows >= 0 && ncols >= 0, "vbsr_count: bad input");
+    PSP_REQUIRE(R >= 1 && R <= 8, "vbsr_count: block height %d out of range (1..8)", R);
+    PSP_REQUIRE(colIdx || rowPtr[nrows] == 0, "vbsr_count: colIdx is null");
+    return bcsr_walk(rowPtr, colIdx, nullptr, nrows, ncols, nullptr, nullptr, nullptr, R);
+}
+
+PSP_EXPORT int psp_vbsr_build(const int *rowPtr, const int *colIdx, const float *val, int nrows, int ncols, int R,
+                              int *rowPtr_b, int *colIdx_b, float *val_b)
+{
+    PSP_REQUIRE(rowPtr && nrows >= 0 && ncols >= 0 && rowPtr_b, "vbsr_build: bad input");
+    PSP_REQUIRE(R >= 1 && R <= 8, "vbsr_build: block height %d out of range (1..8)", R);
+    const bool empty = rowPtr[nrows] == 0;
+    PSP_REQUIRE(empty || (colIdx && val && colIdx_b && val_b), "vbsr_build: null pointer");
+    if (empty) {
+        for (int t = 0; t <= (nrows + R - 1) / R; t++) rowPtr_b[t] = 0;
+        return 0;
+    }
+    return bcsr_walk(rowPtr, colIdx, val, nrows, ncols, rowPtr_b, colIdx_b, val_b, R);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -578,6 +599,29 @@ PSP_EXPORT int psp_spmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b
 {
     return psp_spmm_launch<2, true>(rowPtr_bs, colIdx_b, val_b, target_row, X, Y, Sb, N, rows_out, CF, blkWarpNum,
                                        (hipStream_t)stream, nullptr, nullptr);
+}
+
+PSP_EXPORT int psp_spmm_vec_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *X, float *Y,
+                                int Mb, int N, int rows_out, int vec_size, int CF, int blkWarpNum, psp_stream_t stream)
+{
+    if (vec_size == 2)
+        return psp_spmm_launch<2, false>(rowPtr_b, colIdx_b, val_b, nullptr, X, Y, Mb, N, rows_out, CF, blkWarpNum,
+                                         (hipStream_t)stream, nullptr, nullptr);
+    PSP_REQUIRE(vec_size == 3, "spmm_vec: block height %d is not built (2 and 3 are)", vec_size);
+    return psp_spmm_launch<3, false>(rowPtr_b, colIdx_b, val_b, nullptr, X, Y, Mb, N, rows_out, CF, blkWarpNum,
+                                     (hipStream_t)stream, nullptr, nullptr);
+}
+
+PSP_EXPORT int psp_spmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b,
+                                      const int *target_row, const float *X, float *Y, int Sb, int N, int rows_out,
+                                      int vec_size, int CF, int blkWarpNum, psp_stream_t stream)
+{
+    if (vec_size == 2)
+        return psp_spmm_launch<2, true>(rowPtr_bs, colIdx_b, val_b, target_row, X, Y, Sb, N, rows_out, CF, blkWarpNum,
+                                        (hipStream_t)stream, nullptr, nullptr);
+    PSP_REQUIRE(vec_size == 3, "spmm_vec_split: block height %d is not built (2 and 3 are)", vec_size);
+    return psp_spmm_launch<3, true>(rowPtr_bs, colIdx_b, val_b, target_row, X, Y, Sb, N, rows_out, CF, blkWarpNum,
+                                    (hipStream_t)stream, nullptr, nullptr);
 }
 
 PSP_EXPORT int psp_sddmm_csr_f32(const int *rowPtr, const int *colIdx, const float *A, const float *B,

@@ -55,7 +55,7 @@ __device__ __forceinline__ float psp_bperm_f(int src_lane, float v)
 
 #define PSP_MAX_WAVES 8  // blkWarpNum is 4 or 8
 
-// NR: rows per stored entry (1 = CSR, 2 = 2x1 BCSR).  SPLIT: segments carry an explicit output row.
+// NR: rows per stored entry (1 = CSR, 2 = 2x1 BCSR, 3 = 3x1 blocks: the reference's vec_spmm, SpMM_kernel.cu:1653-1972).  SPLIT: segments carry an explicit output row.
 // SM (CSR layouts): the stored values are attention scores e; the product is taken with softmax weights,
 //   Y[i] = sum_j exp(e_ij - m_i) X[j] / sum_j exp(e_ij - m_i),   m_i = row_max[i] (any upper bound of the row works,
 // the SDDMM kernel delivers the exact maximum).  The weights are formed on the fly, their sum travels with the
@@ -260,6 +260,12 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
             const psp_f32x2 t_ = ((const psp_f32x2 *)val)[pp_];            \
             v_out[0] = ok_ ? t_[0] : 0.0f;                                 \
             v_out[1] = ok_ ? t_[1] : 0.0f;                                 \
+        } else if constexpr (NR > 2) {                                     \
+            _Pragma("unroll") for (int r_ = 0; r_ < NR; r_++)              \
+            {                                                              \
+                const float t_ = val[(size_t)pp_ * NR + r_];               \
+                v_out[r_] = ok_ ? t_ : 0.0f;                               \
+            }                                                              \
         } else {                                                           \
             const float t_ = val[pp_];                                     \
             v_out[0] = ok_ ? t_ : 0.0f;                                    \

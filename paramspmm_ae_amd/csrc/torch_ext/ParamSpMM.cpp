@@ -112,17 +112,89 @@ static double spmm_time_ms(int fmt, Tensor input, Tensor rowPtr, Tensor colIdx, 
                                  [&] { spmm_into(fmt, Y, input, rowPtr, colIdx, values, tr, CF, blkWarpNum); });
 }
 
-// ---- generic vec_size x 1 blocks ------------------------------------------------------------------------------
-// The reference instantiates vec_spmm only for vec_size 3 (SpMM/SpMM.cpp:352,406) and its decider never
-// selects it (decider.py:63).  The names stay importable; calling them reports what is missing.
-[[noreturn]] static void not_built(const char *what)
+// ---- generic vec_size x 1 blocks (SpMM/SpMM.cpp:339-480, 757-889) --------------------------------------------------
+// The reference instantiates these for vec_size 3 only (SpMM/SpMM.cpp:352,406); values is [nblk, vec_size] and the
+// result has the input's rows rounded up to a multiple of vec_size (SpMM_kernel.cu:427-428).  vec_size 2 is accepted
+// as well and runs the 2x1 kernels.
+static void check_vec_args(const Tensor &X, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values,
+                           const Tensor *target_row)
 {
-    TORCH_CHECK(false, what, " is not part of this build (only the PCSR operators csr/csr_split/bcsr/bcsr_split are)");
+    need_gpu(X, "input");
+    need_gpu(rowPtr, "rowPtr");
+    need_gpu(colIdx, "colIdx");
+    need_gpu(values, "values");
+    need_f32(X, "input", 2);
+    need_i32(rowPtr, "rowPtr");
+    need_i32(colIdx, "colIdx");
+    need_f32(values, "values", 2);
+    TORCH_CHECK(values.size(1) == 2 || values.size(1) == 3, "vec_spmm: values must be [nblk, 3] (or [nblk, 2]); got vec_size ",
+                values.size(1));
+    TORCH_CHECK(values.size(0) == colIdx.size(0), "values and colIdx disagree on the number of stored blocks");
+    check_rowptr_vs(rowPtr, "rowPtr");
+    same_device(X, rowPtr, "vec_spmm");
+    same_device(X, colIdx, "vec_spmm");
+    same_device(X, values, "vec_spmm");
+    const long R = values.size(1), padded = (X.size(0) + R - 1) / R * R;
+    if (target_row) {
+        need_gpu(*target_row, "target_row");
+        need_i32(*target_row, "target_row");
+        same_device(X, *target_row, "vec_spmm");
+        TORCH_CHECK(target_row->size(0) == rowPtr.size(0) - 1, "target_row must have one entry per row segment");
+    } else {
+        TORCH_CHECK(R * (rowPtr.size(0) - 1) <= padded, "rowPtr describes more block-rows than input has");
+    }
 }
-static Tensor vec_spmm(Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_spmm (vec_size 3 blocks)"); }
-static Tensor vec_split_spmm(Tensor, Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_split_spmm (vec_size 3 blocks)"); }
-static int vec_spmm_profile(Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_spmm_profile"); }
-static int vec_split_spmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_split_spmm_profile"); }
+static void vec_into(Tensor &Y, const Tensor &X, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values,
+                     const Tensor *target_row, int CF, int blkWarpNum)
+{
+    const int nseg = (int)rowPtr.size(0) - 1, N = (int)X.size(1), rows_out = (int)Y.size(0), R = (int)values.size(1);
+    if (N == 0 || rows_out == 0) return;
+    if (target_row)
+        ok(psp_spmm_vec_split_f32(ip(rowPtr), ip(colIdx), fp(values), ip(*target_row), fp(X), fpw(Y), nseg, N, rows_out, R,
+                                  CF, blkWarpNum, stream_of(X)));
+    else
+        ok(psp_spmm_vec_f32(ip(rowPtr), ip(colIdx), fp(values), fp(X), fpw(Y), nseg, N, rows_out, R, CF, blkWarpNum,
+                            stream_of(X)));
+}
+static Tensor vec_new(const Tensor &X, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values,
+                      const Tensor *target_row, int CF, int blkWarpNum)
+{
+    check_vec_args(X, rowPtr, colIdx, values, target_row);
+    pspglue::DeviceGuard guard(X.device());
+    const long R = values.size(1);
+    auto Y = torch::empty({(X.size(0) + R - 1) / R * R, X.size(1)}, X.options());
+    vec_into(Y, X, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
+    return Y;
+}
+static int vec_profile(const Tensor &X, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values,
+                       const Tensor *target_row, long nnz, int CF, int blkWarpNum)
+{
+    check_vec_args(X, rowPtr, colIdx, values, target_row);
+    pspglue::DeviceGuard guard(X.device());
+    const long R = values.size(1);
+    auto Y = torch::empty({(X.size(0) + R - 1) / R * R, X.size(1)}, X.options());
+    const float ms = time_launches((hipStream_t)stream_of(X), pspglue::kProfileWarmup, pspglue::kProfileIters,
+                                   [&] { vec_into(Y, X, rowPtr, colIdx, values, target_row, CF, blkWarpNum); });
+    return gflops(2.0 * (double)nnz * (double)X.size(1), ms);
+}
+static Tensor vec_spmm(Tensor X, Tensor rowPtr, Tensor colIdx, Tensor values, int CF, int blkWarpNum)
+{
+    return vec_new(X, rowPtr, colIdx, values, nullptr, CF, blkWarpNum);
+}
+static Tensor vec_split_spmm(Tensor X, Tensor rowPtr, Tensor colIdx, Tensor values, Tensor target_row, int CF, int blkWarpNum)
+{
+    return vec_new(X, rowPtr, colIdx, values, &target_row, CF, blkWarpNum);
+}
+// the true non-zero count comes before CF, as for the bcsr twins (SpMM/SpMM.cpp:757-765)
+static int vec_spmm_profile(Tensor X, Tensor rowPtr, Tensor colIdx, Tensor values, int nnz, int CF, int blkWarpNum)
+{
+    return vec_profile(X, rowPtr, colIdx, values, nullptr, nnz, CF, blkWarpNum);
+}
+static int vec_split_spmm_profile(Tensor X, Tensor rowPtr, Tensor colIdx, Tensor values, Tensor target_row, int nnz, int CF,
+                                  int blkWarpNum)
+{
+    return vec_profile(X, rowPtr, colIdx, values, &target_row, nnz, CF, blkWarpNum);
+}
 
 // ---- row-caching baseline under the reference's gespmm_* names (SpMM/Baseline_kernel.cu:744-857) ----------------
 static void rowcache_into(Tensor &Y, const Tensor &X, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values)
@@ -196,14 +268,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("csr_split_spmm", &csr_split_spmm, "row-split CSR SpMM (HIP, gfx950)");
     m.def("bcsr_spmm", &bcsr_spmm, "2x1 BCSR SpMM (HIP, gfx950)");
     m.def("bcsr_split_spmm", &bcsr_split_spmm, "row-split 2x1 BCSR SpMM (HIP, gfx950)");
-    m.def("vec_spmm", &vec_spmm, "not built");
-    m.def("vec_split_spmm", &vec_split_spmm, "not built");
+    m.def("vec_spmm", &vec_spmm, "3x1-block SpMM (HIP, gfx950)");
+    m.def("vec_split_spmm", &vec_split_spmm, "row-split 3x1-block SpMM (HIP, gfx950)");
     m.def("csr_spmm_profile", &csr_spmm_profile, "GFLOP/s of csr_spmm");
     m.def("csr_split_spmm_profile", &csr_split_spmm_profile, "GFLOP/s of csr_split_spmm");
     m.def("bcsr_spmm_profile", &bcsr_spmm_profile, "GFLOP/s of bcsr_spmm");
     m.def("bcsr_split_spmm_profile", &bcsr_split_spmm_profile, "GFLOP/s of bcsr_split_spmm");
-    m.def("vec_spmm_profile", &vec_spmm_profile, "not built");
-    m.def("vec_split_spmm_profile", &vec_split_spmm_profile, "not built");
+    m.def("vec_spmm_profile", &vec_spmm_profile, "GFLOP/s of vec_spmm");
+    m.def("vec_split_spmm_profile", &vec_split_spmm_profile, "GFLOP/s of vec_split_spmm");
     m.def("cusparse_compute", &cusparse_compute, "rocSPARSE SpMM baseline");
     m.def("cusparse_profile", &cusparse_profile, "GFLOP/s of the rocSPARSE SpMM baseline");
     m.def("cusparse_compute_csr_alg2", &cusparse_compute_csr_alg2, "rocSPARSE SpMM baseline");

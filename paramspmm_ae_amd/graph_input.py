@@ -181,14 +181,28 @@ def _use_device(build_on):
     return build_on == "device" or (build_on == "auto" and torch.cuda.is_available())
 
 
-def build_bcsr(rowPtr, colIdx, val, ncols=None, build_on="host", device_arrays=None):
-    """CSR (numpy int32/int32/fp32) -> 2x1 BCSR arrays (numpy) via libparamsp_hip.so: the host builder, or the
-    device builder when ``build_on`` says so and the rows are strictly ascending.  ``device_arrays``: the CSR
-    already on the GPU (rowPtr, colIdx, val) to build from; on return it holds the three BCSR tensors on the GPU."""
+def build_bcsr(rowPtr, colIdx, val, ncols=None, build_on="host", device_arrays=None, blk_size=2):
+    """CSR (numpy int32/int32/fp32) -> blk_size x 1 BCSR arrays (numpy) via libparamsp_hip.so: the host builder, or,
+    for 2x1 blocks, the device builder when ``build_on`` says so and the rows are strictly ascending.
+    ``device_arrays``: the CSR already on the GPU (rowPtr, colIdx, val) to build from; on return it holds the three
+    BCSR tensors on the GPU (emptied when the host built them)."""
     rowPtr = np.ascontiguousarray(rowPtr, np.int32)
     colIdx = np.ascontiguousarray(colIdx, np.int32)
     val = np.ascontiguousarray(val, np.float32)
     n = rowPtr.size - 1
+    if blk_size != 2:
+        # the reference's blk_size argument (graph_input.py:210,245-256); its kernels exist for 3 (vec_spmm)
+        if device_arrays is not None:
+            del device_arrays[:]
+        R = int(blk_size)
+        ncols = (n + R - 1) // R * R if ncols is None else ncols
+        nblk = _capi.check(_capi.lib.psp_vbsr_count(_capi.ptr(rowPtr), _capi.ptr(colIdx), n, ncols, R))
+        rowPtr_b = np.empty((n + R - 1) // R + 1, np.int32)
+        colIdx_b = np.empty(nblk, np.int32)
+        val_b = np.empty((nblk, R), np.float32)
+        _capi.check(_capi.lib.psp_vbsr_build(_capi.ptr(rowPtr), _capi.ptr(colIdx), _capi.ptr(val), n, ncols, R,
+                                             _capi.ptr(rowPtr_b), _capi.ptr(colIdx_b), _capi.ptr(val_b)))
+        return rowPtr_b, colIdx_b, val_b
     if ncols is None and _use_device(build_on):
         from . import device_builder
 
@@ -271,8 +285,11 @@ class graph_input(object):
                       if_mask=False, build_on="auto"):
         """Build every format from a square CSR matrix given as arrays (column indices sorted per row).
         ``build_on``: "host", "device" or "auto" (the GPU when there is one) for the BCSR and row-split arrays."""
-        if blk_size != 2:
-            raise ValueError("this build only has 2x1 blocks (blk_size=2)")
+        if blk_size not in (2, 3):
+            raise ValueError("blocks of 2x1 and 3x1 are built (blk_size 2 or 3)")
+        if if_mask and blk_size != 2:
+            raise ValueError("the CSR -> block mask exists for 2x1 blocks only (SDDMM/sddmm_kernel.cu:78-107)")
+        self.blk_size = blk_size
         t0 = time.perf_counter()
         rowPtr = np.ascontiguousarray(rowPtr, np.int32)
         colIdx = np.ascontiguousarray(colIdx, np.int32)
@@ -291,15 +308,16 @@ class graph_input(object):
 
             on_gpu = [self.csr_data.on_device(k, "cuda") for k in ("rowPtr", "colIdx", "val")]
             # the host builder rejects column indices outside the matrix; so does this path
-            device_builder.check_index(on_gpu[0], on_gpu[1], n + (n & 1), what="load_from_csr")
-        rowPtr_b, colIdx_b, val_b = build_bcsr(rowPtr, colIdx, val, build_on=build_on, device_arrays=on_gpu)
+            device_builder.check_index(on_gpu[0], on_gpu[1], (n + blk_size - 1) // blk_size * blk_size, what="load_from_csr")
+        rowPtr_b, colIdx_b, val_b = build_bcsr(rowPtr, colIdx, val, build_on=build_on, device_arrays=on_gpu,
+                                               blk_size=blk_size)
         nblk = colIdx_b.size
         # graph_input.py:257-266: the blocked format counts block-rows and blocks (the latter as a float)
-        self.bcsr_data = csr_data(rowPtr_b, colIdx_b, val_b, (n + 1) // 2, float(nblk), False)
+        self.bcsr_data = csr_data(rowPtr_b, colIdx_b, val_b, (n + blk_size - 1) // blk_size, float(nblk), False)
         for k, t in zip(("rowPtr", "colIdx", "val"), on_gpu):
             self.bcsr_data._keep_device(k, t)
         self.bcsr_data.init_info(is_avg_granularity=is_avg_granularity, manual_granularity=manual_granularity)
-        self.pack_rate = nnz / (2 * nblk) if nblk else 0.0
+        self.pack_rate = nnz / (blk_size * nblk) if nblk else 0.0  # graph_input.py:274
 
         self.mask = None
         if if_mask:

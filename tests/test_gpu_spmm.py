@@ -209,3 +209,68 @@ def test_full_size_headline_graph_properties(oracle):
     lin = spmm_capi("csr_split", F, X1 + X2, 1, 8)
     both = spmm_capi("csr_split", F, X1, 1, 8) + spmm_capi("csr_split", F, X2, 1, 8)
     assert_close(lin, both.cpu().numpy(), rtol=1e-4, atol=1e-5, what="linearity at full size")
+
+
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("N,CF,bw", [(16, 1, 4), (32, 1, 8), (64, 2, 4), (100, 4, 8), (128, 4, 4), (192, 6, 8), (256, 8, 4), (7, 1, 4)])
+def test_spmm_3x1_blocks(oracle, split, N, CF, bw):
+    """vec_spmm / vec_split_spmm (3x1 blocks) through the C ABI against the oracle: a row count that is not a multiple
+    of 3, a hub row, empty rows; vec_size 2 through the same entry points equals the 2x1 operators."""
+    from paramspmm_ae_amd import _capi
+    from gpu_util import assert_close, dev, stream
+
+    rowPtr, colIdx, val = random_csr(2999, 8, 13, empty_frac=0.1, hub=(10, 1500))
+    n = rowPtr.size - 1
+    L, p = _capi.lib, _capi.ptr
+    for R in (3, 2):
+        rows_out = (n + R - 1) // R * R
+        rpb, cib, vb = oracle.vbsr_build(rowPtr, colIdx, val, R, ncols=rows_out)
+        X = np.random.default_rng(N).standard_normal((rows_out, N)).astype(np.float32)
+        Xd, Y = dev(X), torch.full((rows_out, N), float("nan"), device="cuda")
+        scale = oracle.spmm_vec(rpb, cib, np.abs(vb), np.abs(X), rows_out=rows_out)
+        # device copies stay referenced until the kernel has run: a pointer taken from a temporary tensor dangles as
+        # soon as the caching allocator hands the block to the next allocation
+        cib_d, vb_d = dev(cib), dev(vb)
+        if split:
+            rps, tr = oracle.split_csr(rpb, 8)
+            want = oracle.spmm_vec(rps, cib, vb, X, target_row=tr, rows_out=rows_out)
+            rps_d, tr_d = dev(rps), dev(tr)
+            _capi.check(L.psp_spmm_vec_split_f32(p(rps_d), p(cib_d), p(vb_d), p(tr_d), p(Xd), p(Y), tr.size, N,
+                                                 rows_out, R, CF, bw, stream()))
+        else:
+            want = oracle.spmm_vec(rpb, cib, vb, X, rows_out=rows_out)
+            rpb_d = dev(rpb)
+            _capi.check(L.psp_spmm_vec_f32(p(rpb_d), p(cib_d), p(vb_d), p(Xd), p(Y), rpb.size - 1, N, rows_out, R,
+                                           CF, bw, stream()))
+        torch.cuda.synchronize()
+        assert_close(Y, want, what="%dx1 blocks N=%d CF=%d split=%s" % (R, N, CF, split), scale=scale)
+    # an unsupported block height is an argument error (nothing is launched)
+    assert L.psp_spmm_vec_f32(p(cib_d), p(cib_d), p(vb_d), p(Xd), p(Y), 0, N, rows_out, 4, CF, bw, None) == -1
+
+
+def test_facade_with_3x1_blocks(oracle):
+    """graph_input(blk_size=3) + pcsr_spmm(vec_size=3): the reference's generic-block path (PCSR.py:227-239)."""
+    from paramspmm_ae_amd import synth
+    from paramspmm_ae_amd.graph_input import graph_input
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from gpu_util import assert_close
+
+    r, c, n = synth.chung_lu(5000, 20000, 2.1, seed=3)
+    rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+    g = graph_input("t", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val, blk_size=3)
+    rpb, cib, vb = oracle.vbsr_build(rowPtr, colIdx, val, 3, ncols=(n + 2) // 3 * 3)
+    assert np.array_equal(g.bcsr_data.colIdx.numpy(), cib) and np.array_equal(g.bcsr_data.val.numpy(), vb)
+    assert abs(g.pack_rate - colIdx.size / (3 * cib.size)) < 1e-12
+    X = np.random.default_rng(0).standard_normal((n, 48)).astype(np.float32)
+    want = oracle.spmm_csr(rowPtr, colIdx, val, X)
+    scale = oracle.spmm_csr(rowPtr, colIdx, np.abs(val), np.abs(X))
+    for split in (False, True):
+        op = pcsr_spmm(g, vec_size=3, if_split=split, CF=2, blkWarpNum=4)
+        op.get_spmm_result(x=torch.from_numpy(X))
+        assert op.result.shape == (n, 48)
+        assert_close(op.result, want, what="facade 3x1 split=%s" % split, scale=scale)
+        assert op.profiling(dim=32, verbose=False) > 0
+    with pytest.raises(ValueError, match="blk_size"):
+        pcsr_spmm(g, vec_size=2, if_split=False)

@@ -295,3 +295,20 @@ def test_reference_python_only_uses_exported_names():
     assert len(used) > 30
     for mod, attr in used:
         assert hasattr(mod, attr), (mod.__name__, attr)
+
+
+@pytest.mark.parametrize("R", [1, 2, 3, 4])
+def test_host_vbsr_builder_matches_oracle(oracle, R):
+    """psp_vbsr_build (blocks of R x 1, the reference's blk_size argument) against the oracle, which is pinned to
+    SciPy's tobsr((R,1)); R = 2 must equal psp_bcsr_build."""
+    from paramspmm_ae_amd.graph_input import build_bcsr
+
+    for n in (1, 10, 301, 302):
+        rowPtr, colIdx, val = random_csr(n, 4.0, seed=n * 7 + R, empty_frac=0.2)
+        if R == 2:
+            got = build_bcsr(rowPtr, colIdx, val, build_on="host")
+        else:
+            got = build_bcsr(rowPtr, colIdx, val, build_on="host", blk_size=R)
+        want = oracle.vbsr_build(rowPtr, colIdx, val, R, ncols=(n + R - 1) // R * R)
+        for a, b in zip(got, want):
+            assert a.dtype == b.dtype and np.array_equal(a, b)

@@ -131,3 +131,30 @@ def test_segment_softmax_closed_form(oracle):
         z = np.exp(e[a:b].astype(np.float64) - e[a:b].max())
         np.testing.assert_allclose(out[a:b], z / z.sum(), rtol=1e-6)
         assert abs(out[a:b].sum() - 1) < 1e-5
+
+
+@pytest.mark.parametrize("R", [2, 3])
+def test_spmm_vec_blocks(oracle, R):
+    """R x 1 blocks: every output row sees its own entries in CSR order (a block-row lists row R*t's columns first,
+    each row's entries stay ascending), so the result equals the CSR product bit for bit; R = 2 equals the 2 x 1
+    functions; the row-split variant adds the segments' partial sums."""
+    rowPtr, colIdx, val = random_csr(203, 6.0, seed=5, empty_frac=0.1, hub=(7, 150))
+    n = rowPtr.size - 1
+    X = np.random.default_rng(1).standard_normal((n + R, 24)).astype(np.float32)
+    rpb, cib, vb = oracle.vbsr_build(rowPtr, colIdx, val, R)
+    Y = oracle.spmm_vec(rpb, cib, vb, X)
+    want = oracle.spmm_csr(rowPtr, colIdx, val, X)
+    assert Y.shape[0] % R == 0 and Y.shape[0] >= n
+    # within a block-row the blocks are not column-sorted for rows after the first, so only row R*t is the same chain
+    assert np.array_equal(Y[0:n:R], want[0:n:R])
+    np.testing.assert_allclose(Y[:n], want[:n], rtol=1e-5, atol=1e-6)
+    assert not Y[n:].any()
+    dense = np.zeros((n, n + R))
+    rows = np.repeat(np.arange(n), np.diff(rowPtr))
+    dense[rows, colIdx] = val
+    np.testing.assert_allclose(Y[:n], dense @ X.astype(np.float64), rtol=1e-5, atol=1e-5)
+    if R == 2:
+        assert np.array_equal(Y, oracle.spmm_bcsr(rpb, cib, vb, X, rows_out=Y.shape[0]))
+    rps, tr = oracle.split_csr(rpb, 4)
+    Ys = oracle.spmm_vec(rps, cib, vb, X, target_row=tr, rows_out=Y.shape[0])
+    np.testing.assert_allclose(Ys, Y, rtol=1e-5, atol=1e-6)

@@ -134,3 +134,23 @@ def test_pubmed_counts(oracle, which):
         assert int(np.count_nonzero(cib[mask // 2] != colIdx)) == 454
         # with the diagonal set, as the normalised loaders do
         m2 = m.tolil(); m2.setdiag(1); assert m2.tocsr().nnz == 108365
+
+
+@pytest.mark.parametrize("R", [2, 3, 4])
+@pytest.mark.parametrize("n", [1, 7, 300, 301, 302])
+def test_vbsr_build_matches_scipy_tobsr(oracle, R, n):
+    """R x 1 blocks in SciPy's tobsr((R,1)) order (what graph_input.py:243-266 produces for blk_size = R), rows
+    padded to a multiple of R; R = 2 must equal the dedicated 2 x 1 builder."""
+    import scipy.sparse as sp
+
+    rowPtr, colIdx, val = random_csr(n, 5.0, seed=n + R, empty_frac=0.2)
+    rpb, cib, vb = oracle.vbsr_build(rowPtr, colIdx, val, R)
+    npad = (n + R - 1) // R * R
+    ip = np.concatenate([rowPtr, [rowPtr[-1]] * (npad - n)]).astype(np.int32)
+    bsr = sp.csr_matrix((val, colIdx, ip), shape=(npad, max(npad, n))).tobsr(blocksize=(R, 1))
+    assert np.array_equal(rpb, bsr.indptr)
+    assert np.array_equal(cib, bsr.indices)
+    assert np.array_equal(vb, bsr.data.reshape(-1, R))
+    if R == 2:
+        a, b, c = oracle.bcsr_build(rowPtr, colIdx, val)
+        assert np.array_equal(a, rpb) and np.array_equal(b, cib) and np.array_equal(np.asarray(c).reshape(-1, 2), vb)
