@@ -214,6 +214,16 @@ int psp_sddmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_b, const fl
                              const int *target_row, const float *A, const float *B, float *out, int Sb,
                              int K, int blkWarpNum, psp_stream_t stream);
 
+/* ParamSDDMM.vec_sddmm / vec_split_sddmm, SDDMM/sddmm.cpp:230-336 -> sddmm_kernel.cu:1289-1468: blocks of vec_size x 1,
+ * out is [nblk, vec_size].  The reference's kernels for this are never run and address their shared memory with a
+ * stride of CF*2 instead of CF*vec_size; this is their evident intent (the 2x1 rule for every entry of a block), for
+ * vec_size 3 and, through the 2x1 kernels, 2.  A needs vec_size*Mb rows. */
+int psp_sddmm_vec_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *A, const float *B,
+                      float *out, int Mb, int K, int vec_size, int blkWarpNum, psp_stream_t stream);
+int psp_sddmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b, const int *target_row,
+                            const float *A, const float *B, float *out, int Sb, int K, int vec_size,
+                            int blkWarpNum, psp_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: softmax over the stored entries of every CSR row (out[p] = exp(e[p]-max_r) / sum_r).
  * No counterpart in the reference (its AGNN layer applies no softmax, gnn_conv.py:136-142); it exists for

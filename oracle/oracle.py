@@ -132,6 +132,17 @@ def spmm_vec(rowPtr_b, colIdx_b, val_b, X, target_row=None, rows_out=None):
     return Y
 
 
+def sddmm_vec(rowPtr_b, colIdx_b, val_b, A, B, target_row=None):
+    """SDDMM on R x 1 blocks (R = val_b.shape[1]) -> out[nblk, R]; zero where the block value is zero."""
+    rowPtr_b, colIdx_b, val_b, A, B = _i32(rowPtr_b), _i32(colIdx_b), _f32(val_b), _f32(A), _f32(B)
+    R, nblk = val_b.shape[1], colIdx_b.size
+    out = np.empty((nblk, R), np.float32)
+    tr = None if target_row is None else _pi(_i32(target_row))
+    lib().orc_sddmm_vec(_pi(rowPtr_b), _pi(colIdx_b), _pf(val_b), tr, _pf(A), _pf(B), _pf(out), rowPtr_b.size - 1,
+                        A.shape[1], nblk, R)
+    return out
+
+
 def genmask(rowPtr_b, rowPtr, val_b, nnz):
     """SDDMM/sddmm_kernel.cu:78-141 -> int32[nnz].  rowPtr must cover 2*len(block rows) rows."""
     rowPtr_b, rowPtr, val_b = _i32(rowPtr_b), _i32(rowPtr), _f32(val_b)

@@ -26,6 +26,7 @@
  *   orc_spmm_vec          equals orc_spmm_bcsr(_split) for R = 2; for R = 3 the
  *                         CSR product of the same matrix (entry by entry the
  *                         same FMA chain), fp64 dense product
+ *   orc_sddmm_vec         equals orc_sddmm_bcsr(_split) for R = 2; fp64 dots
  *   orc_sddmm_*           fp64 gathered dot products, A = B = ones -> K
  *   orc_segment_softmax   closed form in fp64 (no reference counterpart)
  */
@@ -341,6 +342,24 @@ ORC_API void orc_sddmm_bcsr_split(const int *rowPtr_bs, const int *colIdx_b, con
                 out[2 * (size_t)p] = warp_dot(A + (size_t)(2 * t) * K, b, K);
             if (val_b[2 * (size_t)p + 1] != 0.0f)
                 out[2 * (size_t)p + 1] = warp_dot(A + (size_t)(2 * t + 1) * K, b, K);
+        }
+    }
+}
+
+/* R x 1 blocks, the intended generalisation of the 2 x 1 functions above (the reference's vec_sddmm kernels,
+ * sddmm_kernel.cu:1289-1468, index their shared memory with CF*2 instead of CF*vec_size and are never run; their
+ * evident intent is restated here, not their bug).  out is [nblk, R]; target_row = NULL: plain format.           */
+ORC_API void orc_sddmm_vec(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const int *target_row,
+                           const float *A, const float *B, float *out, int S, int K, int nblk, int R)
+{
+    memset(out, 0, sizeof(float) * (size_t)R * nblk);
+    for (int s = 0; s < S; s++) {
+        int t = target_row ? target_row[s] : s;
+        for (int p = rowPtr_b[s]; p < rowPtr_b[s + 1]; p++) {
+            const float *b = B + (size_t)colIdx_b[p] * K;
+            for (int q = 0; q < R; q++)
+                if (val_b[(size_t)R * p + q] != 0.0f)
+                    out[(size_t)R * p + q] = warp_dot(A + (size_t)(R * t + q) * K, b, K);
         }
     }
 }

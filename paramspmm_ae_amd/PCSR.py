@@ -97,7 +97,7 @@ class pcsr_spmm(object):
     def __init__(self, graph, vec_size, if_split, mtx_nodes=None, mtx_edges=None, rowPtr=None, colIdx=None,
                  val=None, target_row=None, CF=1, blkWarpNum=4, device="cuda"):
         if vec_size not in (1, 2, 3):
-            raise ValueError("this build has vec_size 1 (CSR), 2 (2x1 BCSR) and 3 (3x1 blocks, SpMM only)")
+            raise ValueError("this build has vec_size 1 (CSR), 2 (2x1 BCSR) and 3 (3x1 blocks)")
         if_split = bool(if_split)
         self.mask = None
         if graph is None:
@@ -184,10 +184,10 @@ class pcsr_spmm(object):
 
     # ---- SDDMM ------------------------------------------------------------------------------
     def _sddmm(self, A, B, blkWarpNum):
-        if self.vec_size == 3:
-            raise NotImplementedError("SDDMM on 3x1 blocks is not part of this build (the reference's vec_sddmm "
-                                      "kernels are never exercised and index their shared memory wrongly)")
-        fn = getattr(SDDMM, _SDDMM[self._key()])
+        if self.vec_size == 3:  # the generic-block operators (PCSR.py:300-345)
+            fn = SDDMM.vec_split_sddmm if self.if_split else SDDMM.vec_sddmm
+        else:
+            fn = getattr(SDDMM, _SDDMM[self._key()])
         CF = (A.size(1) + 31) // 32
         return fn(A, B, *self._sparse_args(), CF, blkWarpNum)
 
@@ -199,7 +199,8 @@ class pcsr_spmm(object):
 
     def get_sddmm_result(self, dim, blkWarpNum):
         assert torch.cuda.is_available()
-        A = torch.ones((self.mtx_nodes + 1) // 2 * 2, dim, device="cuda")
+        pad = max(self.vec_size, 2)
+        A = torch.ones((self.mtx_nodes + pad - 1) // pad * pad, dim, device="cuda")
         B = torch.ones(self.mtx_nodes, dim, device="cuda")
         return self._sddmm(A, B, blkWarpNum)
 

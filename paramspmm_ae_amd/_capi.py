@@ -68,6 +68,8 @@ SIGNATURES = {
     "psp_spmm_csr_split_softmax_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "psp_sddmm_bcsr_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "psp_sddmm_bcsr_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
+    "psp_sddmm_vec_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "psp_sddmm_vec_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "psp_segment_softmax_f32": [_vp, _vp, _vp, _i, _vp],
     "psp_segment_softmax_ws_f32": [_vp, _vp, _vp, _i, _i, _vp, _vp],
     "psp_baseline_rowcache_spmm_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp],

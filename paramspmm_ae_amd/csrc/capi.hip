@@ -401,6 +401,30 @@ PSP_EXPORT int psp_segment_softmax_ws_f32(const int *rowPtr, const float *in, fl
     return psp_check_launch("segment softmax kernels");
 }
 
+PSP_EXPORT int psp_sddmm_vec_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *A,
+                                 const float *B, float *out, int Mb, int K, int vec_size, int blkWarpNum,
+                                 psp_stream_t stream)
+{
+    if (vec_size == 2)
+        return psp_sddmm_launch<2, false>(rowPtr_b, colIdx_b, val_b, nullptr, A, B, nullptr, out, Mb, K, blkWarpNum,
+                                          (hipStream_t)stream, nullptr);
+    PSP_REQUIRE(vec_size == 3, "sddmm_vec: block height %d is not built (2 and 3 are)", vec_size);
+    return psp_sddmm_launch<3, false>(rowPtr_b, colIdx_b, val_b, nullptr, A, B, nullptr, out, Mb, K, blkWarpNum,
+                                      (hipStream_t)stream, nullptr);
+}
+
+PSP_EXPORT int psp_sddmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b,
+                                       const int *target_row, const float *A, const float *B, float *out, int Sb,
+                                       int K, int vec_size, int blkWarpNum, psp_stream_t stream)
+{
+    if (vec_size == 2)
+        return psp_sddmm_launch<2, true>(rowPtr_bs, colIdx_b, val_b, target_row, A, B, nullptr, out, Sb, K, blkWarpNum,
+                                         (hipStream_t)stream, nullptr);
+    PSP_REQUIRE(vec_size == 3, "sddmm_vec_split: block height %d is not built (2 and 3 are)", vec_size);
+    return psp_sddmm_launch<3, true>(rowPtr_bs, colIdx_b, val_b, target_row, A, B, nullptr, out, Sb, K, blkWarpNum,
+                                     (hipStream_t)stream, nullptr);
+}
+
 // ------------------------------------------------------------------------------------------------
 // host: row split (SpMM/SpMM.cpp:15-75)
 // ------------------------------------------------------------------------------------------------
@@ -627,7 +651,7 @@ PSP_EXPORT int psp_spmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b,
 PSP_EXPORT int psp_sddmm_csr_f32(const int *rowPtr, const int *colIdx, const float *A, const float *B,
                                  const float *scale, float *out, int M, int K, int blkWarpNum, psp_stream_t stream)
 {
-    return psp_sddmm_launch<false, false>(rowPtr, colIdx, nullptr, nullptr, A, B, scale, out, M, K, blkWarpNum,
+    return psp_sddmm_launch<1, false>(rowPtr, colIdx, nullptr, nullptr, A, B, scale, out, M, K, blkWarpNum,
                                           (hipStream_t)stream, nullptr);
 }
 
@@ -638,7 +662,7 @@ PSP_EXPORT int psp_sddmm_csr_rowmax_f32(const int *rowPtr, const int *colIdx, co
     PSP_REQUIRE(M >= 0 && (row_max || M == 0), "sddmm rowmax: row_max is null");
     int rc = psp_fill_f32(row_max, (size_t)M, PSP_F32_LOWEST, (hipStream_t)stream);
     if (rc != PSP_OK) return rc;
-    return psp_sddmm_launch<false, false>(rowPtr, colIdx, nullptr, nullptr, A, B, scale, out, M, K, blkWarpNum,
+    return psp_sddmm_launch<1, false>(rowPtr, colIdx, nullptr, nullptr, A, B, scale, out, M, K, blkWarpNum,
                                           (hipStream_t)stream, row_max);
 }
 
@@ -646,7 +670,7 @@ PSP_EXPORT int psp_sddmm_csr_split_f32(const int *rowPtr_split, const int *colId
                                        const float *A, const float *B, const float *scale, float *out, int S,
                                        int K, int blkWarpNum, psp_stream_t stream)
 {
-    return psp_sddmm_launch<false, true>(rowPtr_split, colIdx, nullptr, target_row, A, B, scale, out, S, K,
+    return psp_sddmm_launch<1, true>(rowPtr_split, colIdx, nullptr, target_row, A, B, scale, out, S, K,
                                          blkWarpNum, (hipStream_t)stream, nullptr);
 }
 
@@ -658,14 +682,14 @@ PSP_EXPORT int psp_sddmm_csr_split_rowmax_f32(const int *rowPtr_split, const int
     PSP_REQUIRE(rows >= 0 && (row_max || rows == 0), "sddmm rowmax: row_max is null");
     int rc = psp_fill_f32(row_max, (size_t)rows, PSP_F32_LOWEST, (hipStream_t)stream);
     if (rc != PSP_OK) return rc;
-    return psp_sddmm_launch<false, true>(rowPtr_split, colIdx, nullptr, target_row, A, B, scale, out, S, K,
+    return psp_sddmm_launch<1, true>(rowPtr_split, colIdx, nullptr, target_row, A, B, scale, out, S, K,
                                          blkWarpNum, (hipStream_t)stream, row_max);
 }
 
 PSP_EXPORT int psp_sddmm_bcsr_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *A,
                                   const float *B, float *out, int Mb, int K, int blkWarpNum, psp_stream_t stream)
 {
-    return psp_sddmm_launch<true, false>(rowPtr_b, colIdx_b, val_b, nullptr, A, B, nullptr, out, Mb, K, blkWarpNum,
+    return psp_sddmm_launch<2, false>(rowPtr_b, colIdx_b, val_b, nullptr, A, B, nullptr, out, Mb, K, blkWarpNum,
                                          (hipStream_t)stream, nullptr);
 }
 
@@ -673,6 +697,6 @@ PSP_EXPORT int psp_sddmm_bcsr_split_f32(const int *rowPtr_bs, const int *colIdx_
                                         const int *target_row, const float *A, const float *B, float *out, int Sb,
                                         int K, int blkWarpNum, psp_stream_t stream)
 {
-    return psp_sddmm_launch<true, true>(rowPtr_bs, colIdx_b, val_b, target_row, A, B, nullptr, out, Sb, K,
+    return psp_sddmm_launch<2, true>(rowPtr_bs, colIdx_b, val_b, target_row, A, B, nullptr, out, Sb, K,
                                         blkWarpNum, (hipStream_t)stream, nullptr);
 }

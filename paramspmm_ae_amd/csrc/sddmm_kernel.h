@@ -52,14 +52,14 @@ template <int LOGL> __device__ __forceinline__ float psp_group_max(float v)
 // row_max (CSR layouts, may be null): the largest result of every row is also raised into row_max[row] (atomic
 // max, once per lane group and row; the caller has filled the array with the lowest float).  The attention
 // pipeline's softmax-weighted SpMM takes its reference maxima from there instead of sweeping the entries again.
-template <int LOGL, int C, int V, int U, bool BCSR, bool SPLIT, bool SCALE>
+template <int LOGL, int C, int V, int U, int NR, bool SPLIT, bool SCALE>
 __global__ void __launch_bounds__(512)
 psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
                  const int *__restrict__ target_row, const float *__restrict__ A, const float *__restrict__ B,
                  float *__restrict__ out, int nseg, int K, int logW, int tiles, int stripe, float *__restrict__ row_max)
 {
     typedef typename psp_vec<V>::type vec_t;
-    constexpr int NR = BCSR ? 2 : 1;
+    constexpr bool BCSR = NR > 1;  // NR rows per stored entry: 1 = CSR, 2 = 2x1 blocks, 3 = 3x1 blocks
     constexpr int L = 1 << LOGL;
     constexpr int R = PSP_WAVE >> LOGL;
     static_assert(U <= L, "unroll must not exceed the group width");
@@ -158,10 +158,13 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
         const int q = base + sub;
         const int qq = q < b0 ? q : b0 - 1;
         c_out = colIdx[qq];
-        if constexpr (BCSR) {
+        if constexpr (NR == 2) {
             const psp_f32x2 t = ((const psp_f32x2 *)val)[qq];
             g_out[0] = t[0];
             g_out[1] = t[1];
+        } else if constexpr (NR > 2) {
+#pragma unroll
+            for (int r = 0; r < NR; r++) g_out[r] = val[(size_t)qq * NR + r];
         } else {
             g_out[0] = SCALE ? val[qq] : 1.0f;
         }
@@ -234,12 +237,15 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
             }
         }
         if (ok) {
-            if constexpr (BCSR) {
+            if constexpr (NR == 2) {
                 // entries of a block whose value is zero are padding: written as zero (sddmm_kernel.cu:1103,1115)
                 psp_f32x2 o;
                 o[0] = gate[0] != 0.0f ? res[0] : 0.0f;
                 o[1] = gate[1] != 0.0f ? res[1] : 0.0f;
                 ((psp_f32x2 *)out)[p] = o;
+            } else if constexpr (NR > 2) {
+#pragma unroll
+                for (int r = 0; r < NR; r++) out[(size_t)p * NR + r] = gate[r] != 0.0f ? res[r] : 0.0f;
             } else {
                 out[p] = SCALE ? res[0] * gate[0] : res[0];
             }
@@ -260,21 +266,21 @@ typedef void (*psp_sddmm_kernel_t)(const int *, const int *, const float *, cons
     M_(0, 1, 1) M_(1, 1, 2) M_(2, 1, 4) M_(3, 1, 4) M_(4, 1, 4) \
     M_(4, 2, 4) M_(4, 3, 2) M_(4, 4, 2) M_(5, 4, 2) M_(6, 4, 2)
 
-template <bool BCSR, bool SPLIT, bool SCALE>
+template <int NR, bool SPLIT, bool SCALE>
 static psp_sddmm_kernel_t psp_sddmm_lookup(int logL, int C, int V)
 {
 #define PSP_CASE(L_, C_, U_)                                                               \
     if (logL == L_ && C == C_) {                                                           \
-        if (V == 4) return psp_sddmm_kernel<L_, C_, 4, U_, BCSR, SPLIT, SCALE>;            \
-        if (V == 2) return psp_sddmm_kernel<L_, C_, 2, U_, BCSR, SPLIT, SCALE>;            \
-        return psp_sddmm_kernel<L_, C_, 1, U_, BCSR, SPLIT, SCALE>;                        \
+        if (V == 4) return psp_sddmm_kernel<L_, C_, 4, U_, NR, SPLIT, SCALE>;            \
+        if (V == 2) return psp_sddmm_kernel<L_, C_, 2, U_, NR, SPLIT, SCALE>;            \
+        return psp_sddmm_kernel<L_, C_, 1, U_, NR, SPLIT, SCALE>;                        \
     }
     PSP_SDDMM_FOR_EACH_LCU(PSP_CASE)
 #undef PSP_CASE
     return nullptr;
 }
 
-template <bool BCSR, bool SPLIT>
+template <int NR, bool SPLIT>
 int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
                      const float *A, const float *B, const float *scale, float *out, int nrows, int K,
                      int blkWarpNum, hipStream_t stream, float *row_max);

@@ -2,11 +2,12 @@
 #pragma once
 #include "sddmm_kernel.h"
 
-template <bool BCSR, bool SPLIT>
+template <int NR, bool SPLIT>
 int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
                      const float *A, const float *B, const float *scale, float *out, int nrows, int K,
                      int blkWarpNum, hipStream_t stream, float *row_max)
 {
+    constexpr bool BCSR = NR > 1;
     PSP_REQUIRE(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8");
     PSP_REQUIRE(nrows >= 0 && K >= 1, "sddmm: bad size (rows %d, K %d)", nrows, K);
     if (nrows == 0) return PSP_OK;
@@ -25,8 +26,8 @@ int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, con
     if (logL > 6) return psp_fail(PSP_ERR_RANGE, "sddmm: K = %d is too wide (max %d for this alignment)", K, 256 * V);
     if (logL < 4 && C > 1) C = 1;
 
-    psp_sddmm_kernel_t k = scale ? psp_sddmm_lookup<BCSR, SPLIT, !BCSR>(logL, C, V)
-                                 : psp_sddmm_lookup<BCSR, SPLIT, false>(logL, C, V);
+    psp_sddmm_kernel_t k = scale ? psp_sddmm_lookup<NR, SPLIT, !BCSR>(logL, C, V)
+                                 : psp_sddmm_lookup<NR, SPLIT, false>(logL, C, V);
     if (!k) return psp_fail(PSP_ERR_ARG, "sddmm: no kernel for logL %d coarsen %d vec %d", logL, C, V);
 
     // segments per wavefront: as for SpMM (one per lane group for plain input, 16 for row-split input, fewer for

@@ -1,0 +1,4 @@
+// SDDMM kernels of the 3x1-block format, row-split (instantiations only; the template lives in sddmm_kernel.h).
+#include "sddmm_launch_impl.h"
+template int psp_sddmm_launch<3, true>(const int *, const int *, const float *, const int *, const float *,
+                                      const float *, const float *, float *, int, int, int, hipStream_t, float *);

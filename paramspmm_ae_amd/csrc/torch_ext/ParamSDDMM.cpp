@@ -204,14 +204,85 @@ static Tensor segment_softmax(Tensor rowPtr, Tensor e)
     return out;
 }
 
-[[noreturn]] static void not_built(const char *what)
+// ---- generic vec_size x 1 blocks (SDDMM/sddmm.cpp:221-336, 547-661): values [nblk, vec_size] -> out [nblk, vec_size].
+// The reference instantiates vec_size 3 only, and those kernels are never run (they stride their shared memory by
+// CF*2 instead of CF*vec_size); this is their evident intent: the 2x1 rule for each entry of a block.
+static void check_vec_sddmm_args(const Tensor &A, const Tensor &B, const Tensor &rowPtr, const Tensor &colIdx,
+                                 const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
 {
-    TORCH_CHECK(false, what, " is not part of this build (only the PCSR operators csr/csr_split/bcsr/bcsr_split are)");
+    need_gpu(A, "A");
+    need_gpu(B, "B");
+    need_gpu(rowPtr, "rowPtr");
+    need_gpu(colIdx, "colIdx");
+    need_gpu(values, "values");
+    need_f32(A, "A", 2);
+    need_f32(B, "B", 2);
+    need_i32(rowPtr, "rowPtr");
+    need_i32(colIdx, "colIdx");
+    need_f32(values, "values", 2);
+    TORCH_CHECK(values.size(1) == 2 || values.size(1) == 3, "vec_sddmm: values must be [nblk, 3] (or [nblk, 2]); got vec_size ",
+                values.size(1));
+    TORCH_CHECK(values.size(0) == colIdx.size(0), "values and colIdx disagree on the number of stored blocks");
+    TORCH_CHECK(A.size(1) == B.size(1) && A.size(1) >= 1, "A and B must have the same, non-zero number of columns");
+    check_rowptr_vs(rowPtr, "rowPtr");
+    same_device(A, B, "vec_sddmm");
+    same_device(A, rowPtr, "vec_sddmm");
+    same_device(A, colIdx, "vec_sddmm");
+    same_device(A, values, "vec_sddmm");
+    TORCH_CHECK(CF >= 1 && CF <= 8, "CF must be 1..8");
+    TORCH_CHECK(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8");
+    if (target_row) {
+        need_gpu(*target_row, "target_row");
+        need_i32(*target_row, "target_row");
+        same_device(A, *target_row, "vec_sddmm");
+        TORCH_CHECK(target_row->size(0) == rowPtr.size(0) - 1, "target_row must have one entry per row segment");
+    } else {
+        TORCH_CHECK(values.size(1) * (rowPtr.size(0) - 1) <= A.size(0), "A needs vec_size rows per block-row (pad it)");
+    }
 }
-static Tensor vec_sddmm(Tensor, Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_sddmm (vec_size 3 blocks)"); }
-static Tensor vec_split_sddmm(Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, int, int) { not_built("vec_split_sddmm"); }
-static int vec_sddmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_sddmm_profile"); }
-static int vec_split_sddmm_profile(Tensor, Tensor, Tensor, Tensor, Tensor, Tensor, int, int, int) { not_built("vec_split_sddmm_profile"); }
+static Tensor vec_sddmm_new(const Tensor &A, const Tensor &B, const Tensor &rowPtr, const Tensor &colIdx,
+                            const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
+{
+    check_vec_sddmm_args(A, B, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
+    pspglue::DeviceGuard guard(A.device());
+    auto out = torch::empty_like(values);
+    if (values.numel() == 0) return out;
+    const int nseg = (int)rowPtr.size(0) - 1, K = (int)A.size(1), R = (int)values.size(1);
+    if (target_row)
+        ok(psp_sddmm_vec_split_f32(ip(rowPtr), ip(colIdx), fp(values), ip(*target_row), fp(A), fp(B), fpw(out), nseg, K, R,
+                                   blkWarpNum, stream_of(A)));
+    else
+        ok(psp_sddmm_vec_f32(ip(rowPtr), ip(colIdx), fp(values), fp(A), fp(B), fpw(out), nseg, K, R, blkWarpNum, stream_of(A)));
+    return out;
+}
+static int vec_sddmm_profile_impl(const Tensor &A, const Tensor &B, const Tensor &rowPtr, const Tensor &colIdx,
+                                  const Tensor &values, const Tensor *target_row, long nnz, int CF, int blkWarpNum)
+{
+    check_vec_sddmm_args(A, B, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
+    pspglue::DeviceGuard guard(A.device());
+    const float ms = time_launches((hipStream_t)stream_of(A), kProfileWarmup, kProfileIters, [&] {
+        (void)vec_sddmm_new(A, B, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
+    });
+    return gflops(2.0 * (double)nnz * (double)A.size(1), ms);
+}
+static Tensor vec_sddmm(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, int CF, int blkWarpNum)
+{
+    return vec_sddmm_new(A, B, rowPtr, colIdx, values, nullptr, CF, blkWarpNum);
+}
+static Tensor vec_split_sddmm(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, Tensor target_row, int CF,
+                              int blkWarpNum)
+{
+    return vec_sddmm_new(A, B, rowPtr, colIdx, values, &target_row, CF, blkWarpNum);
+}
+static int vec_sddmm_profile(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, int nnz, int CF, int blkWarpNum)
+{
+    return vec_sddmm_profile_impl(A, B, rowPtr, colIdx, values, nullptr, nnz, CF, blkWarpNum);
+}
+static int vec_split_sddmm_profile(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, Tensor target_row,
+                                   int nnz, int CF, int blkWarpNum)
+{
+    return vec_sddmm_profile_impl(A, B, rowPtr, colIdx, values, &target_row, nnz, CF, blkWarpNum);
+}
 // vendor baseline under the reference's name (SDDMM/sddmm_baseline_kernel.cu): rocSPARSE SDDMM, written in place
 // into `values`, which is also returned
 static Tensor cusparse_sddmm_compute(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values)
@@ -235,14 +306,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("csr_split_sddmm", &csr_split_sddmm, "row-split CSR SDDMM (HIP, gfx950)");
     m.def("bcsr_sddmm", &bcsr_sddmm, "2x1 BCSR SDDMM (HIP, gfx950)");
     m.def("bcsr_split_sddmm", &bcsr_split_sddmm, "row-split 2x1 BCSR SDDMM (HIP, gfx950)");
-    m.def("vec_sddmm", &vec_sddmm, "not built");
-    m.def("vec_split_sddmm", &vec_split_sddmm, "not built");
+    m.def("vec_sddmm", &vec_sddmm, "3x1-block SDDMM (HIP, gfx950)");
+    m.def("vec_split_sddmm", &vec_split_sddmm, "row-split 3x1-block SDDMM (HIP, gfx950)");
     m.def("csr_sddmm_profile", &csr_sddmm_profile, "GFLOP/s of csr_sddmm");
     m.def("csr_split_sddmm_profile", &csr_split_sddmm_profile, "GFLOP/s of csr_split_sddmm");
     m.def("bcsr_sddmm_profile", &bcsr_sddmm_profile, "GFLOP/s of bcsr_sddmm");
     m.def("bcsr_split_sddmm_profile", &bcsr_split_sddmm_profile, "GFLOP/s of bcsr_split_sddmm");
-    m.def("vec_sddmm_profile", &vec_sddmm_profile, "not built");
-    m.def("vec_split_sddmm_profile", &vec_split_sddmm_profile, "not built");
+    m.def("vec_sddmm_profile", &vec_sddmm_profile, "GFLOP/s of vec_sddmm");
+    m.def("vec_split_sddmm_profile", &vec_split_sddmm_profile, "GFLOP/s of vec_split_sddmm");
     m.def("cusparse_sddmm_compute", &cusparse_sddmm_compute, "rocSPARSE SDDMM baseline (in place)");
     m.def("cusparse_sddmm_profile", &cusparse_sddmm_profile, "GFLOP/s of the rocSPARSE SDDMM baseline");
     m.def("genmask", &genmask, "CSR slot -> flat index into the 2x1 block values");

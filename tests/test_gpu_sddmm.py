@@ -266,3 +266,59 @@ def test_fused_attention_modules_match_unfused():
     e, m = ParamSDDMM.csr_split_sddmm_scaled_rowmax(X, X, rps, ci, v, tr, n, 8)
     got = ParamSpMM.csr_split_spmm_softmax(H, rps, ci, e, m, tr, 1, 8)
     torch.testing.assert_close(got, want, rtol=2e-5, atol=2e-6)
+
+
+@pytest.mark.parametrize("split", [False, True])
+@pytest.mark.parametrize("K", [16, 32, 100, 128, 256, 7])
+def test_sddmm_3x1_blocks(oracle, split, K):
+    """vec_sddmm / vec_split_sddmm through the C ABI against the oracle, vec_size 3 and (through the same entry points)
+    2; a row count that is not a multiple of the block height, a hub row, empty rows."""
+    from paramspmm_ae_amd import _capi
+    from gpu_util import assert_close, dev, stream
+
+    rowPtr, colIdx, val = random_csr(2000, 8, 17, empty_frac=0.1, hub=(10, 900), values="uniform")
+    n = rowPtr.size - 1
+    L, p = _capi.lib, _capi.ptr
+    for R in (3, 2):
+        npad = (n + R - 1) // R * R
+        rpb, cib, vb = oracle.vbsr_build(rowPtr, colIdx, val, R, ncols=npad)
+        A, B = unit_rows(npad, K, K), unit_rows(npad, K, K + 1)
+        Ad, Bd, cib_d, vb_d = dev(A), dev(B), dev(cib), dev(vb)  # referenced until the kernel has run
+        out = torch.full((cib.size, R), float("nan"), device="cuda")
+        for bw in (4, 8):
+            if split:
+                rps, tr = oracle.split_csr(rpb, 8)
+                want = oracle.sddmm_vec(rps, cib, vb, A, B, target_row=tr)
+                rps_d, tr_d = dev(rps), dev(tr)
+                _capi.check(L.psp_sddmm_vec_split_f32(p(rps_d), p(cib_d), p(vb_d), p(tr_d), p(Ad), p(Bd), p(out), tr.size, K, R,
+                                                      bw, stream()))
+            else:
+                want = oracle.sddmm_vec(rpb, cib, vb, A, B)
+                rpb_d = dev(rpb)
+                _capi.check(L.psp_sddmm_vec_f32(p(rpb_d), p(cib_d), p(vb_d), p(Ad), p(Bd), p(out), rpb.size - 1, K, R, bw,
+                                                stream()))
+            torch.cuda.synchronize()
+            assert_close(out, want, what="%dx1 blocks K=%d bw=%d split=%s" % (R, K, bw, split))
+
+
+def test_facade_sddmm_with_3x1_blocks(oracle):
+    from paramspmm_ae_amd import synth
+    from paramspmm_ae_amd.graph_input import graph_input
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from gpu_util import assert_close
+
+    r, c, n = synth.chung_lu(3001, 12000, 2.1, seed=4)
+    rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+    g = graph_input("t", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val, blk_size=3)
+    rpb, cib, vb = (g.bcsr_data.rowPtr.numpy(), g.bcsr_data.colIdx.numpy(), g.bcsr_data.val.numpy())
+    npad = (n + 2) // 3 * 3
+    A = unit_rows(npad, 32, 5)
+    want = oracle.sddmm_vec(rpb, cib, vb, A, A)
+    for split in (False, True):
+        op = pcsr_spmm(g, vec_size=3, if_split=split, CF=1, blkWarpNum=4)
+        got = op._sddmm(torch.from_numpy(A).cuda(), torch.from_numpy(A).cuda(), 4)
+        assert_close(got, want, what="facade 3x1 sddmm split=%s" % split)
+        ones = op.get_sddmm_result(64, 8)
+        assert torch.all(ones[torch.from_numpy(vb != 0).cuda()] == 64)

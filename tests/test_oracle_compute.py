@@ -158,3 +158,28 @@ def test_spmm_vec_blocks(oracle, R):
     rps, tr = oracle.split_csr(rpb, 4)
     Ys = oracle.spmm_vec(rps, cib, vb, X, target_row=tr, rows_out=Y.shape[0])
     np.testing.assert_allclose(Ys, Y, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("R", [2, 3])
+def test_sddmm_vec_blocks(oracle, R):
+    """R x 1 blocks: R = 2 equals the 2 x 1 functions; every non-zero entry equals the fp64 dot product of its row of
+    A and column row of B, padding entries are zero; the row-split variant gives the same array."""
+    rowPtr, colIdx, val = random_csr(120, 5.0, seed=9, empty_frac=0.1)
+    n = rowPtr.size - 1
+    npad = (n + R - 1) // R * R
+    rpb, cib, vb = oracle.vbsr_build(rowPtr, colIdx, val, R)
+    rng = np.random.default_rng(2)
+    A = rng.standard_normal((npad, 40)).astype(np.float32)
+    B = rng.standard_normal((npad, 40)).astype(np.float32)
+    out = oracle.sddmm_vec(rpb, cib, vb, A, B)
+    assert out.shape == vb.shape
+    blk_row = np.repeat(np.arange(rpb.size - 1), np.diff(rpb))
+    for q in range(R):
+        want = np.einsum("ij,ij->i", A[R * blk_row + q].astype(np.float64), B[cib].astype(np.float64))
+        nz = vb[:, q] != 0
+        np.testing.assert_allclose(out[nz, q], want[nz], rtol=1e-5, atol=1e-5)
+        assert not out[~nz, q].any()
+    if R == 2:
+        assert np.array_equal(out, np.asarray(oracle.sddmm_bcsr(rpb, cib, vb, A, B)).reshape(-1, 2))
+    rps, tr = oracle.split_csr(rpb, 3)
+    assert np.array_equal(oracle.sddmm_vec(rps, cib, vb, A, B, target_row=tr), out)
