@@ -215,7 +215,31 @@ def bench_sddmm(args):
                       "rocsparse_ms": None if vendor_ms is None else round(vendor_ms, 5)})
     total_ms = sum(r["ms"] for r in per_K)
     value = sum(2.0 * nnz * r["K"] for r in per_K) / total_ms / 1e6
-    print(json.dumps({"metric": "SDDMM GFLOP/s (2*nnz*K) over K = 16..128", "value": round(value, 1), "unit": "GFLOP/s",
+    cpu = None
+    if not args.no_cpu:
+        # CPU path beside it: gathered (A[row] * B[col]).sum(1) in chunks, on a bounded sample of the entries
+        import time as _t
+        K = 64
+        take = min(nnz, 4_000_000)
+        rows_h = torch.from_numpy(np.repeat(np.arange(n, dtype=np.int64), np.diff(rowPtr))[:take])
+        cols_h = torch.from_numpy(colIdx[:take].astype(np.int64))
+        Ah, Bh = torch.randn(rows, K), torch.randn(rows, K)
+        def cpu_once():
+            out = torch.empty(take)
+            for s0 in range(0, take, 1 << 18):
+                sl = slice(s0, min(take, s0 + (1 << 18)))
+                out[sl] = (Ah[rows_h[sl]] * Bh[cols_h[sl]]).sum(1)
+            return out
+        cpu_once()
+        t0 = _t.perf_counter()
+        reps = 0
+        while reps < 3 or _t.perf_counter() - t0 < 5.0:
+            cpu_once()
+            reps += 1
+        dt = (_t.perf_counter() - t0) / reps
+        cpu = {"value": round(2.0 * take * K / dt / 1e9, 2), "unit": "GFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+               "sample": "gathered (A[row]*B[col]).sum(1) with torch on the host, K = 64, the first %d stored entries, %d reps" % (take, reps)}
+    print(json.dumps({"cpu_baseline": cpu, "metric": "SDDMM GFLOP/s (2*nnz*K) over K = 16..128", "value": round(value, 1), "unit": "GFLOP/s",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(total_ms, 4),
                       "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
                       "config": {"workload": "%s SDDMM width sweep" % args.graph, "nodes": n, "nnz": nnz}, "per_K": per_K}))
@@ -448,9 +472,14 @@ def main():
         fmt = fmt_names[(1 if if_split else 0) + (2 if vec == 2 else 0)]
         b_alg = algorithmic_bytes(fmt, F, n, d)
         gbs = b_alg / (ms * 1e-3) / 1e9
+        # no-reuse gather volume: every stored entry fetches its row of X (what a matrix without locality moves)
+        stored = F["nblk"] if fmt.startswith("bcsr") else nnz
+        b_gather = b_alg - 4 * n * d + 4 * stored * d
         per_dim.append({"dim": d, "format": fmt, "CF": cf, "blkWarpNum": bw, "ms": round(ms, 5),
                         "gflops": round(2.0 * nnz * d / (ms * 1e-3) / 1e9, 1), "alg_bytes": b_alg,
-                        "alg_GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4)})
+                        "alg_GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
+                        "gather_bytes": int(b_gather),
+                        "frac_hbm_no_reuse_gather": round(b_gather / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
     # The dominant kernel: widths that share (vectors per lane, vector width, unroll, format) run the same kernel
     # symbol, which is what a rocprofv3 kernel trace averages over; take the symbol with the largest share of time.
     by_symbol = {}
@@ -470,7 +499,9 @@ def main():
                 "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                 "kernel": sym, "widths": [r["dim"] for r in rows_of],
                 "alg_bytes_per_launch": int(sym_bytes / len(rows_of)), "ms_per_launch": round(sym_ms / len(rows_of), 5),
-                "mean_frac_over_widths": round(float(np.mean([r["frac_hbm"] for r in per_dim])), 4)}
+                "mean_frac_over_widths": round(float(np.mean([r["frac_hbm"] for r in per_dim])), 4),
+                "gather_bytes_per_launch": int(sum(r["gather_bytes"] for r in rows_of) / len(rows_of)),
+                "frac_no_reuse_gather": round(sum(r["gather_bytes"] for r in rows_of) / (sym_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)}
 
     out = {
         "metric": "SpMM GFLOP/s (2*nnz*N) over the feature-width sweep N=16..256, with HBM GB/s as fraction of 8 TB/s",
