@@ -274,3 +274,26 @@ def test_facade_with_3x1_blocks(oracle):
         assert op.profiling(dim=32, verbose=False) > 0
     with pytest.raises(ValueError, match="blk_size"):
         pcsr_spmm(g, vec_size=2, if_split=False)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_spmm_non_finite_inputs_stay_in_their_rows(oracle, fmt):
+    """An Inf and a NaN row of X reach exactly the output rows that reference them (the oracle says which); every
+    other element stays finite and equal to the oracle's.  Lanes past the end of a range or of a row must not
+    multiply a padding value into a foreign row."""
+    from gpu_util import Formats, spmm_capi, spmm_oracle
+
+    rowPtr, colIdx, val = random_csr(1500, 7, 31, empty_frac=0.1, hub=(3, 600), values="uniform")
+    F = Formats(oracle, rowPtr, colIdx, val)
+    n = F.n
+    for N, CF, bw in ((16, 1, 4), (64, 2, 8), (100, 4, 4)):
+        X = np.random.default_rng(N).standard_normal((n + (n & 1), N)).astype(np.float32)
+        X[colIdx[5]] = np.inf            # a column some rows reference
+        X[colIdx[colIdx.size // 2]] = np.nan
+        X[n - 1] = np.inf                # the last column: where clamped loads would point
+        want = spmm_oracle(oracle, fmt, F, X)
+        got = spmm_capi(fmt, F, torch.from_numpy(X).cuda(), CF, bw).cpu().numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(want)), (fmt, N)
+        assert np.array_equal(np.isposinf(got), np.isposinf(want)) and np.array_equal(np.isneginf(got), np.isneginf(want))
+        fin = np.isfinite(want)
+        np.testing.assert_allclose(got[fin], want[fin], rtol=1e-4, atol=1e-5)
