@@ -268,6 +268,18 @@ int psp_nll_loss_mean_backward_f32(const long long *labels, const float *grad_lo
                                    int C, float *grad_logp, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
+ * DEVICE: double precision.  The reference dispatches its SpMM / SDDMM kernels for double as well
+ * (AT_DISPATCH_FLOATING_TYPES, SpMM_kernel.cu:149, sddmm_kernel.cu:161); these two entry points serve all six layouts:
+ * vec_size 1 (CSR), 2 or 3 (blocks of vec_size x 1, val [nblk, vec_size]); target_row NULL = plain layout, else
+ * row-split.  Same semantics as the float entry points (Y completely defined; SDDMM unscaled, zero where a block value
+ * is zero).  One wavefront per segment, not tuned: GNN training is single precision.  CF / blkWarpNum do not apply.
+ * ------------------------------------------------------------------------------------------- */
+int psp_spmm_f64(const int *rowPtr, const int *colIdx, const double *val, const int *target_row, const double *X,
+                 double *Y, int nseg, int N, int rows_out, int vec_size, psp_stream_t stream);
+int psp_sddmm_f64(const int *rowPtr, const int *colIdx, const double *val_b, const int *target_row, const double *A,
+                  const double *B, double *out, int nseg, int K, int vec_size, psp_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
  * DEVICE: comparison baseline, ParamSpMM.gespmm_compute (SpMM/Baseline_kernel.cu:616-788): CSR SpMM with one
  * wavefront per row and the row's (column, value) pairs cached in LDS.  Y [M,N] is fully written.
  * ------------------------------------------------------------------------------------------- */

@@ -72,6 +72,8 @@ SIGNATURES = {
     "psp_sddmm_vec_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "psp_segment_softmax_f32": [_vp, _vp, _vp, _i, _vp],
     "psp_segment_softmax_ws_f32": [_vp, _vp, _vp, _i, _i, _vp, _vp],
+    "psp_spmm_f64": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "psp_sddmm_f64": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "psp_baseline_rowcache_spmm_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
     "psp_nll_loss_mean_f32": [_vp, _vp, ctypes.c_longlong, _i, _vp, _vp, _vp],
     "psp_nll_loss_mean_backward_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _vp, _vp],

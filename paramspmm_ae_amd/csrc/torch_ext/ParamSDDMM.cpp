@@ -15,12 +15,14 @@ static void check_sddmm_args(int fmt, const Tensor &A, const Tensor &B, const Te
     need_gpu(rowPtr, "rowPtr");
     need_gpu(colIdx, "colIdx");
     need_gpu(values, "values");
-    need_f32(A, "A", 2);
-    need_f32(B, "B", 2);
+    need_fp(A, "A", 2);
+    need_fp(B, "B", 2);
     need_i32(rowPtr, "rowPtr");
     need_i32(colIdx, "colIdx");
     const bool blocked = fmt >= 2;
-    need_f32(values, "values", blocked ? 2 : 1);
+    need_fp(values, "values", blocked ? 2 : 1);
+    same_dtype(A, B, "sddmm");
+    same_dtype(A, values, "sddmm");
     if (blocked) TORCH_CHECK(values.size(1) == 2, "values of a bcsr format must be [nblk, 2]");
     TORCH_CHECK(values.size(0) == colIdx.size(0), "values and colIdx disagree on the number of stored entries");
     TORCH_CHECK(A.size(1) == B.size(1), "A and B must have the same number of columns");
@@ -54,6 +56,12 @@ static Tensor sddmm_new(int fmt, const Tensor &A, const Tensor &B, const Tensor 
     const int nrows = (int)rowPtr.size(0) - 1, K = (int)A.size(1);
     if (values.numel() == 0) return out;
     psp_stream_t s = stream_of(A);
+    if (is_f64(A)) {
+        TORCH_CHECK(!scale, "the scaled SDDMM variants are float32 only");
+        ok(psp_sddmm_f64(ip(rowPtr), ip(colIdx), fmt >= 2 ? dp(values) : nullptr, target_row ? ip(*target_row) : nullptr, dp(A),
+                         dp(B), dpw(out), nrows, K, fmt >= 2 ? 2 : 1, s));
+        return out;
+    }
     int rc;
     switch (fmt) {
     case 0: rc = psp_sddmm_csr_f32(ip(rowPtr), ip(colIdx), fp(A), fp(B), scale ? fp(*scale) : nullptr, fpw(out), nrows, K, blkWarpNum, s); break;
@@ -215,11 +223,13 @@ static void check_vec_sddmm_args(const Tensor &A, const Tensor &B, const Tensor 
     need_gpu(rowPtr, "rowPtr");
     need_gpu(colIdx, "colIdx");
     need_gpu(values, "values");
-    need_f32(A, "A", 2);
-    need_f32(B, "B", 2);
+    need_fp(A, "A", 2);
+    need_fp(B, "B", 2);
     need_i32(rowPtr, "rowPtr");
     need_i32(colIdx, "colIdx");
-    need_f32(values, "values", 2);
+    need_fp(values, "values", 2);
+    same_dtype(A, B, "vec_sddmm");
+    same_dtype(A, values, "vec_sddmm");
     TORCH_CHECK(values.size(1) == 2 || values.size(1) == 3, "vec_sddmm: values must be [nblk, 3] (or [nblk, 2]); got vec_size ",
                 values.size(1));
     TORCH_CHECK(values.size(0) == colIdx.size(0), "values and colIdx disagree on the number of stored blocks");
@@ -248,6 +258,11 @@ static Tensor vec_sddmm_new(const Tensor &A, const Tensor &B, const Tensor &rowP
     auto out = torch::empty_like(values);
     if (values.numel() == 0) return out;
     const int nseg = (int)rowPtr.size(0) - 1, K = (int)A.size(1), R = (int)values.size(1);
+    if (is_f64(A)) {
+        ok(psp_sddmm_f64(ip(rowPtr), ip(colIdx), dp(values), target_row ? ip(*target_row) : nullptr, dp(A), dp(B), dpw(out),
+                         nseg, K, R, stream_of(A)));
+        return out;
+    }
     if (target_row)
         ok(psp_sddmm_vec_split_f32(ip(rowPtr), ip(colIdx), fp(values), ip(*target_row), fp(A), fp(B), fpw(out), nseg, K, R,
                                    blkWarpNum, stream_of(A)));

@@ -123,10 +123,11 @@ static void check_vec_args(const Tensor &X, const Tensor &rowPtr, const Tensor &
     need_gpu(rowPtr, "rowPtr");
     need_gpu(colIdx, "colIdx");
     need_gpu(values, "values");
-    need_f32(X, "input", 2);
+    need_fp(X, "input", 2);
     need_i32(rowPtr, "rowPtr");
     need_i32(colIdx, "colIdx");
-    need_f32(values, "values", 2);
+    need_fp(values, "values", 2);
+    same_dtype(X, values, "vec_spmm");
     TORCH_CHECK(values.size(1) == 2 || values.size(1) == 3, "vec_spmm: values must be [nblk, 3] (or [nblk, 2]); got vec_size ",
                 values.size(1));
     TORCH_CHECK(values.size(0) == colIdx.size(0), "values and colIdx disagree on the number of stored blocks");
@@ -149,6 +150,11 @@ static void vec_into(Tensor &Y, const Tensor &X, const Tensor &rowPtr, const Ten
 {
     const int nseg = (int)rowPtr.size(0) - 1, N = (int)X.size(1), rows_out = (int)Y.size(0), R = (int)values.size(1);
     if (N == 0 || rows_out == 0) return;
+    if (is_f64(X)) {
+        ok(psp_spmm_f64(ip(rowPtr), ip(colIdx), dp(values), target_row ? ip(*target_row) : nullptr, dp(X), dpw(Y), nseg, N,
+                        rows_out, R, stream_of(X)));
+        return;
+    }
     if (target_row)
         ok(psp_spmm_vec_split_f32(ip(rowPtr), ip(colIdx), fp(values), ip(*target_row), fp(X), fpw(Y), nseg, N, rows_out, R,
                                   CF, blkWarpNum, stream_of(X)));

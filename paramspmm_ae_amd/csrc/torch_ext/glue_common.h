@@ -16,8 +16,8 @@ namespace pspglue {
 using DeviceGuard = c10::hip::HIPGuardMasqueradingAsCUDA;
 
 // Same contract as the reference's CHECK_INPUT / CHECK_CPU_INPUT (SpMM/SpMM.cpp:5-13): a violation is a
-// RuntimeError in Python.  Index tensors must be int32 and value / feature tensors float32 (the reference
-// reaches the same requirement through its int / scalar_t accessors).
+// RuntimeError in Python.  Index tensors must be int32; value / feature tensors float32, or float64 for the
+// SpMM / SDDMM operators proper (the reference reaches the same requirement through its int / scalar_t accessors).
 inline void need_gpu(const torch::Tensor &t, const char *name)
 {
     TORCH_CHECK(t.device().is_cuda(), name, " must be a CUDA tensor");
@@ -38,6 +38,20 @@ inline void need_f32(const torch::Tensor &t, const char *name, int dims)
     TORCH_CHECK(t.scalar_type() == torch::kFloat32, name, " must be float32 (this build computes in fp32 only)");
     TORCH_CHECK(t.dim() == dims, name, " must be ", dims, "-D");
 }
+// The six SpMM / six SDDMM operators also take float64, as the reference's dispatch does (SpMM_kernel.cu:149); all
+// floating tensors of one call must then agree.
+inline void need_fp(const torch::Tensor &t, const char *name, int dims)
+{
+    TORCH_CHECK(t.scalar_type() == torch::kFloat32 || t.scalar_type() == torch::kFloat64, name, " must be float32 or float64");
+    TORCH_CHECK(t.dim() == dims, name, " must be ", dims, "-D");
+}
+inline void same_dtype(const torch::Tensor &a, const torch::Tensor &b, const char *what)
+{
+    TORCH_CHECK(a.scalar_type() == b.scalar_type(), what, ": floating tensors must share one dtype");
+}
+inline bool is_f64(const torch::Tensor &t) { return t.scalar_type() == torch::kFloat64; }
+inline const double *dp(const torch::Tensor &t) { return t.numel() ? t.data_ptr<double>() : nullptr; }
+inline double *dpw(torch::Tensor &t) { return t.numel() ? t.data_ptr<double>() : nullptr; }
 inline void same_device(const torch::Tensor &a, const torch::Tensor &b, const char *what)
 {
     TORCH_CHECK(a.device() == b.device(), what, ": tensors are on different devices");
@@ -108,11 +122,12 @@ inline void check_spmm_args(int fmt, const torch::Tensor &X, const torch::Tensor
     need_gpu(rowPtr, "rowPtr");
     need_gpu(colIdx, "colIdx");
     need_gpu(values, "values");
-    need_f32(X, "input", 2);
+    need_fp(X, "input", 2);
     need_i32(rowPtr, "rowPtr");
     need_i32(colIdx, "colIdx");
     const bool blocked = fmt >= 2;
-    need_f32(values, "values", blocked ? 2 : 1);
+    need_fp(values, "values", blocked ? 2 : 1);
+    same_dtype(X, values, "spmm");
     if (blocked) TORCH_CHECK(values.size(1) == 2, "values of a bcsr format must be [nblk, 2]");
     TORCH_CHECK(values.size(0) == colIdx.size(0), "values and colIdx disagree on the number of stored entries");
     check_rowptr_vs(rowPtr, "rowPtr");
@@ -137,6 +152,11 @@ inline void spmm_into(int fmt, torch::Tensor &Y, const torch::Tensor &X, const t
     const int nrows = (int)rowPtr.size(0) - 1, N = (int)X.size(1), rows_out = (int)Y.size(0);
     if (N == 0 || rows_out == 0) return;
     psp_stream_t s = stream_of(X);
+    if (is_f64(X)) {
+        ok(psp_spmm_f64(ip(rowPtr), ip(colIdx), dp(values), target_row ? ip(*target_row) : nullptr, dp(X), dpw(Y), nrows, N,
+                        rows_out, fmt >= 2 ? 2 : 1, s));
+        return;
+    }
     int rc;
     switch (fmt) {
     case 0: rc = psp_spmm_csr_f32(ip(rowPtr), ip(colIdx), fp(values), fp(X), fpw(Y), nrows, N, rows_out, CF, blkWarpNum, s); break;

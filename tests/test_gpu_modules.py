@@ -95,8 +95,11 @@ def test_extension_argument_errors():
         ParamSpMM.csr_spmm(x.cpu(), rp, ci, v, 1, 4)
     with pytest.raises(RuntimeError, match="int32"):
         ParamSpMM.csr_spmm(x, rp.long(), ci, v, 1, 4)
-    with pytest.raises(RuntimeError, match="float32"):
-        ParamSpMM.csr_spmm(x.double(), rp, ci, v.double(), 1, 4)
+    with pytest.raises(RuntimeError, match="share one dtype"):
+        ParamSpMM.csr_spmm(x.double(), rp, ci, v, 1, 4)
+    with pytest.raises(RuntimeError, match="float32 or float64"):
+        ParamSpMM.csr_spmm(x.half(), rp, ci, v.half(), 1, 4)
+    assert ParamSpMM.csr_spmm(x.double(), rp, ci, v.double(), 1, 4).dtype == torch.float64
     assert torch.count_nonzero(ParamSpMM.gespmm_compute(x, rp, ci, v)) == 0
     with pytest.raises(RuntimeError, match=r"\[nblk, 3\]"):
         ParamSDDMM.vec_sddmm(x, x, rp, ci, torch.zeros(0, 5, device="cuda"), 1, 4)
