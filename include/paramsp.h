@@ -244,6 +244,13 @@ int psp_segment_softmax_ws_f32(const int *rowPtr, const float *in, float *out, i
  * ------------------------------------------------------------------------------------------- */
 int psp_gemm_atb_supported(int K1, int K2);
 int psp_gemm_atb_f32(const float *A, const float *B, float *C, long long n, int K1, int K2, psp_stream_t stream);
+/* Same product without atomics: every workgroup stores its partial product in the caller's workspace and a second
+ * kernel adds them in a fixed order (so results repeat bit for bit, and the 20-60 us the contended atomics take are
+ * saved).  workspace: psp_gemm_atb_workspace_floats(n, K1, K2) floats of device memory, contents irrelevant on
+ * entry; 0 means the shape runs the atomic kernel and needs none. */
+long long psp_gemm_atb_workspace_floats(long long n, int K1, int K2);
+int psp_gemm_atb_ws_f32(const float *A, const float *B, float *C, long long n, int K1, int K2, float *workspace,
+                        long long workspace_floats, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: Y[n,K2] = X[n,K1] * W (transW = 0, W is [K1,K2] row-major) or X * W^T (transW != 0, W is [K2,K1]) for

@@ -36,7 +36,7 @@ class SpmmPlan(ctypes.Structure):
         return {k: getattr(self, k) for k, _ in self._fields_}
 
 
-# name -> argtypes; every entry returns int.  Keep in step with include/paramsp.h.
+# name -> argtypes; the entries return int unless RESTYPES says otherwise.  Keep in step with include/paramsp.h.
 SIGNATURES = {
     "psp_version": [],
     "psp_spmm_plan_for": [_i, _i, _i, ctypes.POINTER(SpmmPlan)],
@@ -81,12 +81,16 @@ SIGNATURES = {
     "psp_gemm_xw_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _i, _vp],
     "psp_gemm_atb_supported": [_i, _i],
     "psp_gemm_atb_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _vp],
+    "psp_gemm_atb_workspace_floats": [ctypes.c_longlong, _i, _i],
+    "psp_gemm_atb_ws_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _vp, ctypes.c_longlong, _vp],
 }
+# the entries that do not return int
+RESTYPES = {"psp_gemm_atb_workspace_floats": ctypes.c_longlong}
 
 for _name, _args in SIGNATURES.items():
     _fn = getattr(lib, _name)
     _fn.argtypes = _args
-    _fn.restype = _i
+    _fn.restype = RESTYPES.get(_name, _i)
 lib.psp_last_error.argtypes = []
 lib.psp_last_error.restype = ctypes.c_char_p
 

@@ -35,7 +35,11 @@ static Tensor weight_gradient(const Tensor &H, const Tensor &AG)
     Tensor Hc = H.contiguous(), Gc = AG.contiguous();
     DeviceGuard guard(Hc.device());
     Tensor dW = torch::empty({Hc.size(1), Gc.size(1)}, Hc.options());
-    ok(psp_gemm_atb_f32(fp(Hc), fp(Gc), fpw(dW), Hc.size(0), (int)Hc.size(1), (int)Gc.size(1), stream_of(Hc)));
+    // partial products of the workgroups go through a workspace and are added in a fixed order (no atomics)
+    const long long ws_floats = psp_gemm_atb_workspace_floats(Hc.size(0), (int)Hc.size(1), (int)Gc.size(1));
+    Tensor ws = torch::empty({(long)ws_floats}, Hc.options());
+    ok(psp_gemm_atb_ws_f32(fp(Hc), fp(Gc), fpw(dW), Hc.size(0), (int)Hc.size(1), (int)Gc.size(1), fpw(ws), ws_floats,
+                           stream_of(Hc)));
     return dW;
 }
 

@@ -226,7 +226,8 @@ def test_training_driver_runs_gcn_gin_agnn():
         assert all(ms > 0 for ms in res.values())
 
 
-@pytest.mark.parametrize("K1,K2", [(16, 16), (32, 16), (16, 64), (48, 32), (64, 64), (128, 128), (112, 16), (32, 128)])
+@pytest.mark.parametrize("K1,K2", [(16, 16), (32, 16), (16, 64), (48, 32), (64, 64), (128, 128), (112, 16), (32, 128), (64, 128), (128, 64),
+                                   (48, 80), (16, 128), (96, 96), (112, 128), (80, 64)])
 def test_tall_skinny_weight_gradient_product(K1, K2):
     """psp_gemm_atb_f32 (the H^T * AG of the fused GCN backward) against a float64 product; n is not a multiple
     of the 64-row tile and the output is poisoned first."""
@@ -243,6 +244,18 @@ def test_tall_skinny_weight_gradient_product(K1, K2):
     want = A.double().t() @ B.double()
     # fp32 accumulation over 70k terms of magnitude ~1: error ~ sqrt(n) * eps * |terms|
     torch.testing.assert_close(C.double(), want, rtol=1e-4, atol=2e-2)
+    # the workspace variant: same product, partial sums added in a fixed order, so two runs agree bit for bit
+    ws_floats = _capi.lib.psp_gemm_atb_workspace_floats(n, K1, K2)
+    ws = torch.full((max(ws_floats, 1),), float("nan"), device="cuda")
+    C2 = torch.full((K1, K2), float("nan"), device="cuda")
+    C3 = torch.full((K1, K2), float("nan"), device="cuda")
+    st = torch.cuda.current_stream().cuda_stream
+    _capi.check(_capi.lib.psp_gemm_atb_ws_f32(p(A), p(B), p(C2), n, K1, K2, p(ws), ws_floats, st))
+    _capi.check(_capi.lib.psp_gemm_atb_ws_f32(p(A), p(B), p(C3), n, K1, K2, p(ws), ws_floats, st))
+    torch.testing.assert_close(C2.double(), want, rtol=1e-4, atol=2e-2)
+    if ws_floats:
+        assert torch.equal(C2, C3)
+        assert _capi.lib.psp_gemm_atb_ws_f32(p(A), p(B), p(C2), n, K1, K2, p(ws), ws_floats - 1, None) == -1
     assert _capi.lib.psp_gemm_atb_f32(p(A), p(B), p(C), n, K1, 20, None) == -1
     _capi.check(_capi.lib.psp_gemm_atb_f32(p(A), p(B), p(C), 0, K1, K2, None))
     torch.cuda.synchronize()
