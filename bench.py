@@ -234,7 +234,25 @@ def bench_sddmm(args):
         dt = _t.perf_counter() - t0
         cpu = {"value": round(2.0 * take * K / dt / 1e9, 3), "unit": "GFLOP/s", "cores": 1, "kind": "port",
                "sample": "oracle orc_sddmm_csr (scalar C) on the first %d rows (%d stored entries) of the same graph, K = 64, one pass (%.1f s)" % (m, take, dt)}
-    print(json.dumps({"cpu_baseline": cpu, "metric": "SDDMM GFLOP/s (2*nnz*K) over K = 16..128", "value": round(value, 1), "unit": "GFLOP/s",
+        # beside it, the gathered product in torch on all host threads (a dense [n, n] mask is impossible at this size)
+        rows_h = torch.from_numpy(np.repeat(np.arange(m, dtype=np.int64), np.diff(rowPtr[:m + 1])))
+        cols_h = torch.from_numpy(colIdx[:take].astype(np.int64))
+        At, Bt = torch.from_numpy(Ah), torch.from_numpy(Bh)
+
+        def torch_once():
+            o = torch.empty(take)
+            for s0 in range(0, take, 1 << 18):
+                sl = slice(s0, min(take, s0 + (1 << 18)))
+                o[sl] = (At[rows_h[sl]] * Bt[cols_h[sl]]).sum(1)
+            return o
+        torch_once()
+        t0, reps = _t.perf_counter(), 0
+        while reps < 3 or _t.perf_counter() - t0 < 3.0:
+            torch_once()
+            reps += 1
+        cpu_torch = {"value": round(2.0 * take * K * reps / (_t.perf_counter() - t0) / 1e9, 2), "unit": "GFLOP/s",
+                     "cores": torch.get_num_threads()}
+    print(json.dumps({"cpu_baseline": cpu, "cpu_torch_gathered": cpu_torch if cpu else None, "metric": "SDDMM GFLOP/s (2*nnz*K) over K = 16..128", "value": round(value, 1), "unit": "GFLOP/s",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(total_ms, 4),
                       "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
                       "config": {"workload": "%s SDDMM width sweep" % args.graph, "nodes": n, "nnz": nnz}, "per_K": per_K}))
