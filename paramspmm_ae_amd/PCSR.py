@@ -270,3 +270,131 @@ class pcsr_spmm(object):
         return SpMM.spmm_time_ms(fmt, X, self.rowPtr, self.colIdx, self.val, self.target_row,
                                  self.CF if CF is None else CF, self.blkWarpNum if blkWarpNum is None else blkWarpNum,
                                  warmup, iters)
+
+
+# ---- training-set construction: `python -m paramspmm_ae_amd.PCSR` (PCSR.py:660-871) -----------------------------
+def get_mtx_info(filelist, path, dim=32, if_auto_gran=True, blk_size=2):
+    """One row of the 15 decider features per ``<path>/<name>.mtx`` (PCSR.py:660-669)."""
+    import pandas as pd
+
+    from .graph_input import graph_input
+
+    frames = []
+    for name in filelist:
+        graph = graph_input(mtx_name=name, path=path)
+        graph.load(load_from_mtx=True, is_avg_granularity=not if_auto_gran, blk_size=blk_size)
+        frames.append(graph.mtxinfo_to_pandas())
+    return pd.concat(frames, axis=0, ignore_index=True) if frames else pd.DataFrame()
+
+
+def profile_engine(filelist, path, dim_list, vec_size=2, if_DCP=True, if_auto_gran=True, verbose=True):
+    """({dim: GFLOP/s table}, {dim: baseline table}) over the matrices of ``filelist`` (PCSR.py:672-806).
+
+    Every swept configuration and both baselines are first checked against ``torch.sparse.mm`` with X = ones; the
+    columns run blkWarpNum-major, then CF, then vec1 / vec1_split / vecV / vecV_split, so the index of the best
+    column is the decider's class code.  ``if_DCP`` False sweeps CF 1..ceil(dim/32) without the gap rule."""
+    import numpy as np
+    import pandas as pd
+
+    from . import sweep as sw
+    from .graph_input import graph_input
+    from .verification import SpMM_verification
+
+    cfs = {d: dynamic_CF_prompter(d) if if_DCP else list(range(1, 9))[: math.ceil(d / 32)] for d in dim_list}
+    tp = {d: [] for d in dim_list}
+    base = {d: [] for d in dim_list}
+    for name in filelist:
+        if verbose:
+            print("-------------{}-------------".format(name))
+        graph = graph_input(mtx_name=name, path=path)
+        graph.verbose = verbose
+        graph.load(load_from_mtx=True, is_avg_granularity=not if_auto_gran, blk_size=vec_size)
+        c = graph.csr_data
+        check = SpMM_verification(dim_list[0], c.rowPtr, c.colIdx, c.val, baseline=True)
+        ops = sw.operators_of(graph, vec_size)
+        for d in dim_list:
+            check.reference(d, verbose=False)
+            check.compare(ops[0].cusparse_ref(d), name, verbose)
+            check.compare(ops[0].gespmm_ref(d), name, verbose)
+            base[d].append([ops[0].cusparse_ref(d, is_profiling=True, verbose=verbose),
+                            ops[0].gespmm_ref(d, is_profiling=True, verbose=verbose)])
+            _, gflops = sw.sweep_dim(ops, d, graph.mtx_edges, graph.mtx_nodes, cfs=cfs[d],
+                                     verify=lambda y, col: check.compare(y.to("cpu"), "%s %s" % (name, col), False))
+            tp[d].append(gflops)
+        del ops, graph
+        torch.cuda.empty_cache()
+    tables = {d: pd.DataFrame(np.array(tp[d]).reshape(len(filelist), -1), columns=sw.column_names(d, cfs[d], vec_size))
+              for d in dim_list}
+    baselines = {d: pd.DataFrame(np.array(base[d], dtype=np.float64).reshape(len(filelist), 2), columns=["cusparse", "gespmm"])
+                 for d in dim_list}
+    return tables, baselines
+
+
+def training_data_gen(dim_list, vec_size, info_df, filelist, path, csv_path, if_DCP=True, if_auto_gran=True, verbose=True):
+    """Writes ``dim<d>.csv``, ``dim<d>_OP_SpMM.csv`` (features + best column) and ``dim<d>_baseline.csv`` under
+    ``csv_path`` (PCSR.py:809-824): the files ``train_decider fit --data csv_path`` reads."""
+    import os
+
+    import pandas as pd
+
+    tables, baselines = profile_engine(filelist, path, dim_list, vec_size, if_DCP, if_auto_gran, verbose)
+    os.makedirs(csv_path, exist_ok=True)
+    for d in dim_list:
+        tables[d].to_csv(os.path.join(csv_path, "dim%d.csv" % d), index=False)
+        best = pd.DataFrame({"OP_SpMM": tables[d].to_numpy().argmax(axis=1)})
+        pd.concat([info_df.reset_index(drop=True), best], axis=1).to_csv(os.path.join(csv_path, "dim%d_OP_SpMM.csv" % d), index=False)
+        baselines[d].to_csv(os.path.join(csv_path, "dim%d_baseline.csv" % d), index=False)
+    return tables, baselines
+
+
+def main(argv=None):
+    import argparse
+    import glob
+    import os
+
+    import pandas as pd
+
+    flag = dict(type=str, choices=["True", "False"])
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--path", type=str, default="./toy_dataset/", help="path to the mtx files")
+    parser.add_argument("--dim_list", nargs="*", type=int, default=list(range(16, 257, 16)), help="dim_list for training data generation")
+    parser.add_argument("--vec_size", type=int, default=2, help="vec_size(besides 1) for SpMM")
+    parser.add_argument("--if_DCP", default="True", help="If to use DCP", **flag)
+    parser.add_argument("--if_reorder", default="True", help="If to use graph reordering (the path must then name a rabbit-ordered set)", **flag)
+    parser.add_argument("--if_auto_gran", default="True", help="If to use auto-Granularity, else use avg_row_nnz as split-granularity", **flag)
+    parser.add_argument("--approx_eval", default="False", help="accepted for compatibility; unused in the reference as well", **flag)
+    parser.add_argument("--csv_path", type=str, default=None, help="where the tables go (default: the reference's ./ParamSpMM-log/ tree)")
+    args = parser.parse_args(argv)
+    print(args)
+    if_DCP, if_auto_gran, if_reorder = args.if_DCP == "True", args.if_auto_gran == "True", args.if_reorder == "True"
+    # the reference's output tree (PCSR.py:846-866)
+    if if_DCP and if_auto_gran:
+        csv_path = "./ParamSpMM-log/"
+    elif if_DCP:
+        csv_path = "./ParamSpMM-log/ablation_study/auto-Gran/"
+    elif if_auto_gran:
+        csv_path = "./ParamSpMM-log/ablation_study/woDCP/"
+    else:
+        raise ValueError("input if_DCP and if_auto_gran options are not supported")
+    if if_reorder:
+        assert "rabbit" in args.path, "--if_reorder True expects a path of rabbit-ordered matrices"
+    else:
+        assert "rabbit" not in args.path
+        csv_path = "./ParamSpMM-log/ablation_study/wo_reorder/"
+    if args.vec_size != 2:
+        csv_path = "./ParamSpMM-log/ablation_study/vec_size%d/" % args.vec_size
+    if args.csv_path is not None:
+        csv_path = args.csv_path
+    os.makedirs(csv_path, exist_ok=True)
+    filelist = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(args.path, "*.mtx")))
+    info_file = os.path.join(csv_path, "mtx_info.csv")
+    if os.path.exists(info_file):
+        info_df = pd.read_csv(info_file)
+    else:
+        info_df = get_mtx_info(filelist, args.path, if_auto_gran=if_auto_gran, blk_size=args.vec_size)
+        info_df.to_csv(info_file, index=False)
+    return training_data_gen(args.dim_list, args.vec_size, info_df, filelist, args.path, csv_path, if_DCP, if_auto_gran)
+
+
+if __name__ == "__main__":
+    main()

@@ -12,8 +12,11 @@ WARP_NUMS = (4, 8)
 REPRESENTATIONS = (("vec1", 1, False), ("vec1_split", 1, True), ("vec2", 2, False), ("vec2_split", 2, True))
 
 
-def column_names(dim):
-    return ["%s_TP_%d%d" % (rep, cf, bw) for bw in WARP_NUMS for cf in dynamic_CF_prompter(dim) for rep, _, _ in REPRESENTATIONS]
+def column_names(dim, cfs=None, vec_size=2):
+    """``cfs``: the CF list when it is not ``dynamic_CF_prompter(dim)`` (the reference's --if_DCP False ablation)"""
+    cfs = dynamic_CF_prompter(dim) if cfs is None else cfs
+    reps = ("vec1", "vec1_split", "vec%d" % vec_size, "vec%d_split" % vec_size)
+    return ["%s_TP_%d%d" % (rep, cf, bw) for bw in WARP_NUMS for cf in cfs for rep in reps]
 
 
 def decode_column(dim, col):
@@ -25,29 +28,35 @@ def decode_column(dim, col):
     return int(if_split), vec_size, cf, bw
 
 
-def operators_of(graph):
+def operators_of(graph, vec_size=2):
     """The four representations of a loaded graph_input on the GPU, in column order."""
-    return [pcsr_spmm(graph, vec_size=v, if_split=s) for _, v, s in REPRESENTATIONS]
+    return [pcsr_spmm(graph, vec_size=v if v == 1 else vec_size, if_split=s) for _, v, s in REPRESENTATIONS]
 
 
-def sweep_dim(ops, dim, nnz, n_rows, warmup=3, iters=10, X=None, verify=None):
+def sweep_dim(ops, dim, nnz, n_rows, warmup=3, iters=10, X=None, verify=None, cfs=None):
     """Times all columns for one width.  Returns (ms[cols], gflops[cols]).
 
     ``verify``: optional callable(result_tensor, column_name) run once per column on A*X before timing
     (the reference verifies every swept configuration, PCSR.py:759-770).
     """
-    rows = (n_rows + 1) // 2 * 2
+    pad = max(op.vec_size for op in ops)
+    pad = 2 if pad == 1 else pad
+    rows = (n_rows + pad - 1) // pad * pad
     if X is None:
         X = torch.ones(rows, dim, device="cuda")
-    names = column_names(dim)
+    cfs = dynamic_CF_prompter(dim) if cfs is None else cfs
+    names = column_names(dim, cfs, ops[-1].vec_size if ops[-1].vec_size != 1 else 2)
     ms = np.zeros(len(names))
     col = 0
     for bw in WARP_NUMS:
-        for cf in dynamic_CF_prompter(dim):
+        for cf in cfs:
             for op in ops:
                 if verify is not None:
                     verify(op._spmm(X, CF=cf, blkWarpNum=bw)[:n_rows], names[col])
-                ms[col] = op.time_ms(X, CF=cf, blkWarpNum=bw, warmup=warmup, iters=iters)
+                if op.vec_size == 3:  # the generic-block operators have no event-timed twin: use their *_profile
+                    ms[col] = 2.0 * nnz * dim / 1e6 / max(op.cf_warpnum_profiling(cf, bw, x=X, verbose=False), 1)
+                else:
+                    ms[col] = op.time_ms(X, CF=cf, blkWarpNum=bw, warmup=warmup, iters=iters)
                 col += 1
     gflops = 2.0 * nnz * dim / 1e6 / ms
     return ms, gflops

@@ -1,6 +1,9 @@
 """GPU tests of the PyTorch extension modules (ParamSpMM / ParamSDDMM / ParamSpCONV), the pcsr_spmm facade,
 the format builder with its device-side mask, and the GNN layers against dense torch autograd."""
+import os
+
 import numpy as np
+import pandas as pd
 import pytest
 import torch
 
@@ -384,3 +387,72 @@ def test_dense_xw_matches_torch(K1, K2):
     # few rows: torch::mm path, same answer
     small = ParamSpCONV.dense_xw(X[:100].contiguous(), W, False)
     assert torch.all((small.double() - want[:100]).abs() <= 1e-5 * scale[:100] + 1e-6)
+
+
+@pytest.mark.parametrize("vec_size", [2, 3])
+def test_sddmm_sweep_harness(tmp_path, vec_size):
+    """SDDMM.py's facade and sweep (SDDMM.py:46-383) on the reference's pubmed pattern read from a .mtx file and on a
+    synthetic graph: every variant is verified against the vendor result inside the sweep (ones -> dim per entry),
+    the tables have the reference's column order, and the vendor call leaves the shared value array alone."""
+    import scipy.io
+    import scipy.sparse as sp
+    from conftest import pubmed_pattern
+    from paramspmm_ae_amd import SDDMM as S
+
+    scipy.io.mmwrite(str(tmp_path / "pm.mtx"), sp.tril(pubmed_pattern("orig")).tocoo(), symmetry="symmetric")
+    tables = S.main(["--path", str(tmp_path) + os.sep, "--mtx_name", "pm", "--dim_list", "32", "48", "--vec_size",
+                     str(vec_size), "--csv_path", str(tmp_path / "log") + os.sep])
+    assert sorted(tables) == [32, 48]
+    names = ["vec1_TP_4", "vec1_split_TP_4", "vec%d_TP_4" % vec_size, "vec%d_split_TP_4" % vec_size,
+             "vec1_TP_8", "vec1_split_TP_8", "vec%d_TP_8" % vec_size, "vec%d_split_TP_8" % vec_size]
+    for dim, tp in tables.items():
+        assert list(tp.columns) == names and tp.shape == (1, 8) and bool((tp.to_numpy() > 0).all())
+        best = pd.read_csv(tmp_path / "log" / ("dim%d_OP_SpMM.csv" % dim))
+        assert best.shape == (1, 17) and int(best["OP_SpMM"][0]) == int(tp.to_numpy().argmax())
+    # synthetic graph, facade by hand
+    g = S._load("C1", None, True, 2, True)
+    op = S.pcsr_sddmm(g, vec_size=1, if_split=False)
+    before = op.val.clone()
+    want = op.cusparse_ref(64)
+    assert torch.equal(op.val, before) and bool((want == 64).all())
+    S.compare(op.get_sddmm_result(64, 8), want, verbose=False)
+    blocked = S.pcsr_sddmm(g, vec_size=2, if_split=True)
+    S.compare_2d(blocked.get_sddmm_result(64, 4), want, blocked.mask, verbose=False)
+    assert op.cusparse_ref(64, is_profiling=True, verbose=False) > 0 and blocked.profiling(4, 64, verbose=False) > 0
+    with pytest.raises(ValueError, match="cusparse only support"):
+        blocked.cusparse_ref(64)
+    with pytest.raises(ValueError, match="Verification FAILED"):
+        S.compare(want + 1.0, want, verbose=False)
+
+
+def test_training_set_construction_from_mtx_files(tmp_path):
+    """`python PCSR.py` of the reference (PCSR.py:660-871): features, the swept GFLOP/s table in class-code order, the
+    best column and the vendor baselines, written as the csv files the decider training reads; every configuration
+    is verified against torch.sparse.mm on the way."""
+    import scipy.io
+    import scipy.sparse as sp
+    from conftest import pubmed_pattern
+    from paramspmm_ae_amd import PCSR as P
+
+    d = tmp_path / "rabbit"
+    d.mkdir()
+    scipy.io.mmwrite(str(d / "pm.mtx"), sp.tril(pubmed_pattern("rabbit")).tocoo(), symmetry="symmetric")
+    out = str(tmp_path / "log") + os.sep
+    tables, baselines = P.main(["--path", str(d) + os.sep, "--dim_list", "16", "80", "--csv_path", out])
+    for dim in (16, 80):
+        cfs = P.dynamic_CF_prompter(dim)
+        tp = pd.read_csv(out + "dim%d.csv" % dim)
+        assert tp.shape == (1, 8 * len(cfs)) and bool((tp.to_numpy() > 0).all())
+        # blkWarpNum-major, then CF, then the four representations: the order decode_tree relies on
+        assert list(tp.columns) == ["%s_TP_%d%d" % (rep, cf, bw) for bw in (4, 8) for cf in cfs
+                                    for rep in ("vec1", "vec1_split", "vec2", "vec2_split")]
+        lab = pd.read_csv(out + "dim%d_OP_SpMM.csv" % dim)
+        assert lab.shape == (1, 17) and int(lab["OP_SpMM"][0]) == int(tp.to_numpy().argmax())
+        b = pd.read_csv(out + "dim%d_baseline.csv" % dim)
+        assert list(b.columns) == ["cusparse", "gespmm"] and bool((b.to_numpy() > 0).all())
+    # without the gap rule dim 80 sweeps CF 1..3
+    t2, _ = P.profile_engine(["pm"], str(d) + os.sep, [80], if_DCP=False, verbose=False)
+    assert t2[80].shape == (1, 8 * 3)
+    # 3x1 blocks in place of 2x1
+    t3, _ = P.profile_engine(["pm"], str(d) + os.sep, [32], vec_size=3, verbose=False)
+    assert list(t3[32].columns)[2:4] == ["vec3_TP_14", "vec3_split_TP_14"] and bool((t3[32].to_numpy() > 0).all())
