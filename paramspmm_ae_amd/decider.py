@@ -60,3 +60,83 @@ class SpMMDecider(object):
             raise ValueError("dim-" + str(dim) + " not found in model_dict")
         code = self.model_dict[dim].predict(graph.get_info()).item()
         return self.decode_tree(code, math.ceil(dim / 16) * 16)
+
+
+def evaluate(filelist, path, dim_list, pickle_path=DEFAULT_PICKLE_PATH, verbose=True):
+    """The reference's evaluation run (decider.py:97-175): for every matrix and width the decider's configuration is
+    verified against ``torch.sparse.mm`` and then timed beside the vendor library (COO, CSC and CSR formats) and the
+    row-caching baseline.  ``path`` None takes ``filelist`` as names of the seeded
+    synthetic graphs.  Returns one row per (matrix, width) with the GFLOP/s of each."""
+    import pandas as pd
+    import torch
+
+    from .PCSR import coo_spmm, csc_spmm, pcsr_spmm
+    from .graph_input import graph_input
+    from .verification import SpMM_verification
+
+    decider = SpMMDecider(pickle_path)
+    decider.gen_model_dict(dim_list)
+    rows = []
+    for name in filelist:
+        if verbose:
+            print("-------------mtx: {}-------------".format(name))
+        graph = graph_input(mtx_name=name, path=path or "")
+        graph.verbose = verbose
+        if path is None:
+            from . import synth
+
+            rowPtr, colIdx, val, _ = synth.config_graph(name)
+            graph.load_from_csr(rowPtr, colIdx, val, if_mask=True)
+        else:
+            graph.load(load_from_mtx=True, if_mask=True)
+        c = graph.csr_data
+        check = SpMM_verification(1, c.rowPtr, c.colIdx, c.val, baseline=True)
+        coo, csc = coo_spmm(graph), csc_spmm(graph)
+        plain = pcsr_spmm(graph, vec_size=1, if_split=False)
+        for dim in dim_list:
+            check.reference(dim, verbose=False)
+            if_split, vec_size, CF, blkWarpNum = decider.config_PCSR(graph, dim)
+            op = pcsr_spmm(graph=graph, vec_size=vec_size, if_split=if_split, CF=CF, blkWarpNum=blkWarpNum)
+            op.get_spmm_result(dim)
+            check.compare(op.result, name, verbose)
+            rows.append({"mtx_name": name, "dim": dim, "if_split": int(if_split), "vec_size": vec_size, "CF": CF,
+                         "blkWarpNum": blkWarpNum, "param": op.profiling(dim, verbose=verbose),
+                         "coo": coo.profiling(dim, verbose=verbose), "csc": csc.profiling(dim, verbose=verbose),
+                         "cusparse": plain.cusparse_ref(dim, is_profiling=True, verbose=verbose),
+                         "gespmm": plain.gespmm_ref(dim, is_profiling=True, verbose=verbose)})
+            if verbose:
+                print("=======================================")
+        del coo, csc, plain, graph
+        torch.cuda.empty_cache()
+    return pd.DataFrame(rows)
+
+
+def main(argv=None):
+    import argparse
+    import glob
+
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--path", type=str, default="./dataset/all-mtx/", help="path to the mtx files")
+    parser.add_argument("--dim_list", nargs="*", type=int, default=[16, 32, 48, 64, 80, 96, 112, 128])
+    parser.add_argument("--mtx_name", type=str, default="", help="mtx file name")
+    parser.add_argument("--pickle_path", type=str, default=DEFAULT_PICKLE_PATH, help="directory of rnd_tree_<dim>.pkl")
+    parser.add_argument("--synthetic", nargs="*", default=None, help="seeded synthetic graphs (C1, C2, ...) instead of mtx files")
+    args = parser.parse_args(argv)
+    print(args)
+    if args.synthetic:
+        path, filelist = None, list(args.synthetic)
+    elif args.mtx_name:
+        path, filelist = args.path, [args.mtx_name]
+    else:
+        path = args.path
+        filelist = sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(path, "*.mtx")))
+    table = evaluate(filelist, path, args.dim_list, args.pickle_path)
+    if len(table):
+        print(table.to_string(index=False))
+        ratio = table["param"] / table["cusparse"].clip(lower=1)
+        print("geometric-mean speedup over the vendor CSR SpMM: %.2f" % math.exp(ratio.apply(math.log).mean()))
+    return table
+
+
+if __name__ == "__main__":
+    main()

@@ -456,3 +456,19 @@ def test_training_set_construction_from_mtx_files(tmp_path):
     # 3x1 blocks in place of 2x1
     t3, _ = P.profile_engine(["pm"], str(d) + os.sep, [32], vec_size=3, verbose=False)
     assert list(t3[32].columns)[2:4] == ["vec3_TP_14", "vec3_split_TP_14"] and bool((t3[32].to_numpy() > 0).all())
+
+
+def test_decider_evaluation_run(tmp_path):
+    """decider.py's command line (decider.py:97-175): the pick of the shipped forests is verified and timed beside
+    the four baselines, on a .mtx file and on a synthetic graph."""
+    import scipy.io
+    import scipy.sparse as sp
+    from conftest import pubmed_pattern
+    from paramspmm_ae_amd import decider as D
+
+    scipy.io.mmwrite(str(tmp_path / "pm.mtx"), sp.tril(pubmed_pattern("orig")).tocoo(), symmetry="symmetric")
+    t = D.main(["--path", str(tmp_path) + os.sep, "--mtx_name", "pm", "--dim_list", "16", "96"])
+    assert list(t["dim"]) == [16, 96] and bool((t[["param", "coo", "csc", "cusparse", "gespmm"]].to_numpy() > 0).all())
+    assert set(t["vec_size"]) <= {1, 2} and set(t["blkWarpNum"]) <= {4, 8}
+    t2 = D.evaluate(["C1"], None, [32], verbose=False)
+    assert t2.shape[0] == 1 and t2["param"][0] > 0
