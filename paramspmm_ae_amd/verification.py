@@ -58,3 +58,35 @@ class SpMM_verification(object):
             print("Mismatch at position ({}, {}): Expected {}, Found {}".format(
                 row, col, self.result_ref[row, col].item(), result[row, col].item()))
         raise ValueError("Verification FAILED in {}".format(mtx_name))
+
+
+def main(argv=None):
+    """torch.sparse.mm on the CPU and on the GPU for every matrix of a directory (verification.py:105-128)."""
+    import argparse
+    import glob
+    import os
+
+    from .graph_input import graph_input
+
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--path", type=str, default="./artifact_dataset/all-mtx/rabbit/", help="path to the mtx files")
+    parser.add_argument("--dim", type=int, default=32)
+    args = parser.parse_args(argv)
+    out = {}
+    for name in sorted(os.path.basename(f)[:-4] for f in glob.glob(os.path.join(args.path, "*.mtx"))):
+        print("-------------{}-------------".format(name))
+        graph = graph_input(mtx_name=name, path=args.path)
+        graph.load(load_from_mtx=True)
+        c = graph.csr_data
+        check = SpMM_verification(args.dim, c.rowPtr, c.colIdx, c.val, baseline=True)
+        check.reference()
+        _, cpu = check.torch_compute("cpu")
+        got, gpu = check.torch_compute("cuda")
+        check.compare(got.to("cpu"), name)
+        out[name] = (cpu, gpu)
+        print("=======================================")
+    return out
+
+
+if __name__ == "__main__":
+    main()

@@ -472,3 +472,8 @@ def test_decider_evaluation_run(tmp_path):
     assert set(t["vec_size"]) <= {1, 2} and set(t["blkWarpNum"]) <= {4, 8}
     t2 = D.evaluate(["C1"], None, [32], verbose=False)
     assert t2.shape[0] == 1 and t2["param"][0] > 0
+    # verification.py's own command line on the same directory
+    from paramspmm_ae_amd import verification as V
+
+    res = V.main(["--path", str(tmp_path) + os.sep, "--dim", "16"])
+    assert list(res) == ["pm"] and res["pm"][0] > 0 and res["pm"][1] > 0
