@@ -477,3 +477,26 @@ def test_decider_evaluation_run(tmp_path):
 
     res = V.main(["--path", str(tmp_path) + os.sep, "--dim", "16"])
     assert list(res) == ["pm"] and res["pm"][0] > 0 and res["pm"][1] > 0
+
+
+@pytest.mark.parametrize("n", [1, 5, 63, 64, 257, 4099])
+@pytest.mark.parametrize("K1,K2", [(16, 16), (64, 64), (128, 128), (96, 96)])
+def test_weight_gradient_product_small_row_counts(n, K1, K2):
+    """row counts around the kernels' chunk sizes (4-row groups, 8 / 16 / 32-row chunks, fewer chunks than wavefronts)"""
+    from paramspmm_ae_amd import _capi
+
+    g = torch.Generator(device="cuda").manual_seed(n)
+    A = torch.randn(n, K1, device="cuda", generator=g)
+    B = torch.randn(n, K2, device="cuda", generator=g)
+    p = _capi.ptr
+    st = torch.cuda.current_stream().cuda_stream
+    want = A.double().t() @ B.double()
+    ws_floats = _capi.lib.psp_gemm_atb_workspace_floats(n, K1, K2)
+    ws = torch.full((max(ws_floats, 1),), float("nan"), device="cuda")
+    for entry in ("ws", "atomic"):
+        C = torch.full((K1, K2), float("nan"), device="cuda")
+        if entry == "ws":
+            _capi.check(_capi.lib.psp_gemm_atb_ws_f32(p(A), p(B), p(C), n, K1, K2, p(ws), ws_floats, st))
+        else:
+            _capi.check(_capi.lib.psp_gemm_atb_f32(p(A), p(B), p(C), n, K1, K2, st))
+        torch.testing.assert_close(C.double(), want, rtol=1e-4, atol=1e-3)
