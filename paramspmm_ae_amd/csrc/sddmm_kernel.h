@@ -64,6 +64,12 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
     constexpr int R = PSP_WAVE >> LOGL;
     static_assert(U <= L, "unroll must not exceed the group width");
     __shared__ int2 s_seg[PSP_MAX_WAVES][PSP_WAVE];  // (end offset, A row) of the wavefront's filled segments
+    // CSR results of narrow groups wait here until the group has 32 of them (a 128-byte line of `out`) and then leave
+    // in one burst of stores: a group stores only L floats at a time, and lines written piecemeal are evicted from the
+    // L2 half-written by the gather stream (measured: 3x the result's bytes in HBM writes at L = 4).
+    // 2x1 blocks hold pairs (16 blocks to a line); 3x1 blocks are stored directly.
+    constexpr int HOLD = (NR <= 2 && LOGL >= 2 && LOGL + NR <= 5) ? ((32 / NR) >> LOGL) : 1;  // chunks held back per group
+    __shared__ __align__(8) float s_hold[HOLD > 1 ? PSP_MAX_WAVES : 1][HOLD > 1 ? HOLD * PSP_WAVE * NR : 1];
 
     const int tile = psp_xcd_tile(stripe);
     if (tile >= tiles) return;
@@ -172,6 +178,21 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
     int c_cur;
     float gate[NR];
     fetch(a0, c_cur, gate);
+    int held = 0;         // chunks waiting in s_hold (group-uniform)
+    int hold_base = a0;   // entry of the first of them
+    // every lane reads back what it wrote itself, so the wavefront's program order is all the ordering needed
+    auto release = [&]() {
+#pragma unroll
+        for (int j = 0; j < HOLD; j++) {
+            const int pp = hold_base + (j << LOGL) + sub;
+            if (j < held && pp < b0) {
+                if constexpr (NR == 2) ((psp_f32x2 *)out)[pp] = ((const psp_f32x2 *)s_hold[wave])[j * PSP_WAVE + lane];
+                else out[pp] = s_hold[wave][j * PSP_WAVE + lane];
+            }
+        }
+        hold_base += held << LOGL;
+        held = 0;
+    };
 
     for (int base = a0; base < b0; base += L) {
         const int p = base + sub;
@@ -237,7 +258,7 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
             }
         }
         if (ok) {
-            if constexpr (NR == 2) {
+            if constexpr (NR == 2 && HOLD == 1) {
                 // entries of a block whose value is zero are padding: written as zero (sddmm_kernel.cu:1103,1115)
                 psp_f32x2 o;
                 o[0] = gate[0] != 0.0f ? res[0] : 0.0f;
@@ -246,14 +267,26 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
             } else if constexpr (NR > 2) {
 #pragma unroll
                 for (int r = 0; r < NR; r++) out[(size_t)p * NR + r] = gate[r] != 0.0f ? res[r] : 0.0f;
-            } else {
+            } else if constexpr (HOLD == 1) {
                 out[p] = SCALE ? res[0] * gate[0] : res[0];
             }
+        }
+        if constexpr (HOLD > 1) {
+            if constexpr (NR == 2) {
+                psp_f32x2 o;  // padding entries of a block (value zero) are written as zero (sddmm_kernel.cu:1103,1115)
+                o[0] = gate[0] != 0.0f ? res[0] : 0.0f;
+                o[1] = gate[1] != 0.0f ? res[1] : 0.0f;
+                ((psp_f32x2 *)s_hold[wave])[held * PSP_WAVE + lane] = o;
+            } else {
+                s_hold[wave][held * PSP_WAVE + lane] = SCALE ? res[0] * gate[0] : res[0];
+            }
+            if (++held == HOLD) release();
         }
         c_cur = c_nxt;
 #pragma unroll
         for (int r = 0; r < NR; r++) gate[r] = gate_nxt[r];
     }
+    if constexpr (HOLD > 1) release();
     if (want_max) emit_row_max(mykey);
 }
 
