@@ -184,6 +184,8 @@ int psp_spmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b, const floa
  * kernels never multiply them in, SDDMM/sddmm_kernel.cu:917-983).  A and B are [*, K] row-major.
  * `scale` may be NULL; when given (an extension of this library used by the attention benchmark) the result
  * is multiplied by scale[p] (csr) -- pass NULL for the reference semantics.
+ * colIdx, out and the block values may all be NULL for a matrix without stored entries (an empty device
+ * allocation has no address, and only rowPtr -- on the device -- says whether there are any).
  * ------------------------------------------------------------------------------------------- */
 
 /* ParamSDDMM.csr_sddmm, SDDMM/sddmm.cpp:15-65 -> sddmm_kernel.cu:143-192, 917-983.  out[nnz]. */

@@ -117,8 +117,10 @@ PSP_EXPORT int psp_sddmm_f64(const int *rowPtr, const int *colIdx, const double 
     PSP_REQUIRE(nseg >= 0 && K >= 1, "sddmm_f64: bad size (segments %d, K %d)", nseg, K);
     PSP_REQUIRE(vec_size >= 1 && vec_size <= 3, "sddmm_f64: vec_size must be 1, 2 or 3 (got %d)", vec_size);
     if (nseg == 0) return PSP_OK;
-    PSP_REQUIRE(rowPtr && colIdx && A && B && out, "sddmm_f64: null pointer");
-    PSP_REQUIRE(vec_size == 1 || val_b, "sddmm_f64: block values are null");
+    // colIdx, out and the block values may be null for a matrix without stored entries (only rowPtr, on the device, tells)
+    PSP_REQUIRE(rowPtr && A && B, "sddmm_f64: null pointer");
+    PSP_REQUIRE((colIdx != nullptr) == (out != nullptr), "sddmm_f64: colIdx and out must both be given (or both be null for a matrix without entries)");
+    PSP_REQUIRE(vec_size == 1 || val_b || !colIdx, "sddmm_f64: block values are null");
     hipStream_t st = (hipStream_t)stream;
     if (vec_size == 1) return sddmm_f64_launch<1>(rowPtr, colIdx, val_b, target_row, A, B, out, nseg, K, st);
     if (vec_size == 2) return sddmm_f64_launch<2>(rowPtr, colIdx, val_b, target_row, A, B, out, nseg, K, st);

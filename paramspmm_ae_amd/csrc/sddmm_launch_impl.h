@@ -11,9 +11,12 @@ int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, con
     PSP_REQUIRE(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8");
     PSP_REQUIRE(nrows >= 0 && K >= 1, "sddmm: bad size (rows %d, K %d)", nrows, K);
     if (nrows == 0) return PSP_OK;
-    PSP_REQUIRE(rowPtr && colIdx && A && B && out, "sddmm: null pointer");
+    // colIdx, out and the block values may be null for a matrix without stored entries: whether there are any is
+    // written in rowPtr, which is on the device, and the kernel touches none of the three then
+    PSP_REQUIRE(rowPtr && A && B, "sddmm: null pointer");
+    PSP_REQUIRE((colIdx != nullptr) == (out != nullptr), "sddmm: colIdx and out must both be given (or both be null for a matrix without entries)");
     PSP_REQUIRE(!SPLIT || target_row, "sddmm: target_row is null");
-    PSP_REQUIRE(!BCSR || val, "sddmm: block values are null");
+    PSP_REQUIRE(!BCSR || val || !colIdx, "sddmm: block values are null");
     PSP_REQUIRE(!(BCSR && scale), "sddmm: scale is only supported for csr formats");
     PSP_REQUIRE(!(BCSR && row_max), "sddmm: row maxima are only supported for csr formats");
 
