@@ -87,3 +87,64 @@ def test_sddmm_structures(oracle, name, deg):
                     assert_close(got, want, rtol=1e-5, atol=2e-6, what="%s: %s g=%s K=%d bw=%d" % (name, fmt, g, K, bw))
         if colIdx.size == 0:
             break
+
+
+@pytest.mark.parametrize("name,deg", CASES, ids=[c[0] for c in CASES])
+def test_device_builders_structures(oracle, name, deg):
+    """row split and 2x1 blocks built on the device: bit for bit the oracle's arrays"""
+    from paramspmm_ae_amd import device_builder
+    from gpu_util import dev
+
+    rowPtr, colIdx, val = from_degrees(deg, len(deg) + 2)
+    for g in (1, 7, 32, 1000):
+        rs, tr = device_builder.split_csr_device(dev(rowPtr), g)
+        want_rs, want_tr = oracle.split_csr(rowPtr, g)
+        assert np.array_equal(rs.cpu().numpy(), want_rs) and np.array_equal(tr.cpu().numpy(), want_tr), (name, g)
+    got = device_builder.build_bcsr_device(dev(rowPtr), dev(colIdx), dev(val))
+    for a, b in zip(got, oracle.bcsr_build(rowPtr, colIdx, val)):
+        a = a.cpu().numpy()
+        assert np.array_equal(a, np.asarray(b).reshape(a.shape)), name
+
+
+@pytest.mark.parametrize("name,deg", CASES, ids=[c[0] for c in CASES])
+def test_fused_attention_structures(oracle, name, deg):
+    """scaled SDDMM with row maxima -> softmax-weighted SpMM on both CSR layouts against the oracle's three steps"""
+    from paramspmm_ae_amd import _capi
+    from gpu_util import Formats, assert_close, dev, stream
+
+    rowPtr, colIdx, val = from_degrees(deg, len(deg) + 3)
+    if colIdx.size == 0:
+        pytest.skip("no stored entries: nothing to weight")
+    n, K, N = rowPtr.size - 1, 16, 32
+    rng = np.random.default_rng(n)
+    A = (rng.standard_normal((n, K)) / 2).astype(np.float32)
+    H = rng.standard_normal((n, N)).astype(np.float32)
+    e_want = oracle.sddmm_csr(rowPtr, colIdx, A, A) * val
+    w_want = oracle.segment_softmax(rowPtr, e_want)
+    y_want = oracle.spmm_csr(rowPtr, colIdx, w_want, H)
+    scale = oracle.spmm_csr(rowPtr, colIdx, w_want, np.abs(H))
+    e_scale = oracle.sddmm_csr(rowPtr, colIdx, np.abs(A), np.abs(A)) * np.abs(val)
+    L, p = _capi.lib, _capi.ptr
+    Ad, Hd = dev(A), dev(H)
+    for g in (8, 64):
+        F = Formats(oracle, rowPtr, colIdx, val, g=g, gb=g)
+        d = F.d
+        for split in (False, True):
+            e = torch.full((F.nnz,), float("nan"), device="cuda")
+            m = torch.full((n,), float("nan"), device="cuda")
+            Y = torch.full((n, N), float("nan"), device="cuda")
+            if split:
+                row_sum = torch.full((n,), float("nan"), device="cuda")
+                _capi.check(L.psp_sddmm_csr_split_rowmax_f32(p(d["rps"]), p(d["colIdx"]), p(d["tr"]), p(Ad), p(Ad), p(d["val"]),
+                                                             p(e), p(m), F.tr.size, n, K, 4, stream()))
+                _capi.check(L.psp_spmm_csr_split_softmax_f32(p(d["rps"]), p(d["colIdx"]), p(e), p(d["tr"]), p(m), p(row_sum),
+                                                             p(Hd), p(Y), F.tr.size, N, n, 1, 4, stream()))
+            else:
+                _capi.check(L.psp_sddmm_csr_rowmax_f32(p(d["rowPtr"]), p(d["colIdx"]), p(Ad), p(Ad), p(d["val"]), p(e), p(m),
+                                                       n, K, 8, stream()))
+                _capi.check(L.psp_spmm_csr_softmax_f32(p(d["rowPtr"]), p(d["colIdx"]), p(e), p(m), p(Hd), p(Y), n, N, n, 1, 8,
+                                                       stream()))
+            torch.cuda.synchronize()
+            what = "%s g=%d split=%s" % (name, g, split)
+            assert_close(e, e_want, rtol=1e-5, atol=1e-6, what=what + " scores", scale=e_scale)
+            assert_close(Y, y_want, rtol=1e-4, atol=1e-5, what=what + " product", scale=scale)
