@@ -312,3 +312,32 @@ def test_host_vbsr_builder_matches_oracle(oracle, R):
         want = oracle.vbsr_build(rowPtr, colIdx, val, R, ncols=(n + R - 1) // R * R)
         for a, b in zip(got, want):
             assert a.dtype == b.dtype and np.array_equal(a, b)
+
+
+def test_sddmm_harness_checks_and_column_orders():
+    """compare / compare_2d (SDDMM.py:19-43) and the column orders of the two sweep tables"""
+    import torch
+    from paramspmm_ae_amd import SDDMM as S
+    from paramspmm_ae_amd import sweep
+    from paramspmm_ae_amd.PCSR import dynamic_CF_prompter
+
+    ref = torch.tensor([32.0, 32.0, 32.0])
+    S.compare(ref * (1 + 5e-5), ref, verbose=False)
+    with pytest.raises(ValueError, match="Verification FAILED"):
+        S.compare(ref * (1 + 2e-4), ref, verbose=False)
+    with pytest.raises(ValueError, match="is None"):
+        S.compare(None, ref)
+    blocked = torch.tensor([[32.0, 0.0], [32.0, 32.0]])  # slot 1 is padding
+    S.compare_2d(blocked, ref, torch.tensor([0, 2, 3], dtype=torch.int32), verbose=False)
+    assert S.column_names(3) == ["vec1_TP_4", "vec1_split_TP_4", "vec3_TP_4", "vec3_split_TP_4",
+                                 "vec1_TP_8", "vec1_split_TP_8", "vec3_TP_8", "vec3_split_TP_8"]
+    # SpMM sweep: blkWarpNum-major, then CF, then representation; an explicit CF list replaces the prompter's
+    assert sweep.column_names(80)[:5] == ["vec1_TP_%d4" % dynamic_CF_prompter(80)[0], "vec1_split_TP_%d4" % dynamic_CF_prompter(80)[0],
+                                          "vec2_TP_%d4" % dynamic_CF_prompter(80)[0], "vec2_split_TP_%d4" % dynamic_CF_prompter(80)[0],
+                                          "vec1_TP_%d4" % dynamic_CF_prompter(80)[1]]
+    assert sweep.column_names(80, cfs=[1, 2, 3], vec_size=3)[10:13] == ["vec3_TP_34", "vec3_split_TP_34", "vec1_TP_18"]
+    for dim in (16, 80, 256):
+        names = sweep.column_names(dim)
+        for col, name in enumerate(names):
+            if_split, vec_size, cf, bw = sweep.decode_column(dim, col)
+            assert name == "vec%d%s_TP_%d%d" % (vec_size, "_split" if if_split else "", cf, bw)
