@@ -175,6 +175,32 @@ __device__ __forceinline__ int find_col(const int *__restrict__ col, int lo, int
     return -1;
 }
 
+// first position in the ascending range col[lo, hi) whose column is not below c[k], for ILP columns at once: the
+// searches have the same depth (`top` = largest power of two not above hi - lo, at least 1), so their loads overlap
+template <int ILP>
+__device__ __forceinline__ void lower_bound_batch(const int *__restrict__ col, int lo, int hi, int top, const int (&c)[ILP],
+                                                  int (&pos)[ILP])
+{
+#pragma unroll
+    for (int k = 0; k < ILP; k++) pos[k] = lo;
+    if (hi <= lo) return;
+    for (int step = top; step >= 1; step >>= 1) {
+#pragma unroll
+        for (int k = 0; k < ILP; k++)
+            if (pos[k] + step <= hi && col[pos[k] + step - 1] < c[k]) pos[k] += step;
+    }
+}
+__device__ __forceinline__ int top_power_of_two(int len)
+{
+    int top = 1;
+    while (top * 2 <= len) top *= 2;
+    return top;
+}
+
+// Block-rows with more stored entries than this are built by a whole workgroup (bcsr_long_kernel): walked by a single
+// wavefront, the hub rows of a skewed graph were the tail of the launch (4.5 of 4.8 ms on an R-MAT graph).
+#define BCSR_LONG 2048
+
 // One wavefront per block-row t (rows 2t and 2t+1).  Blocks: the entries of row 2t in order, then the entries of
 // row 2t+1 whose column row 2t does not hold, in order -- the first-encounter order of the host builder.
 template <bool FILL>
@@ -190,6 +216,7 @@ __global__ void __launch_bounds__(256) bcsr_kernel(const int *__restrict__ rowPt
     const int a0 = rowPtr[2 * t], a1 = rowPtr[2 * t + 1];
     const int b1 = (2 * t + 1 < nrows) ? rowPtr[2 * t + 2] : a1;  // odd row count: the last block-row has one row
     const int len0 = a1 - a0;
+    if (a1 >= a0 && b1 >= a1 && b1 - a0 > BCSR_LONG) return;  // wave-uniform: bcsr_long_kernel takes this block-row
 
     if (!FILL) {
         // strictly ascending columns inside both rows?
@@ -234,6 +261,137 @@ __global__ void __launch_bounds__(256) bcsr_kernel(const int *__restrict__ rowPt
     if (!FILL && lane == 0) counts[t] = len0 + fresh;
 }
 
+// The long block-rows, one workgroup of 1024 lanes at a time.  Workgroup w looks at the block-rows w, w + G, w + 2G, ...
+// (hub rows often sit next to each other; this spreads them over the workgroups), 1024 of them per round: the lanes
+// list the long ones in LDS, then build each together.  Every lane looks up four entries at once, the ranks of the
+// entries that open their own block come from ballots, a prefix over the 16 wavefronts and the running total.
+template <bool FILL>
+__global__ void __launch_bounds__(1024) bcsr_long_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
+                                                         const float *__restrict__ val, int nrows, int nbr,
+                                                         int *__restrict__ counts, const int *__restrict__ rowPtr_b,
+                                                         int *__restrict__ colIdx_b, float *__restrict__ val_b,
+                                                         int *__restrict__ status)
+{
+    constexpr int ILP = 4, WAVES = 16;
+    __shared__ int s_list[1024];
+    __shared__ int s_nlist;
+    __shared__ int s_wave[ILP][WAVES];
+    const int tid = threadIdx.x, lane = tid & (PSP_WAVE - 1), wave = tid >> 6;
+    const long long G = gridDim.x;
+    for (long long i0 = 0; i0 * G < nbr; i0 += 1024) {
+        if (tid == 0) s_nlist = 0;
+        __syncthreads();
+        const long long tt = (i0 + tid) * G + blockIdx.x;
+        const int mine_t = (int)tt;
+        if (tt < nbr) {
+            const int a0 = rowPtr[2 * mine_t], a1 = rowPtr[2 * mine_t + 1];
+            const int b1 = (2 * mine_t + 1 < nrows) ? rowPtr[2 * mine_t + 2] : a1;
+            if (a1 >= a0 && b1 >= a1 && b1 - a0 > BCSR_LONG) s_list[atomicAdd(&s_nlist, 1)] = mine_t;
+        }
+        __syncthreads();
+        const int nlist = s_nlist;
+        for (int li = 0; li < nlist; li++) {
+            const int t = s_list[li];  // the order of the list does not matter: every block-row has its own output range
+            const int a0 = rowPtr[2 * t], a1 = rowPtr[2 * t + 1];
+            const int b1 = (2 * t + 1 < nrows) ? rowPtr[2 * t + 2] : a1;
+            const int len0 = a1 - a0;
+            if (!FILL) {
+                bool bad = false;  // strictly ascending columns inside both rows?
+                for (int p = a0 + tid; p < b1; p += 1024)
+                    if (p != a0 && p != a1 && colIdx[p] <= colIdx[p - 1]) bad = true;
+                if (bad) atomicOr(status, PSP_BUILD_UNSORTED);
+            } else {
+                const int base = rowPtr_b[t];
+                const int top1 = top_power_of_two(b1 - a1);
+                for (int i0e = 0; i0e < len0; i0e += ILP * 1024) {
+                    int c[ILP], q[ILP];
+#pragma unroll
+                    for (int k = 0; k < ILP; k++) {
+                        const int i = i0e + k * 1024 + tid;
+                        c[k] = i < len0 ? colIdx[a0 + i] : 0;
+                    }
+                    lower_bound_batch<ILP>(colIdx, a1, b1, top1, c, q);
+#pragma unroll
+                    for (int k = 0; k < ILP; k++) {
+                        const int i = i0e + k * 1024 + tid;
+                        if (i < len0) {
+                            const bool hit = q[k] < b1 && colIdx[q[k]] == c[k];
+                            colIdx_b[base + i] = c[k];
+                            val_b[2 * (size_t)(base + i)] = val[a0 + i];
+                            val_b[2 * (size_t)(base + i) + 1] = hit ? val[q[k]] : 0.0f;
+                        }
+                    }
+                }
+            }
+            // entries of row 2t+1 that open a block of their own, ranked in order
+            const int top = top_power_of_two(len0);
+            int fresh = 0;
+            for (int p0 = a1; p0 < b1; p0 += ILP * 1024) {
+                int c[ILP], lo[ILP];
+                bool in[ILP], mine[ILP];
+#pragma unroll
+                for (int k = 0; k < ILP; k++) {
+                    const int p = p0 + k * 1024 + tid;
+                    in[k] = p < b1;
+                    c[k] = in[k] ? colIdx[p] : 0;
+                }
+                lower_bound_batch<ILP>(colIdx, a0, a1, top, c, lo);
+#pragma unroll
+                for (int k = 0; k < ILP; k++) {
+                    mine[k] = in[k] && !(lo[k] < a1 && colIdx[lo[k]] == c[k]);
+                    const unsigned long long m = __ballot(mine[k]);
+                    if (lane == 0) s_wave[k][wave] = __popcll(m);
+                    lo[k] = __popcll(m & ((1ull << lane) - 1ull));  // rank inside the wavefront
+                }
+                __syncthreads();
+                int before = fresh;  // blocks opened by earlier chunks, earlier wavefronts of this chunk
+#pragma unroll
+                for (int k = 0; k < ILP; k++) {
+                    int chunk_total = 0, ahead = 0;
+#pragma unroll
+                    for (int w = 0; w < WAVES; w++) {
+                        const int n_w = s_wave[k][w];
+                        if (w < wave) ahead += n_w;
+                        chunk_total += n_w;
+                    }
+                    if (FILL && mine[k]) {
+                        const int slot = rowPtr_b[t] + len0 + before + ahead + lo[k];
+                        const int p = p0 + k * 1024 + tid;
+                        colIdx_b[slot] = c[k];
+                        val_b[2 * (size_t)slot] = 0.0f;
+                        val_b[2 * (size_t)slot + 1] = val[p];
+                    }
+                    before += chunk_total;
+                }
+                fresh = before;
+                __syncthreads();  // s_wave is rewritten by the next round
+            }
+            if (!FILL && tid == 0) counts[t] = len0 + fresh;
+        }
+        __syncthreads();  // s_list / s_nlist are rewritten by the next slab
+    }
+}
+
+static void launch_bcsr(bool fill, const int *rowPtr, const int *colIdx, const float *val, int nrows, int nbr, int *counts,
+                        const int *rowPtr_b, int *colIdx_b, float *val_b, int *status, hipStream_t st)
+{
+    // about two workgroups of 1024 lanes per CU; a prime (odd) count, because the workgroups take block-rows by index
+    // modulo the count and hub rows of generated graphs share their low index bits
+    int long_wgs = psp_ceil_div(nbr, 64);
+    long_wgs = long_wgs >= 509 ? 509 : (long_wgs | 1);
+    if (fill) {
+        hipLaunchKernelGGL(bcsr_kernel<true>, dim3(psp_ceil_div(nbr, 4)), dim3(256), 0, st, rowPtr, colIdx, val, nrows, nbr,
+                           counts, rowPtr_b, colIdx_b, val_b, status);
+        hipLaunchKernelGGL(bcsr_long_kernel<true>, dim3(long_wgs), dim3(1024), 0, st, rowPtr, colIdx, val, nrows, nbr, counts,
+                           rowPtr_b, colIdx_b, val_b, status);
+    } else {
+        hipLaunchKernelGGL(bcsr_kernel<false>, dim3(psp_ceil_div(nbr, 4)), dim3(256), 0, st, rowPtr, colIdx, val, nrows, nbr,
+                           counts, rowPtr_b, colIdx_b, val_b, status);
+        hipLaunchKernelGGL(bcsr_long_kernel<false>, dim3(long_wgs), dim3(1024), 0, st, rowPtr, colIdx, val, nrows, nbr, counts,
+                           rowPtr_b, colIdx_b, val_b, status);
+    }
+}
+
 PSP_EXPORT int psp_bcsr_offsets_dev(const int *rowPtr, const int *colIdx, int nrows, int *rowPtr_b, int *workspace,
                                     int workspace_ints, int *status, psp_stream_t stream)
 {
@@ -241,9 +399,7 @@ PSP_EXPORT int psp_bcsr_offsets_dev(const int *rowPtr, const int *colIdx, int nr
     const int nbr = (nrows + 1) / 2;
     hipStream_t st = (hipStream_t)stream;
     if (nbr > 0) {  // colIdx may be null for a matrix without entries (the host cannot tell, rowPtr is on the device)
-        hipLaunchKernelGGL(bcsr_kernel<false>, dim3(psp_ceil_div(nbr, 4)), dim3(256), 0, st, rowPtr, colIdx,
-                           (const float *)nullptr, nrows, nbr, rowPtr_b, (const int *)nullptr, (int *)nullptr,
-                           (float *)nullptr, status);
+        launch_bcsr(false, rowPtr, colIdx, nullptr, nrows, nbr, rowPtr_b, nullptr, nullptr, nullptr, status, st);
     }
     return exclusive_scan(rowPtr_b, rowPtr_b, nbr, workspace, workspace_ints, status, st);
 }
@@ -254,8 +410,7 @@ PSP_EXPORT int psp_bcsr_fill_dev(const int *rowPtr, const int *colIdx, const flo
     PSP_REQUIRE(rowPtr && rowPtr_b && nrows >= 0, "bcsr_fill_dev: bad input");
     const int nbr = (nrows + 1) / 2;
     if (nbr == 0) return PSP_OK;  // the entry arrays may be null when rowPtr_b says there are no blocks
-    hipLaunchKernelGGL(bcsr_kernel<true>, dim3(psp_ceil_div(nbr, 4)), dim3(256), 0, (hipStream_t)stream, rowPtr, colIdx, val,
-                       nrows, nbr, (int *)nullptr, rowPtr_b, colIdx_b, val_b, (int *)nullptr);
+    launch_bcsr(true, rowPtr, colIdx, val, nrows, nbr, nullptr, rowPtr_b, colIdx_b, val_b, nullptr, (hipStream_t)stream);
     return psp_check_launch("bcsr fill kernel");
 }
 

@@ -33,6 +33,7 @@ CASES = [
     dict(n=3000, avg_deg=9.0, seed=3, hub=(17, 2500)),         # a row far longer than a wavefront
     dict(n=3001, avg_deg=4.0, seed=4, empty_frac=0.1, hub=(3000, 700)),  # odd row count, hub in the unpaired row
     dict(n=5000, avg_deg=0.2, seed=5, empty_frac=0.5),          # mostly empty
+    dict(n=20000, avg_deg=3.0, seed=6, hub=(1001, 9000)),       # a block-row built by a whole workgroup, several rounds
 ]
 
 

@@ -39,6 +39,9 @@ def structures():
     yield "alternating 0 / 130", [0 if i % 2 else 130 for i in range(400)]
     yield "lengths around 32", [31, 32, 33] * 150
     yield "geometric", [min(1 << (i % 11), 1000) for i in range(1100)]
+    # block-rows long enough for the device builder's workgroup path: both rows long, only the odd one, only the even one
+    long_rows = {10: 5000, 11: 4000, 4000: 3, 4001: 3000, 2000: 2500, 2001: 0, 5999: 2100}
+    yield "long block-rows", [long_rows.get(i, int(d)) for i, d in enumerate(rng.poisson(1.5, 6000))]
 
 
 CASES = list(structures())
