@@ -13,7 +13,7 @@ SuiteSparse / OGB collection the reference downloads.
                 the reference's two statistics (accuracy, mean normalised performance) plus the share of
                 matrices whose pick is within 10 % of the best swept configuration.
 
-    python -m paramspmm_ae_amd.train_decider sweep --out gpurun_out/decider [--part 0/3]
+    python -m paramspmm_ae_amd.train_decider sweep --out ParamSpMM-log/decider [--part 0/3]
     python -m paramspmm_ae_amd.train_decider fit --data paramspmm_ae_amd/models/train_data --out paramspmm_ae_amd/models
 """
 import argparse
@@ -297,7 +297,7 @@ def main(argv=None):
     ap = argparse.ArgumentParser()
     sub = ap.add_subparsers(dest="cmd", required=True)
     s = sub.add_parser("sweep")
-    s.add_argument("--out", default="gpurun_out/decider")
+    s.add_argument("--out", default="ParamSpMM-log/decider")
     s.add_argument("--part", default="0/1", help="i/n: every n-th matrix starting at i")
     s.add_argument("--limit", type=int, default=0)
     s.add_argument("--warmup", type=int, default=2)
