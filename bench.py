@@ -252,7 +252,21 @@ def bench_sddmm(args):
             reps += 1
         cpu_torch = {"value": round(2.0 * take * K * reps / (_t.perf_counter() - t0) / 1e9, 2), "unit": "GFLOP/s",
                      "cores": torch.get_num_threads()}
-    print(json.dumps({"cpu_baseline": cpu, "cpu_torch_gathered": cpu_torch if cpu else None, "metric": "SDDMM GFLOP/s (2*nnz*K) over K = 16..128", "value": round(value, 1), "unit": "GFLOP/s",
+    # roofline of the width that takes the most time; HBM traffic from the committed counter summary when it has the
+    # same configuration (| K | layout | wavefronts | ... | HBM bytes | in column 11)
+    dom = max(per_K, key=lambda r: r["ms"])
+    traffic = None
+    prof = os.path.join(ROOT, "profiles", "psp_sddmm_kernel_%s_trace_and_pmc.md" % args.graph)
+    if os.path.exists(prof):
+        for line in open(prof):
+            cells = [c.strip() for c in line.strip().strip("|").split("|")]
+            if len(cells) >= 11 and cells[0].isdigit() and (int(cells[0]), cells[1], int(cells[2])) == (dom["K"], dom["format"], dom["blkWarpNum"]):
+                traffic = int(cells[10])
+    roofline = {"bound": "hbm", "achieved": dom["alg_GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": dom["frac_hbm"],
+                "traffic": traffic, "kernel": "psp_sddmm_kernel, K = %d, %s, %d wavefronts per workgroup" % (dom["K"], dom["format"], dom["blkWarpNum"]),
+                "alg_bytes_per_launch": dom["alg_bytes"], "ms_per_launch": dom["ms"]}
+    print(json.dumps({"cpu_baseline": cpu, "cpu_torch_gathered": cpu_torch if cpu else None, "roofline": roofline,
+                      "metric": "SDDMM GFLOP/s (2*nnz*K) over K = 16..128", "value": round(value, 1), "unit": "GFLOP/s",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(total_ms, 4),
                       "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
                       "config": {"workload": "%s SDDMM width sweep" % args.graph, "nodes": n, "nnz": nnz}, "per_K": per_K}))
