@@ -238,6 +238,18 @@ int psp_segment_softmax_f32(const int *rowPtr, const float *in, float *out, int 
 int psp_segment_softmax_ws_f32(const int *rowPtr, const float *in, float *out, int M, int nnz, float *workspace,
                                psp_stream_t stream);
 
+/* The same softmax for callers that cannot allocate device memory.  It has no counterpart in the reference: it is
+ * for code under HIP graph capture, tight serving loops and harnesses that forbid hipMalloc.  Same result as
+ * psp_segment_softmax_ws_f32, whose kernels it runs, but the 2*M floats of workspace are a fixed array inside the
+ * library (16 MiB of device memory on every GPU the library is used on, held until the process ends); the call
+ * allocates and frees nothing.  M may not exceed PSP_SEGMENT_SOFTMAX_STATIC_MAX_ROWS (PSP_ERR_ARG beyond it: use the
+ * _ws_ form).  The stream's device must be the current device.  All calls on one GPU share the array: two calls
+ * that overlap on one GPU (different streams, or graphs replayed concurrently) race on it; calls on one stream, or
+ * otherwise ordered, do not. */
+#define PSP_SEGMENT_SOFTMAX_STATIC_MAX_ROWS (1 << 21)
+int psp_segment_softmax_static_f32(const int *rowPtr, const float *in, float *out, int M, int nnz,
+                                   psp_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: C[K1,K2] = A^T * B for tall-skinny row-major A [n,K1] and B [n,K2]; C is overwritten.
  * Stands in for the weight-gradient product torch::mm(H.t(), AG) of the fused GCN backward

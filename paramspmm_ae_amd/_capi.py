@@ -72,6 +72,7 @@ SIGNATURES = {
     "psp_sddmm_vec_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "psp_segment_softmax_f32": [_vp, _vp, _vp, _i, _vp],
     "psp_segment_softmax_ws_f32": [_vp, _vp, _vp, _i, _i, _vp, _vp],
+    "psp_segment_softmax_static_f32": [_vp, _vp, _vp, _i, _i, _vp],
     "psp_spmm_f64": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "psp_sddmm_f64": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "psp_baseline_rowcache_spmm_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp],

@@ -1,6 +1,7 @@
 // extern "C" surface of libparamsp_hip.so (declared in include/paramsp.h), the small utility kernels
 // (zero fill, genmask, segment softmax) and the host-side PCSR index construction.
 #include <algorithm>
+#include <mutex>
 #include <thread>
 #include <vector>
 #include <string.h>
@@ -399,6 +400,54 @@ PSP_EXPORT int psp_segment_softmax_ws_f32(const int *rowPtr, const float *in, fl
     hipLaunchKernelGGL(psp_softmax_long_kernel<1>, grid, dim3(256), 0, st, rowPtr, in, out, M, nnz, workspace);
     hipLaunchKernelGGL(psp_softmax_long_kernel<2>, grid, dim3(256), 0, st, rowPtr, in, out, M, nnz, workspace);
     return psp_check_launch("segment softmax kernels");
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same softmax for callers that cannot allocate (code under HIP graph capture, serving loops, harnesses that
+// forbid hipMalloc): the (max, sum) pairs of the long rows live in a fixed array inside the library's device image
+// instead of a caller's workspace.  Every GPU holds its own copy of the array at its own address, so the address
+// is looked up once per device (hipGetSymbolAddress, no allocation) and the kernels receive it as an argument like
+// any workspace.  In host code the array's name is only a handle for that lookup, never a device address.
+// ------------------------------------------------------------------------------------------------
+#define PSP_STATIC_SOFTMAX_MAX_ROWS PSP_SEGMENT_SOFTMAX_STATIC_MAX_ROWS  // include/paramsp.h
+#define PSP_MAX_DEVICES 64
+static __device__ __align__(256) float psp_softmax_scratch[2 * PSP_STATIC_SOFTMAX_MAX_ROWS];  // 16 MiB per GPU
+static float *g_softmax_scratch[PSP_MAX_DEVICES];  // device address of the array on each GPU, null = not looked up
+static std::mutex g_softmax_scratch_lock;
+
+static int psp_softmax_scratch_ptr(float **out)
+{
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return psp_fail(PSP_ERR_LAUNCH, "segment_softmax_static: hipGetDevice: %s", hipGetErrorString(e));
+    PSP_REQUIRE(dev >= 0 && dev < PSP_MAX_DEVICES, "segment_softmax_static: device %d outside 0..%d", dev, PSP_MAX_DEVICES - 1);
+    std::lock_guard<std::mutex> hold(g_softmax_scratch_lock);
+    if (!g_softmax_scratch[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(psp_softmax_scratch));
+        if (e != hipSuccess || !p)
+            return psp_fail(PSP_ERR_LAUNCH, "segment_softmax_static: hipGetSymbolAddress on device %d: %s", dev, hipGetErrorString(e));
+        g_softmax_scratch[dev] = (float *)p;
+    }
+    *out = g_softmax_scratch[dev];
+    return PSP_OK;
+}
+
+PSP_EXPORT int psp_segment_softmax_static_f32(const int *rowPtr, const float *in, float *out, int M, int nnz,
+                                              psp_stream_t stream)
+{
+    PSP_REQUIRE(M >= 0 && nnz >= 0, "segment_softmax_static: negative size");
+    PSP_REQUIRE(M <= PSP_STATIC_SOFTMAX_MAX_ROWS,
+                "segment_softmax_static: %d rows exceed the built-in scratch of %d rows; use psp_segment_softmax_ws_f32", M,
+                PSP_STATIC_SOFTMAX_MAX_ROWS);
+    if (M == 0 || nnz == 0) return PSP_OK;
+    PSP_REQUIRE(rowPtr && in && out, "segment_softmax_static: null pointer");
+    float *scratch = nullptr;
+    const int rc = psp_softmax_scratch_ptr(&scratch);
+    if (rc != PSP_OK) return rc;
+    // Nothing has to start at zero: the first kernel resets the pair of every long row of this call, and pairs of
+    // other rows (left by earlier calls) are never read.
+    return psp_segment_softmax_ws_f32(rowPtr, in, out, M, nnz, scratch, stream);
 }
 
 PSP_EXPORT int psp_sddmm_vec_f32(const int *rowPtr_b, const int *colIdx_b, const float *val_b, const float *A,
