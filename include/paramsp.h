@@ -34,8 +34,22 @@ const char *psp_last_error(void);
 int psp_version(void);
 
 /* How a (N, CF, blkWarpNum) request of the Python layer maps onto the wave64 kernels.
- * CF keeps its meaning "column coarsening": the number of `vec`-wide column vectors one lane owns;
- * blkWarpNum keeps its meaning "wavefronts per workgroup" (4 or 8, SpMM/SpMM.cpp:77-141). */
+ * CF 1..8 keeps its meaning "column coarsening": the number of `vec`-wide column vectors one lane owns;
+ * blkWarpNum keeps its meaning "wavefronts per workgroup" (4 or 8, SpMM/SpMM.cpp:77-141).  The reference's callers
+ * pass CF through as an opaque int (PCSR.py:224-237), so the same argument also carries the NATIVE parameter space of
+ * the wave64 kernel, which the reference's <CF, blkWarpNum> cannot express: a value with PSP_CF_NATIVE set names
+ *   coarsen     1..8   column vectors per lane,
+ *   log_lanes   0..6   lanes that share one sparse row = 2^log_lanes (rows per wavefront = 64 / lanes),
+ *   log_unroll  0..3   stored entries whose feature loads are in flight together per lane = 2^log_unroll
+ *                      (coarsen * unroll <= 8, unroll <= lanes),
+ *   segs_sel    0..7   0 = segments per wavefront chosen by the library, s >= 1 = 2^(s-1) segments per wavefront
+ * (build one with PSP_CF_PACK).  The sweep times such configurations and the decider's forests are trained on them
+ * (decider.py:63-80 decodes CF from a list, so the list may hold packed values). */
+#define PSP_CF_NATIVE (1 << 16)
+#define PSP_CF_EVEN_SPLIT (1 << 11) /* with PSP_CF_NATIVE: always divide a wavefront's entries evenly between the
+                                      lane groups, never hand them whole segments (see the option "align_pct") */
+#define PSP_CF_PACK(coarsen, log_lanes, log_unroll, segs_sel) \
+    (PSP_CF_NATIVE | ((coarsen) - 1) | ((log_lanes) << 3) | ((log_unroll) << 6) | ((segs_sel) << 8))
 typedef struct psp_spmm_plan {
     int vec;            /* floats per feature load: 4 (N%4==0), 2 (N%2==0) or 1 */
     int coarsen;        /* column vectors per lane (the request's CF, 1..8) */
@@ -44,8 +58,21 @@ typedef struct psp_spmm_plan {
     int unroll;         /* non-zeros whose feature loads are in flight together per lane */
     int col_tiles;      /* grid.y: ceil(N / (lanes_per_row*coarsen*vec)) */
     int waves_per_block;
+    int log_segs_per_wave; /* -1: chosen at launch from the format and the matrix size */
+    int even_split;        /* 1: the wavefront's entries are always divided evenly between the lane groups */
 } psp_spmm_plan;
 int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan);
+
+/* Library-wide tuning options (no counterpart in the reference, whose launch shapes are compile-time constants):
+ *   "xcd_stripe_rows"  rows (segments) dealt to one XCD at a time by the SpMM kernels (default 8192),
+ *   "align_pct"        lane groups take whole segments when that costs at most this many percent more steps than
+ *                      the even division of a wavefront's entries (default 50),
+ *   "split_clear_min"  row-split outputs of at least this many floats are cleared selectively (default 32 Mi).
+ * The environment (PSP_XCD_STRIPE_ROWS, PSP_ALIGN_PCT, PSP_SPLIT_CLEAR_MIN) sets the initial values, once.
+ * psp_get_option returns the value, or a negative psp_status for an unknown name.  Not synchronised with running
+ * launches: set options before the calls they should affect. */
+int psp_set_option(const char *name, long long value);
+long long psp_get_option(const char *name);
 
 /* ---------------------------------------------------------------------------------------------
  * HOST: PCSR index construction

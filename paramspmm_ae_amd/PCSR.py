@@ -40,6 +40,43 @@ def dynamic_CF_prompter(dim, CF_set=None, warp_size=32, verbose=False):
     return keep
 
 
+def native_CF_prompter(dim):
+    """Configurations of the wave64 kernel that the reference's <CF, blkWarpNum> cannot express, as packed values
+    for the ``CF`` argument (``_capi.pack_cf``; the operators pass CF through as an opaque int, PCSR.py:224-237):
+    lane groups of 16 and 32 lanes (4 and 2 sparse rows per wavefront, fewer column tiles) and the even division
+    of a wavefront's entries between its lane groups.  The list depends only on the 32-wide band of ``dim``, like
+    the forest that serves a width (decider.py:52-55), so both stay in step."""
+    from ._capi import pack_cf
+
+    band = math.ceil(dim / 32)
+    if band <= 1:
+        return [pack_cf(1, 8 if dim > 16 else 4, 4, even_split=True)]
+    cf_max = dynamic_CF_prompter(band * 32)[-1]
+    extra = [pack_cf(1, 16, 4), pack_cf(1, 8, 4, even_split=True),
+             pack_cf(cf_max, 8, 2 if cf_max <= 4 else 1, even_split=True)]
+    if band >= 4:
+        extra.append(pack_cf(1, 32, 4))
+    return extra
+
+
+def decider_CF_list(dim):
+    """The CF axis of the decider's class space: the reference's list (PCSR.py:30-42) followed by the native
+    configurations.  Class count per width = 4 representations x len(list) x 2 workgroup sizes."""
+    return dynamic_CF_prompter(dim) + native_CF_prompter(dim)
+
+
+def cf_label(cf):
+    """Text of a CF value in a sweep column name: the number itself for the reference's CF, c<vectors per lane>l<lanes
+    per row>u<entries in flight>[e] for a native configuration."""
+    from ._capi import unpack_cf
+
+    u = unpack_cf(int(cf))
+    if u is None:
+        return str(int(cf))
+    c, lanes, unroll, segs, even = u
+    return "c%dl%du%d%s%s" % (c, lanes, unroll, "" if segs is None else "w%d" % segs, "e" if even else "")
+
+
 class _VendorFormatSpMM(object):
     """Vendor-library SpMM on a re-formatted copy of the graph's CSR matrix (PCSR.py:45-124)."""
 

@@ -30,6 +30,8 @@ class SpmmPlan(ctypes.Structure):
         ("unroll", _i),
         ("col_tiles", _i),
         ("waves_per_block", _i),
+        ("log_segs_per_wave", _i),
+        ("even_split", _i),
     ]
 
     def as_dict(self):
@@ -39,6 +41,8 @@ class SpmmPlan(ctypes.Structure):
 # name -> argtypes; the entries return int unless RESTYPES says otherwise.  Keep in step with include/paramsp.h.
 SIGNATURES = {
     "psp_version": [],
+    "psp_set_option": [ctypes.c_char_p, ctypes.c_longlong],
+    "psp_get_option": [ctypes.c_char_p],
     "psp_spmm_plan_for": [_i, _i, _i, ctypes.POINTER(SpmmPlan)],
     "psp_split_csr_count": [_vp, _i, _i],
     "psp_split_csr": [_vp, _i, _i, _vp, _vp],
@@ -86,7 +90,7 @@ SIGNATURES = {
     "psp_gemm_atb_ws_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _vp, ctypes.c_longlong, _vp],
 }
 # the entries that do not return int
-RESTYPES = {"psp_gemm_atb_workspace_floats": ctypes.c_longlong}
+RESTYPES = {"psp_gemm_atb_workspace_floats": ctypes.c_longlong, "psp_get_option": ctypes.c_longlong}
 
 for _name, _args in SIGNATURES.items():
     _fn = getattr(lib, _name)
@@ -105,6 +109,43 @@ def check(rc):
     if rc < 0:
         raise ParamSpError("libparamsp_hip: %s (status %d)" % (lib.psp_last_error().decode(), rc))
     return rc
+
+
+CF_NATIVE = 1 << 16  # PSP_CF_NATIVE of include/paramsp.h
+
+
+def pack_cf(coarsen, lanes, unroll=None, segs_per_wave=None, even_split=False):
+    """Native SpMM configuration for the CF argument (PSP_CF_PACK): ``coarsen`` column vectors per lane, ``lanes``
+    lanes per sparse row, ``unroll`` entries in flight (default: the largest with coarsen*unroll <= 4 ... 8 that the
+    kernels are built for), ``segs_per_wave`` segments per wavefront (None = chosen by the library)."""
+    if unroll is None:
+        unroll = 4 if coarsen == 1 else 2 if coarsen <= 4 else 1
+        unroll = min(unroll, lanes)
+    log_l, log_u = lanes.bit_length() - 1, unroll.bit_length() - 1
+    if 1 << log_l != lanes or 1 << log_u != unroll or not 1 <= coarsen <= 8 or lanes > 64 or unroll > 8:
+        raise ValueError("pack_cf: coarsen 1..8, lanes and unroll powers of two (lanes <= 64, unroll <= 8)")
+    sel = 0
+    if segs_per_wave is not None:
+        sel = segs_per_wave.bit_length()
+        if 1 << (sel - 1) != segs_per_wave or sel > 7:
+            raise ValueError("pack_cf: segs_per_wave must be a power of two up to 64")
+    return CF_NATIVE | (coarsen - 1) | (log_l << 3) | (log_u << 6) | (sel << 8) | (int(bool(even_split)) << 11)
+
+
+def unpack_cf(CF):
+    """(coarsen, lanes, unroll, segs_per_wave or None, even_split) of a native CF value; None for a legacy CF."""
+    if not CF & CF_NATIVE:
+        return None
+    sel = (CF >> 8) & 7
+    return (CF & 7) + 1, 1 << ((CF >> 3) & 7), 1 << ((CF >> 6) & 3), (1 << (sel - 1)) if sel else None, bool(CF & (1 << 11))
+
+
+def set_option(name, value):
+    check(lib.psp_set_option(name.encode(), int(value)))
+
+
+def get_option(name):
+    return check(lib.psp_get_option(name.encode()))
 
 
 def spmm_plan(N, CF, blkWarpNum):

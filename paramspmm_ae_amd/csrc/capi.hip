@@ -24,48 +24,106 @@ int psp_fail(int code, const char *fmt, ...)
     return code;
 }
 
-int psp_stripe_rows(void)
+// Library-wide options: defaults, overridden once by the environment (PSP_XCD_STRIPE_ROWS, PSP_ALIGN_PCT,
+// PSP_SPLIT_CLEAR_MIN) when the library is first used, and afterwards only through psp_set_option.
+psp_options &psp_opts(void)
 {
-    static int rows = [] {
-        const char *e = getenv("PSP_XCD_STRIPE_ROWS");
-        const int v = e ? atoi(e) : 0;
-        return v > 0 ? v : 8192;
+    static psp_options o = [] {
+        psp_options d;
+        d.stripe_rows = 8192;
+        d.align_pct = 50;
+        d.split_clear_min = (long long)32 << 20;
+        if (const char *e = getenv("PSP_XCD_STRIPE_ROWS")) {
+            if (atoi(e) > 0) d.stripe_rows = atoi(e);
+        }
+        if (const char *e = getenv("PSP_ALIGN_PCT")) {
+            if (atoi(e) >= 0) d.align_pct = atoi(e);
+        }
+        if (const char *e = getenv("PSP_SPLIT_CLEAR_MIN")) {
+            if (atoll(e) >= 0) d.split_clear_min = atoll(e);
+        }
+        return d;
     }();
-    return rows;
+    return o;
+}
+int psp_stripe_rows(void) { return psp_opts().stripe_rows; }
+
+PSP_EXPORT int psp_set_option(const char *name, long long value)
+{
+    PSP_REQUIRE(name != nullptr, "set_option: name is null");
+    psp_options &o = psp_opts();
+    if (!strcmp(name, "xcd_stripe_rows")) {
+        PSP_REQUIRE(value >= 1 && value <= (1 << 30), "set_option: xcd_stripe_rows must be positive");
+        o.stripe_rows = (int)value;
+    } else if (!strcmp(name, "align_pct")) {
+        PSP_REQUIRE(value >= 0 && value <= 100000, "set_option: align_pct must be 0..100000");
+        o.align_pct = (int)value;
+    } else if (!strcmp(name, "split_clear_min")) {
+        PSP_REQUIRE(value >= 0, "set_option: split_clear_min must not be negative");
+        o.split_clear_min = value;
+    } else {
+        return psp_fail(PSP_ERR_ARG, "set_option: unknown option '%s'", name);
+    }
+    return PSP_OK;
+}
+
+PSP_EXPORT long long psp_get_option(const char *name)
+{
+    if (!name) return psp_fail(PSP_ERR_ARG, "get_option: name is null");
+    const psp_options &o = psp_opts();
+    if (!strcmp(name, "xcd_stripe_rows")) return o.stripe_rows;
+    if (!strcmp(name, "align_pct")) return o.align_pct;
+    if (!strcmp(name, "split_clear_min")) return o.split_clear_min;
+    return psp_fail(PSP_ERR_ARG, "get_option: unknown option '%s'", name);
 }
 
 PSP_EXPORT const char *psp_last_error(void) { return g_err; }
-PSP_EXPORT int psp_version(void) { return 100; }
+PSP_EXPORT int psp_version(void) { return 200; }
 
 // ------------------------------------------------------------------------------------------------
 // (N, CF, blkWarpNum) -> wave64 launch plan
 // ------------------------------------------------------------------------------------------------
+static bool psp_cu_pair_exists(int C, int U)
+{
+#define PSP_HAS(C_, U_) \
+    if (C == C_ && U == U_) return true;
+    PSP_SPMM_FOR_EACH_CU(PSP_HAS)
+#undef PSP_HAS
+    return false;
+}
+
 PSP_EXPORT int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan)
 {
     PSP_REQUIRE(plan != nullptr, "plan is null");
     PSP_REQUIRE(N >= 1, "feature dimension must be positive (got %d)", N);
-    PSP_REQUIRE(CF >= 1 && CF <= 8, "CF must be 1..8 (got %d)", CF);
     PSP_REQUIRE(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8 (got %d)", blkWarpNum);
-    // A lane group owns a tile of 32*CF columns, as the reference's warp does (CF columns per lane of a 32-lane
-    // warp, SpMM_kernel.cu:162-165); the remaining columns go to further column tiles (grid.y).  Natively the
-    // 32-column slab is 8 lanes x float4 (16 x float2 / 32 x float when N is not a multiple of 4) and CF is the
-    // number of such vectors per lane, so a wavefront carries 8 rows whatever CF is.
     const int V = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
     const int nvec = N / V;
-    int C = std::min(CF, nvec);
-    int L = 32 / V;
-    while (L > 1 && (L / 2) * C >= nvec) L >>= 1;  // one tile already covers N: no wider than needed
-    if (const char *e = getenv("PSP_FORCE_LANES")) {  // tuning aid
-        const int f = atoi(e);
-        if (f >= 1 && f <= 64 && (f & (f - 1)) == 0) L = f;
+    int C, L, U, logW = -1;
+    if (CF & PSP_CF_NATIVE) {
+        // native configuration: every field of the wave64 mapping chosen by the caller (the sweep / the decider)
+        PSP_REQUIRE((CF & ~(PSP_CF_NATIVE | 0xfff)) == 0, "CF 0x%x: unknown bits in a native configuration", CF);
+        C = (CF & 7) + 1;
+        const int logL = (CF >> 3) & 7, logU = (CF >> 6) & 3, wsel = (CF >> 8) & 7;
+        PSP_REQUIRE(logL <= 6, "native configuration: 2^%d lanes per row exceed the wavefront", logL);
+        L = 1 << logL;
+        U = 1 << logU;
+        PSP_REQUIRE(U <= L, "native configuration: %d entries in flight need at least as many lanes per row (got %d)", U, L);
+        C = std::min(C, nvec);
+        PSP_REQUIRE(psp_cu_pair_exists(C, U), "native configuration: no kernel for %d vectors per lane with %d entries in flight", C, U);
+        if (wsel) logW = wsel - 1;
+    } else {
+        PSP_REQUIRE(CF >= 1 && CF <= 8, "CF must be 1..8 (got %d)", CF);
+        // A lane group owns a tile of 32*CF columns, as the reference's warp does (CF columns per lane of a 32-lane
+        // warp, SpMM_kernel.cu:162-165); the remaining columns go to further column tiles (grid.y).  Natively the
+        // 32-column slab is 8 lanes x float4 (16 x float2 / 32 x float when N is not a multiple of 4) and CF is the
+        // number of such vectors per lane, so a wavefront carries 8 rows whatever CF is.
+        C = std::min(CF, nvec);
+        L = 32 / V;
+        while (L > 1 && (L / 2) * C >= nvec) L >>= 1;  // one tile already covers N: no wider than needed
+        U = C == 1 ? 4 : C <= 4 ? 2 : 1;  // feature vectors in flight per lane: U entries x C vectors
+        while (U > L) U >>= 1;
     }
-    // feature vectors in flight per lane: U entries x C vectors
-    int U = C == 1 ? 4 : C <= 4 ? 2 : 1;
-    if (const char *e = getenv("PSP_FORCE_UNROLL")) {  // tuning aid
-        const int f = atoi(e);
-        if (f == 1 || f == 2 || f == 4 || f == 8) U = (C * f <= 8) ? f : U;
-    }
-    while (U > L) U >>= 1;
     plan->vec = V;
     plan->coarsen = C;
     plan->lanes_per_row = L;
@@ -73,6 +131,8 @@ PSP_EXPORT int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *p
     plan->unroll = U;
     plan->col_tiles = psp_ceil_div(nvec, L * C);
     plan->waves_per_block = blkWarpNum;
+    plan->log_segs_per_wave = logW;
+    plan->even_split = (CF & PSP_CF_NATIVE) && (CF & PSP_CF_EVEN_SPLIT) ? 1 : 0;
     return PSP_OK;
 }
 
@@ -137,35 +197,69 @@ int psp_row_scale(float *Y, const float *s, int rows, int N, hipStream_t stream)
 }
 
 // ------------------------------------------------------------------------------------------------
-// selective clear for row-split SpMM: one lane per segment (plus one for the rows past the last segment)
+// selective clear for row-split SpMM.  A workgroup owns 256 consecutive target rows: it finds the segments that
+// target them (target_row is sorted: two binary searches), marks in LDS which rows a segment targets and which of
+// those the SpMM kernel will add to rather than store (a row continuing across two wavefronts, a row with an empty
+// segment), and then clears the rows that need it -- rows nothing targets included -- one wavefront per row with
+// 16-byte stores.  Runs of untargeted rows of any length are thus spread over the whole grid.
 // ------------------------------------------------------------------------------------------------
-__device__ __forceinline__ void psp_clear_rows(float *Y, long long r0, long long r1, int N)
-{
-    for (long long i = r0 * N; i < r1 * N; i++) Y[i] = 0.0f;
-}
+#define PSP_CLEAR_ROWS 256
 
 __global__ void __launch_bounds__(256)
 psp_split_clear_kernel(const int *__restrict__ rowPtr_split, const int *__restrict__ target_row, float *__restrict__ Y,
                        int nseg, int N, int nr, int rows_out, int logW)
 {
-    const int s = blockIdx.x * blockDim.x + threadIdx.x;
-    if (s > nseg) return;
-    if (s == nseg) {  // rows after the last targeted row
-        psp_clear_rows(Y, (long long)(target_row[nseg - 1] + 1) * nr, rows_out, N);
-        return;
+    __shared__ int s_targeted[PSP_CLEAR_ROWS], s_added[PSP_CLEAR_ROWS], s_list[PSP_CLEAR_ROWS];
+    __shared__ int s_range[2], s_count;
+    const int ntargets = (rows_out + nr - 1) / nr;
+    const int t0 = blockIdx.x * PSP_CLEAR_ROWS, t1 = min(ntargets, t0 + PSP_CLEAR_ROWS);
+    s_targeted[threadIdx.x] = 0;
+    s_added[threadIdx.x] = 0;
+    if (threadIdx.x == 0) s_count = 0;
+    if (threadIdx.x < 2) {  // first segment whose target is >= t0 (lane 0) / >= t1 (lane 1)
+        const int key = threadIdx.x == 0 ? t0 : t1;
+        int lo = 0, hi = nseg;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (target_row[mid] < key) lo = mid + 1; else hi = mid;
+        }
+        s_range[threadIdx.x] = lo;
     }
-    const int t = target_row[s];
-    const int prev = s > 0 ? target_row[s - 1] : -1;
-    if (t > prev + 1) psp_clear_rows(Y, (long long)(prev + 1) * nr, (long long)t * nr, N);  // rows no segment targets
-    const bool boundary = s > 0 && (s & ((1 << logW) - 1)) == 0 && prev == t;              // row continues across two wavefronts
-    const bool empty = rowPtr_split[s] == rowPtr_split[s + 1];
-    if (boundary || empty) psp_clear_rows(Y, (long long)t * nr, (long long)(t + 1) * nr, N);
+    __syncthreads();
+    const int lo = s_range[0], hi = s_range[1];
+    for (int s = lo + threadIdx.x; s < hi; s += 256) {
+        const int t = target_row[s];
+        s_targeted[t - t0] = 1;  // every writer stores the same value
+        const bool boundary = s > 0 && (s & ((1 << logW) - 1)) == 0 && target_row[s - 1] == t;  // continues across two wavefronts
+        const bool empty = rowPtr_split[s] == rowPtr_split[s + 1];
+        if (boundary || empty) s_added[t - t0] = 1;
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < t1 - t0 && (!s_targeted[threadIdx.x] || s_added[threadIdx.x]))
+        s_list[atomicAdd(&s_count, 1)] = t0 + threadIdx.x;
+    __syncthreads();
+    const int count = s_count;
+    const int lane = threadIdx.x & 63;
+    const size_t per_target = (size_t)nr * N, total = (size_t)rows_out * N;
+    const bool vec4 = (per_target & 3) == 0 && ((uintptr_t)Y & 15) == 0;
+    for (int i = threadIdx.x >> 6; i < count; i += 4) {
+        const size_t b0 = (size_t)s_list[i] * per_target;
+        const size_t b1 = min(total, b0 + per_target);  // the last target row may be cut by rows_out
+        if (vec4 && ((b1 - b0) & 3) == 0) {
+            const psp_f32x4 z = {0.f, 0.f, 0.f, 0.f};
+            for (size_t j = b0 + 4 * (size_t)lane; j < b1; j += 256) *(psp_f32x4 *)(Y + j) = z;
+        } else {
+            for (size_t j = b0 + lane; j < b1; j += 64) Y[j] = 0.0f;
+        }
+    }
 }
 
 int psp_split_clear(const int *rowPtr_split, const int *target_row, float *Y, int nseg, int N, int nr, int rows_out,
                     int logW, hipStream_t stream)
 {
-    hipLaunchKernelGGL(psp_split_clear_kernel, dim3(psp_ceil_div((long long)nseg + 1, 256)), dim3(256), 0, stream,
+    const int ntargets = (rows_out + nr - 1) / nr;
+    if (ntargets == 0 || N == 0) return PSP_OK;
+    hipLaunchKernelGGL(psp_split_clear_kernel, dim3(psp_ceil_div(ntargets, PSP_CLEAR_ROWS)), dim3(256), 0, stream,
                        rowPtr_split, target_row, Y, nseg, N, nr, rows_out, logW);
     return psp_check_launch("split clear kernel");
 }

@@ -52,7 +52,13 @@ __device__ __forceinline__ int psp_xcd_tile(int stripe)
     const int xcd = blockIdx.x % PSP_XCDS, idx = blockIdx.x / PSP_XCDS;
     return ((idx / stripe) * PSP_XCDS + xcd) * stripe + idx % stripe;
 }
-// rows (or segments) one stripe should span; PSP_XCD_STRIPE_ROWS in the environment overrides it (tuning aid)
+// library-wide options (psp_set_option); the environment is consulted once, when they are first needed
+struct psp_options {
+    int stripe_rows;            // rows (or segments) one XCD stripe should span
+    int align_pct;              // whole segments per lane group when that costs at most this many percent more steps
+    long long split_clear_min;  // row-split outputs of at least this many floats are cleared selectively
+};
+psp_options &psp_opts(void);
 int psp_stripe_rows(void);
 
 // zero-fill used instead of hipMemsetAsync (callers may capture these launches in a HIP graph)

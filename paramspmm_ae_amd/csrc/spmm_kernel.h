@@ -14,7 +14,10 @@
 //     of an X row per load;
 //   * colIdx / values are read once per L entries, coalesced (lane s takes entry base+s), and handed
 //     round the group with ds_bpermute; the next L are prefetched while the current ones are consumed;
-//   * U entries are unrolled so U*C feature loads are in flight per lane before the first FMA;
+//   * the walk is software-pipelined over batches of U entries, whatever rows they belong to: the U*C
+//     feature loads of batch t+1 are issued before batch t is added (two register sets alternate), so every
+//     lane group issues the same loads at the same time and only the closing of a row -- a store where a row
+//     ends -- diverges between groups;
 //   * a row cut by a group boundary is summed across the groups in registers (ds_bpermute), in group order,
 //     so plain CSR needs neither atomics nor a cleared Y.  Only a row whose segments lie in several
 //     wavefronts (row-split formats) is accumulated with fp32 atomics, once per wavefront.
@@ -278,94 +281,123 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     for (int r = 0; r < NR; r++) v_cur[r] = 0.0f;
     if (busy) PSP_FETCH(a, c_cur, v_cur);
 
-    // One step of the walk: U entries starting at chunk position k, all of the current row.  `guard` keeps
-    // entries past run_end (they belong to the next row or lie past the range) out of the sums.
-#define PSP_BATCH(GUARDED)                                                                          \
-    {                                                                                               \
-        int ck[U];                                                                                  \
-        float vk[U][NR];                                                                            \
-        _Pragma("unroll") for (int u = 0; u < U; u++)                                               \
-        {                                                                                           \
-            const int src = grp_base + min(k + u, L - 1);                                           \
-            ck[u] = psp_bperm_i(src, c_cur);                                                        \
-            _Pragma("unroll") for (int r = 0; r < NR; r++) vk[u][r] = psp_bperm_f(src, v_cur[r]);   \
-            if constexpr (SM) vk[u][0] = __expf(vk[u][0] - m_cur);                                  \
-        }                                                                                           \
-        vec_t x[U][C];                                                                              \
-        _Pragma("unroll") for (int u = 0; u < U; u++)                                               \
-        {                                                                                           \
-            const float *xr = X + (size_t)ck[u] * (size_t)N;                                        \
-            _Pragma("unroll") for (int i = 0; i < C; i++) x[u][i] = *(const vec_t *)(xr + off[i]);  \
-        }                                                                                           \
-        _Pragma("unroll") for (int u = 0; u < U; u++)                                               \
-        {                                                                                           \
-            if (!(GUARDED) || k + u < run_end) {                                                    \
-                if constexpr (SM) acc_l += vk[u][0];                                                \
-                _Pragma("unroll") for (int r = 0; r < NR; r++)                                      \
-                {                                                                                   \
-                    /* 2x1 blocks: a zero entry is skipped (SpMM_kernel.cu:1399,1405) */            \
-                    if (NR == 1 || vk[u][r] != 0.0f) {                                              \
-                        _Pragma("unroll") for (int i = 0; i < C; i++)                               \
-                            _Pragma("unroll") for (int e = 0; e < V; e++)                           \
-                                acc[r][i][e] = __builtin_fmaf(vk[u][r], psp_elem<V>(x[u][i], e), acc[r][i][e]); \
-                    }                                                                               \
-                }                                                                                   \
-            }                                                                                       \
-        }                                                                                           \
-    }
-
-    for (int base = a; base < b; base += L) {
-        int c_nxt = 0;
-        float v_nxt[NR];
+    // The entry just added closed its segment and the group's range goes on: move to the next filled segment
+    // (the table holds filled segments only) and, when that belongs to another row, hand the finished row on.
+    auto next_segment = [&]() {
+        const int2 nx = w_seg[++cur];
+        row_end = nx.x;
+        const int nkey = nx.y;
+        if (nkey != mykey) {
+            if (first_run && head_valid) {
 #pragma unroll
-        for (int r = 0; r < NR; r++) v_nxt[r] = 0.0f;
-        if (base + L < b) PSP_FETCH(base + L, c_nxt, v_nxt);
-
-        const int cnt = min(L, b - base);
-        int k = 0;
-        while (k < cnt) {
-            // the current row's entries inside this chunk: positions [k, run_end)
-            const int run_end = min(cnt, row_end - base);
-            for (; k + U <= run_end; k += U) PSP_BATCH(false)
-            if (k < run_end) PSP_BATCH(true)
-            k = run_end;
-            const int p = base + k;
-            if (p == row_end && p < b) {
-                // next segment (the table holds filled segments only, and p < b <= P1)
-                const int2 nx = w_seg[++cur];
-                row_end = nx.x;
-                const int nkey = nx.y;
-                if (nkey != mykey) {
-                    if (first_run && head_valid) {
+                for (int r = 0; r < NR; r++)
 #pragma unroll
-                        for (int r = 0; r < NR; r++)
+                    for (int i = 0; i < C; i++)
 #pragma unroll
-                            for (int i = 0; i < C; i++)
-#pragma unroll
-                                for (int e = 0; e < V; e++) head[r][i][e] = acc[r][i][e];
-                        head_l = acc_l;
-                        flags = F_HEAD | F_CLOSED;
-                    } else {
-                        write_out(mykey, first_run && ext_head);
-                    }
-#pragma unroll
-                    for (int r = 0; r < NR; r++)
-#pragma unroll
-                        for (int i = 0; i < C; i++)
-#pragma unroll
-                            for (int e = 0; e < V; e++) acc[r][i][e] = 0.0f;
-                    acc_l = 0.0f;
-                    first_run = false;
-                    mykey = nkey;
-                    if constexpr (SM) m_cur = s_m[wave][cur];
-                }
+                        for (int e = 0; e < V; e++) head[r][i][e] = acc[r][i][e];
+                head_l = acc_l;
+                flags = F_HEAD | F_CLOSED;
+            } else {
+                write_out(mykey, first_run && ext_head);
             }
-        }
-        c_cur = c_nxt;
 #pragma unroll
-        for (int r = 0; r < NR; r++) v_cur[r] = v_nxt[r];
+            for (int r = 0; r < NR; r++)
+#pragma unroll
+                for (int i = 0; i < C; i++)
+#pragma unroll
+                    for (int e = 0; e < V; e++) acc[r][i][e] = 0.0f;
+            acc_l = 0.0f;
+            first_run = false;
+            mykey = nkey;
+            if constexpr (SM) m_cur = s_m[wave][cur];
+        }
+    };
+
+    // The walk is software-pipelined over batches of U entries, whatever rows they belong to.  GATHER takes the
+    // next U (column, value) pairs of the group from the lanes that hold them and issues the feature loads;
+    // CONSUME adds a batch entry by entry and closes a row where one ends.  Two register sets alternate, so the
+    // loads of batch t+1 are in flight while batch t is added: every lane group of the wavefront issues the same
+    // loads at the same time (nothing before them depends on the row lengths), and only the short row-closing
+    // part diverges between groups.  Entries past the group's range (last, partial batch) are loaded from a valid
+    // address but never added, so values of other rows cannot leak in.
+    int pos = a;      // first entry of the next batch to gather
+    int cbase = a;    // first entry of the chunk c_cur / v_cur hold (lane `sub` holds entry cbase + sub)
+    int c_nxt = 0;
+    float v_nxt[NR];
+#pragma unroll
+    for (int r = 0; r < NR; r++) v_nxt[r] = 0.0f;
+    if (busy && a + L < b) PSP_FETCH(a + L, c_nxt, v_nxt);
+
+#define PSP_DECLARE(S)      \
+    int S##_ck[U], S##_pos; \
+    float S##_vk[U][NR];    \
+    vec_t S##_x[U][C];
+#define PSP_GATHER(S)                                                                                  \
+    {                                                                                                  \
+        int k_ = pos - cbase;                                                                          \
+        if (k_ == L) { /* the chunk is used up: the prefetched one becomes current, the next is requested */ \
+            c_cur = c_nxt;                                                                             \
+            _Pragma("unroll") for (int r = 0; r < NR; r++) v_cur[r] = v_nxt[r];                        \
+            cbase += L;                                                                                \
+            if (cbase + L < b) PSP_FETCH(cbase + L, c_nxt, v_nxt);                                     \
+            k_ = 0;                                                                                    \
+        }                                                                                              \
+        S##_pos = pos;                                                                                 \
+        _Pragma("unroll") for (int u = 0; u < U; u++)                                                  \
+        {                                                                                              \
+            const int src = grp_base + min(k_ + u, L - 1);                                             \
+            S##_ck[u] = psp_bperm_i(src, c_cur);                                                       \
+            _Pragma("unroll") for (int r = 0; r < NR; r++) S##_vk[u][r] = psp_bperm_f(src, v_cur[r]);  \
+        }                                                                                              \
+        _Pragma("unroll") for (int u = 0; u < U; u++)                                                  \
+        {                                                                                              \
+            const float *xr = X + (size_t)S##_ck[u] * (size_t)N;                                       \
+            _Pragma("unroll") for (int i = 0; i < C; i++) S##_x[u][i] = *(const vec_t *)(xr + off[i]); \
+        }                                                                                              \
+        pos += U;                                                                                      \
     }
-#undef PSP_BATCH
+#define PSP_CONSUME(S)                                                                                 \
+    {                                                                                                  \
+        _Pragma("unroll") for (int u = 0; u < U; u++)                                                  \
+        {                                                                                              \
+            const int p1 = S##_pos + u + 1;                                                            \
+            if (p1 <= b) {                                                                             \
+                if constexpr (SM) {                                                                    \
+                    S##_vk[u][0] = __expf(S##_vk[u][0] - m_cur);                                       \
+                    acc_l += S##_vk[u][0];                                                             \
+                }                                                                                      \
+                _Pragma("unroll") for (int r = 0; r < NR; r++)                                         \
+                {                                                                                      \
+                    /* 2x1 blocks: a zero entry is skipped (SpMM_kernel.cu:1399,1405) */               \
+                    if (NR == 1 || S##_vk[u][r] != 0.0f) {                                             \
+                        _Pragma("unroll") for (int i = 0; i < C; i++)                                  \
+                            _Pragma("unroll") for (int e = 0; e < V; e++)                              \
+                                acc[r][i][e] = __builtin_fmaf(S##_vk[u][r], psp_elem<V>(S##_x[u][i], e), acc[r][i][e]); \
+                    }                                                                                  \
+                }                                                                                      \
+                if (p1 == row_end && p1 < b) next_segment();                                           \
+            }                                                                                          \
+        }                                                                                              \
+    }
+
+    if (busy) {
+        PSP_DECLARE(A)
+        PSP_DECLARE(B)
+        PSP_GATHER(A)
+        while (true) {
+            bool more = pos < b;
+            if (more) PSP_GATHER(B)
+            PSP_CONSUME(A)
+            if (!more) break;
+            more = pos < b;
+            if (more) PSP_GATHER(A)
+            PSP_CONSUME(B)
+            if (!more) break;
+        }
+    }
+#undef PSP_DECLARE
+#undef PSP_GATHER
+#undef PSP_CONSUME
 #undef PSP_FETCH
 
     // ---- the row this group stopped in ----------------------------------------------------------------

@@ -32,19 +32,18 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     // wavefronts for every SIMD.
     const int logR = 6 - logL;
     int logW = SPLIT ? (logR > 4 ? logR : 4) : logR;
-    const char *w_env = getenv("PSP_LOG_SEGS_PER_WAVE");  // tuning aid
-    if (w_env && atoi(w_env) >= 0 && atoi(w_env) <= 6) logW = atoi(w_env);
+    if (plan.log_segs_per_wave >= 0) logW = plan.log_segs_per_wave;  // chosen by a native configuration
     while (logW > 0 && (nrows >> logW) < 4096) logW--;
     if (logW < logR - 1) logW = logR - 1;
+    if (logW > 6) logW = 6;
+    const psp_options &opt = psp_opts();
 
     // rows the kernel does not store to must read as zero
     if (SPLIT) {
         // The kernel stores rows that one wavefront holds alone and adds (atomics) to rows shared by several
         // wavefronts.  Large outputs are therefore not cleared as a whole: a pass over the segments clears only
         // the shared rows and the rows without segments.  Small outputs are cheaper to clear outright.
-        size_t clear_min = (size_t)32 << 20;  // floats
-        if (const char *c_env = getenv("PSP_SPLIT_CLEAR_MIN")) clear_min = (size_t)atoll(c_env);  // tuning / test aid
-        if ((size_t)rows_out * N >= clear_min && nrows > 0)
+        if ((long long)rows_out * N >= opt.split_clear_min && nrows > 0)
             rc = psp_split_clear(rowPtr, target_row, Y, nrows, N, NR, rows_out, logW, stream);
         else
             rc = psp_zero_f32(Y, (size_t)rows_out * N, stream);
@@ -61,16 +60,14 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
         if (rc != PSP_OK) return rc;
     }
 
+    const int segs_per_block = plan.waves_per_block << logW;
     psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll, softmax);
     if (!k)
         return psp_fail(PSP_ERR_ARG, "spmm%s: no kernel for coarsen %d vec %d unroll %d%s", softmax ? " softmax" : "", plan.coarsen,
                         plan.vec, plan.unroll, softmax ? " (needs N % 4 == 0 and CF <= 4)" : "");
 
-    int align_pct = 50;
-    const char *a_env = getenv("PSP_ALIGN_PCT");  // tuning aid
-    if (a_env) align_pct = atoi(a_env);
-    const int segs_per_block = plan.waves_per_block << logW;
-    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block), psp_stripe_rows() / segs_per_block);
+    const int align_pct = plan.even_split ? 0 : opt.align_pct;
+    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block), opt.stripe_rows / segs_per_block);
     dim3 grid(g.launch, plan.col_tiles, 1), block(plan.waves_per_block * PSP_WAVE, 1, 1);
     hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.stripe, align_pct, row_max, row_sum);
     rc = psp_check_launch("spmm kernel");

@@ -45,6 +45,12 @@ static void check_sddmm_args(int fmt, const Tensor &A, const Tensor &B, const Te
     }
     if (fmt == 0) TORCH_CHECK(rows <= A.size(0), "rowPtr describes more rows than A has");
     if (fmt == 2) TORCH_CHECK(2 * rows <= A.size(0), "A needs two rows per block-row (pad it to an even row count)");
+    // Row-split block format: the segments do not say how many block-rows there are, but the matrix is square
+    // (B has one row per column, as everywhere in the reference), and the kernel reads both rows of a block-row
+    // whatever the block values are.  So A must cover B's rows rounded up to whole blocks.
+    if (fmt == 3)
+        TORCH_CHECK(A.size(0) % 2 == 0 && A.size(0) >= (B.size(0) + 1) / 2 * 2,
+                    "A needs two rows per block-row: pad it to an even row count of at least ", (B.size(0) + 1) / 2 * 2);
 }
 
 static Tensor sddmm_new(int fmt, const Tensor &A, const Tensor &B, const Tensor &rowPtr, const Tensor &colIdx,
@@ -246,6 +252,10 @@ static void check_vec_sddmm_args(const Tensor &A, const Tensor &B, const Tensor 
         need_i32(*target_row, "target_row");
         same_device(A, *target_row, "vec_sddmm");
         TORCH_CHECK(target_row->size(0) == rowPtr.size(0) - 1, "target_row must have one entry per row segment");
+        // square matrix: A must cover B's rows rounded up to whole blocks (the kernel reads every row of a block-row)
+        const long R = values.size(1), need = (B.size(0) + R - 1) / R * R;
+        TORCH_CHECK(A.size(0) % R == 0 && A.size(0) >= need, "A needs vec_size rows per block-row: pad it to a multiple of ", R,
+                    " of at least ", need);
     } else {
         TORCH_CHECK(values.size(1) * (rowPtr.size(0) - 1) <= A.size(0), "A needs vec_size rows per block-row (pad it)");
     }

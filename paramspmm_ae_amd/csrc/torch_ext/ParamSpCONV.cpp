@@ -9,7 +9,7 @@ using torch::Tensor;
 static void check_cf(int CF)
 {
     // SpCONV dispatches CF 1..4 only (SpCONV/SpCONV.cpp:92-124)
-    TORCH_CHECK(CF >= 1 && CF <= 8, "CF must be 1..8");
+    TORCH_CHECK((CF >= 1 && CF <= 8) || (CF & PSP_CF_NATIVE), "CF must be 1..8 (or a native configuration)");
 }
 
 // A*D for a dense D, result cut back to rows(D) (the blocked formats compute into an even-padded buffer,

@@ -36,7 +36,8 @@ static Tensor spmm_softmax(int fmt, const Tensor &X, const Tensor &rowPtr, const
     need_gpu(row_max, "row_max");
     need_f32(row_max, "row_max", 1);
     TORCH_CHECK(row_max.size(0) >= X.size(0) || fmt == 0, "row_max must hold one value per matrix row");
-    TORCH_CHECK(X.size(1) % 4 == 0 && CF <= 4, "softmax-weighted SpMM needs a width that is a multiple of 4 and CF <= 4");
+    TORCH_CHECK(X.size(1) % 4 == 0 && ((CF & PSP_CF_NATIVE) ? (CF & 7) < 4 : CF <= 4),
+                "softmax-weighted SpMM needs a width that is a multiple of 4 and CF <= 4");
     pspglue::DeviceGuard guard(X.device());
     auto Y = torch::empty_like(X);
     const int nseg = (int)rowPtr.size(0) - 1, N = (int)X.size(1), rows_out = (int)Y.size(0);
@@ -263,6 +264,8 @@ static py::dict spmm_plan(int N, int CF, int blkWarpNum)
     d["unroll"] = p.unroll;
     d["col_tiles"] = p.col_tiles;
     d["waves_per_block"] = p.waves_per_block;
+    d["log_segs_per_wave"] = p.log_segs_per_wave;
+    d["even_split"] = p.even_split;
     return d;
 }
 

@@ -3,14 +3,15 @@ matrix features (same surface as the reference's decider.py:18-93).
 
 The forests are the ones trained on MI355X timings by ``train_decider.py`` and stored as
 ``rnd_tree_<dim>.pkl`` (one per multiple of 16 up to 256).  The class code is the column index of the sweep
-table: blkWarpNum-major, then CF in ``dynamic_CF_prompter(dim)`` order, then the four representations
+table: blkWarpNum-major, then CF in ``decider_CF_list(dim)`` order (the reference's ``dynamic_CF_prompter`` list
+followed by native wave64 configurations packed into the same integer), then the four representations
 (vec1, vec1_split, vec2, vec2_split) -- see ``decode_tree``.
 """
 import math
 import os
 import pickle
 
-from .PCSR import dynamic_CF_prompter
+from .PCSR import decider_CF_list, dynamic_CF_prompter
 
 DEFAULT_PICKLE_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "models") + os.sep
 
@@ -43,9 +44,11 @@ class SpMMDecider(object):
             raise ValueError("dim_list must be assigned and non-empty")
         self.model_dict = {dim: self.load_pickle(model_dim_for(dim)) for dim in dim_list}
 
-    def decode_tree(self, code, dim, vec_size_list=(1, 2), warpNum_list=(4, 8)):
-        """class code -> (if_split, vec_size, CF, blkWarpNum) (decider.py:63-80); if_split is the int 0/1."""
-        CF_list = dynamic_CF_prompter(dim)
+    def decode_tree(self, code, dim, vec_size_list=(1, 2), warpNum_list=(4, 8), CF_list=None):
+        """class code -> (if_split, vec_size, CF, blkWarpNum) (decider.py:63-80); if_split is the int 0/1.
+        ``CF_list``: the CF axis the forest was trained on; default ``decider_CF_list(dim)`` (the reference's list
+        followed by the native configurations)."""
+        CF_list = decider_CF_list(dim) if CF_list is None else CF_list
         code = int(code)
         if_split = code % 2
         code //= 2
@@ -58,8 +61,13 @@ class SpMMDecider(object):
     def config_PCSR(self, graph, dim):
         if dim not in self.model_dict:
             raise ValueError("dim-" + str(dim) + " not found in model_dict")
-        code = self.model_dict[dim].predict(graph.get_info()).item()
-        return self.decode_tree(code, math.ceil(dim / 16) * 16)
+        model = self.model_dict[dim]
+        code = model.predict(graph.get_info()).item()
+        # a forest records the CF axis of its training table in ``psp_cf_list_`` (train_decider.py); one without it
+        # was trained on the reference's own table (python -m paramspmm_ae_amd.PCSR, PCSR.py:781-788)
+        rounded = math.ceil(dim / 16) * 16
+        cf_list = getattr(model, "psp_cf_list_", None)
+        return self.decode_tree(code, rounded, CF_list=dynamic_CF_prompter(rounded) if cf_list is None else list(cf_list))
 
 
 def evaluate(filelist, path, dim_list, pickle_path=DEFAULT_PICKLE_PATH, verbose=True):

@@ -1,27 +1,35 @@
 """Configuration sweep: times every ``<representation, CF, blkWarpNum>`` of a graph for a list of feature
 widths.  It is the counterpart of the reference's ``profile_engine`` (PCSR.py:672-806) and produces the same
-column order -- blkWarpNum-major, then CF in ``dynamic_CF_prompter`` order, then the representations vec1,
-vec1_split, vec2, vec2_split -- so that the arg-max column index is the class code ``decode_tree`` expects.
+column order -- blkWarpNum-major, then CF in list order, then the representations vec1, vec1_split, vec2,
+vec2_split -- so that the arg-max column index is the class code ``decode_tree`` expects.  The CF list is
+``decider_CF_list``: the reference's ``dynamic_CF_prompter`` entries followed by native wave64 configurations
+(lanes per row, entries in flight, even division), which travel in the same integer argument.
 """
 import numpy as np
 import torch
 
-from .PCSR import dynamic_CF_prompter, pcsr_spmm
+from .PCSR import cf_label, decider_CF_list, dynamic_CF_prompter, native_CF_prompter, pcsr_spmm
 
 WARP_NUMS = (4, 8)
 REPRESENTATIONS = (("vec1", 1, False), ("vec1_split", 1, True), ("vec2", 2, False), ("vec2_split", 2, True))
 
 
+def native_configs(dim):
+    """The packed CF values the sweep adds to the reference's list for ``dim``."""
+    return native_CF_prompter(dim)
+
+
 def column_names(dim, cfs=None, vec_size=2):
-    """``cfs``: the CF list when it is not ``dynamic_CF_prompter(dim)`` (the reference's --if_DCP False ablation)"""
-    cfs = dynamic_CF_prompter(dim) if cfs is None else cfs
+    """``cfs``: the CF list when it is not ``decider_CF_list(dim)`` (the reference's own list, or its --if_DCP False
+    ablation)"""
+    cfs = decider_CF_list(dim) if cfs is None else cfs
     reps = ("vec1", "vec1_split", "vec%d" % vec_size, "vec%d_split" % vec_size)
-    return ["%s_TP_%d%d" % (rep, cf, bw) for bw in WARP_NUMS for cf in cfs for rep in reps]
+    return ["%s_TP_%s%d" % (rep, cf_label(cf), bw) for bw in WARP_NUMS for cf in cfs for rep in reps]
 
 
-def decode_column(dim, col):
+def decode_column(dim, col, cfs=None):
     """column index -> (if_split, vec_size, CF, blkWarpNum): the arithmetic of decider.py:63-80."""
-    cfs = dynamic_CF_prompter(dim)
+    cfs = decider_CF_list(dim) if cfs is None else cfs
     _, vec_size, if_split = REPRESENTATIONS[col % 4]
     cf = cfs[col // 4 % len(cfs)]
     bw = WARP_NUMS[col // (4 * len(cfs))]
@@ -44,7 +52,7 @@ def sweep_dim(ops, dim, nnz, n_rows, warmup=3, iters=10, X=None, verify=None, cf
     rows = (n_rows + pad - 1) // pad * pad
     if X is None:
         X = torch.ones(rows, dim, device="cuda")
-    cfs = dynamic_CF_prompter(dim) if cfs is None else cfs
+    cfs = decider_CF_list(dim) if cfs is None else cfs
     names = column_names(dim, cfs, ops[-1].vec_size if ops[-1].vec_size != 1 else 2)
     ms = np.zeros(len(names))
     col = 0

@@ -255,7 +255,17 @@ def fit_main(args):
               "seed / hub degree / ordering): every matrix is predicted by a forest that has seen neither it nor "
               "its siblings", "per_dim": {}}
     folds = list(GroupKFold(5).split(X, groups=groups))
+    from . import sweep as sw
+    from .PCSR import decider_CF_list, dynamic_CF_prompter
+
+    cf_lists = {}
     for d in DIMS:
+        # the table's CF axis: the widened list, or the reference's own when the data come from its sweep
+        if list(tps[d].columns) == sw.column_names(d):
+            cf_lists[d] = decider_CF_list(d)
+        else:
+            assert list(tps[d].columns) == sw.column_names(d, dynamic_CF_prompter(d)), "unknown column set at dim %d" % d
+            cf_lists[d] = dynamic_CF_prompter(d)
         TP = tps[d].to_numpy(dtype=np.float64)
         y = TP.argmax(axis=1)  # class code = column index (PCSR.py:815-818)
         # label csv in the reference's schema
@@ -272,7 +282,26 @@ def fit_main(args):
                 if best is None or score > best[0]:
                     best = (score, near, n_est, leaves, pick, norm)
         (within10, mean_norm), near, n_est, leaves, pick, norm = best
+        n_legacy = 4 * len(dynamic_CF_prompter(d))
+        legacy_cols = np.array([c % (4 * len(cf_lists[d])) < n_legacy for c in range(TP.shape[1])])
+        best_all, best_legacy = TP.max(axis=1), TP[:, legacy_cols].max(axis=1)
+        gain = best_all / best_legacy  # what the native configurations add over the reference's <CF, blkWarpNum> space
+        by_family = {}
+        for fam in ("cl_", "rmat_", "sbm_", "stencil_", "grid_", "band_"):
+            sel = np.array([n.startswith(fam) for n in info["mtx_name"]])
+            if fam == "sbm_":
+                for tag, m in (("sbm_ordered", np.array([n.split("_r")[0].endswith("_s") for n in info["mtx_name"]])),
+                               ("sbm_permuted", np.array([n.split("_r")[0].endswith("_p") for n in info["mtx_name"]]))):
+                    if (sel & m).any():
+                        by_family[tag] = float(gain[sel & m].mean())
+            elif sel.any():
+                by_family[fam.rstrip("_")] = float(gain[sel].mean())
         report["per_dim"][d] = {
+            "cf_axis": [sw.cf_label(c) for c in cf_lists[d]],
+            "native_gain_over_reference_space": {"mean": float(gain.mean()), "max": float(gain.max()),
+                                                 "share_of_matrices_with_gain_over_5pct": float(np.mean(gain > 1.05)),
+                                                 "mean_by_family": by_family},
+            "share_of_picks_that_are_native": float(np.mean(~legacy_cols[pick])),
             "near_best_threshold": near, "n_estimators": n_est, "max_leaf_nodes": leaves, "classes": int(TP.shape[1]),
             "validated_matrices": int(len(X)), "accuracy": float(np.mean(pick == y)),
             "mean_normalised_performance": mean_norm, "share_within_10pct_of_best": within10,
@@ -281,6 +310,7 @@ def fit_main(args):
         # the shipped model is refitted on every matrix
         final = _fit_forest(X, TP, near, n_est, leaves)
         final.n_jobs = 1
+        final.psp_cf_list_ = [int(c) for c in cf_lists[d]]  # the CF axis of the class codes (decider.config_PCSR)
         with open(os.path.join(args.out, "rnd_tree_%d.pkl" % d), "wb") as f:
             pickle.dump(final, f)
         print("dim %3d: %2d classes  near %.2f  n_estimators %d  leaves %d  acc %.3f  mean norm perf %.4f  within 10%%: %.3f  worst %.3f" % (

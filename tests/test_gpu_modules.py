@@ -108,6 +108,24 @@ def test_extension_argument_errors():
         ParamSDDMM.vec_sddmm(x, x, rp, ci, torch.zeros(0, 5, device="cuda"), 1, 4)
     with pytest.raises(RuntimeError, match="same number of columns"):
         ParamSDDMM.csr_sddmm(x, torch.zeros(8, 8, device="cuda"), rp, ci, v, 1, 4)
+    # odd row count and an unpadded A: the row-split block operators refuse it like the plain ones (the kernel
+    # reads both rows of the last block-row)
+    a7, b7 = torch.zeros(7, 16, device="cuda"), torch.zeros(7, 16, device="cuda")
+    rps = torch.tensor([0, 1], dtype=torch.int32, device="cuda")
+    tr = torch.tensor([3], dtype=torch.int32, device="cuda")
+    ci1 = torch.tensor([2], dtype=torch.int32, device="cuda")
+    with pytest.raises(RuntimeError, match="two rows per block-row"):
+        ParamSDDMM.bcsr_sddmm(a7, b7, torch.tensor([0, 0, 0, 0, 1], dtype=torch.int32, device="cuda"), ci1,
+                              torch.ones(1, 2, device="cuda"), 1, 4)
+    with pytest.raises(RuntimeError, match="two rows per block-row"):
+        ParamSDDMM.bcsr_split_sddmm(a7, b7, rps, ci1, torch.ones(1, 2, device="cuda"), tr, 1, 4)
+    with pytest.raises(RuntimeError, match="vec_size rows per block-row"):
+        ParamSDDMM.vec_split_sddmm(a7, b7, rps, ci1, torch.ones(1, 3, device="cuda"),
+                                   torch.tensor([2], dtype=torch.int32, device="cuda"), 1, 4)
+    a8 = torch.ones(8, 16, device="cuda")
+    got = ParamSDDMM.bcsr_split_sddmm(a8, torch.ones(7, 16, device="cuda"), rps, ci1,
+                                      torch.tensor([[1.0, 0.0]], device="cuda"), tr, 1, 4)
+    assert got.tolist() == [[16.0, 0.0]]
     # bcsr output is padded to an even number of rows
     xo = torch.zeros(7, 16, device="cuda")
     rpb = torch.zeros(5, dtype=torch.int32, device="cuda")

@@ -129,14 +129,24 @@ def test_spmm_linearity_and_format_agreement_at_scale(oracle):
     assert_close(spmm_capi("csr", F, X1[:, :16].contiguous(), 1, 4), want, what="rmat17 N=16")
 
 
+@pytest.fixture
+def selective_clear_always():
+    """Row-split outputs of any size take the selective-clear path while the test runs."""
+    from paramspmm_ae_amd import _capi
+
+    before = _capi.get_option("split_clear_min")
+    _capi.set_option("split_clear_min", 0)
+    yield
+    _capi.set_option("split_clear_min", before)
+
+
 @pytest.mark.parametrize("fmt", ["csr_split", "bcsr_split"])
-def test_split_selective_clear_path(oracle, fmt, monkeypatch):
+def test_split_selective_clear_path(oracle, fmt, selective_clear_always):
     """Large outputs of the row-split formats are not cleared as a whole: only rows shared by two wavefronts, rows
     of empty segments and rows without segments are.  Force that path on a small matrix with long rows, empty
-    rows at the start, in the middle and at the end, and a poisoned Y."""
+    rows at the start, in the middle and at the end (runs of hundreds of rows nothing targets), and a poisoned Y."""
     from gpu_util import Formats, spmm_capi, spmm_oracle, spmm_abs_scale, assert_close
 
-    monkeypatch.setenv("PSP_SPLIT_CLEAR_MIN", "0")
     rowPtr, colIdx, val = random_csr(6000, 14, 21, empty_frac=0.3, hub=(3000, 2500), values="uniform")
     k = np.diff(rowPtr).copy()
     k[:70] = 0
@@ -146,7 +156,7 @@ def test_split_selective_clear_path(oracle, fmt, monkeypatch):
     rowPtr = np.concatenate([[0], np.cumsum(k)]).astype(np.int32)
     colIdx, val = colIdx[keep], val[keep]
     F = Formats(oracle, rowPtr, colIdx, val, g=8, gb=8)
-    for N in (16, 128):
+    for N in (16, 128, 50):
         X = np.random.default_rng(N).standard_normal((F.n, N)).astype(np.float32)
         want = spmm_oracle(oracle, fmt, F, X)
         scale = spmm_abs_scale(oracle, F, X, want.shape[0])
@@ -297,3 +307,38 @@ def test_spmm_non_finite_inputs_stay_in_their_rows(oracle, fmt):
         assert np.array_equal(np.isposinf(got), np.isposinf(want)) and np.array_equal(np.isneginf(got), np.isneginf(want))
         fin = np.isfinite(want)
         np.testing.assert_allclose(got[fin], want[fin], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_spmm_native_configurations(oracle, fmt):
+    """The wave64 parameter space carried in the CF argument (lanes per row, vectors per lane, entries in flight,
+    segments per wavefront, even division) against the oracle: every combination the sweep can emit, on a matrix
+    with a hub row, empty rows and an odd row count, at widths with and without a partial column tile."""
+    from gpu_util import Formats, spmm_capi, spmm_oracle, spmm_abs_scale, assert_close
+    from paramspmm_ae_amd import _capi
+    from paramspmm_ae_amd.sweep import native_configs
+
+    rowPtr, colIdx, val = random_csr(3001, 9, 77, empty_frac=0.15, hub=(17, 1900), values="normal")
+    F = Formats(oracle, rowPtr, colIdx, val)
+    for N in (16, 48, 100, 128, 256):
+        X = np.random.default_rng(N).standard_normal((F.n + (F.n & 1), N)).astype(np.float32)
+        want = spmm_oracle(oracle, fmt, F, X)
+        scale = spmm_abs_scale(oracle, F, X, want.shape[0])
+        Xd = torch.from_numpy(X).cuda()
+        cfs = list(native_configs(N))
+        # beyond the sweep's list: odd corners of the space
+        cfs += [_capi.pack_cf(1, 1, 1), _capi.pack_cf(1, 64, 1, 1), _capi.pack_cf(1, 2, 2, 64, even_split=True),
+                _capi.pack_cf(3, 8, 2, 4), _capi.pack_cf(8, 4, 1, 2)]
+        for cf in cfs:
+            for bw in (4, 8):
+                print("case", fmt, N, _capi.unpack_cf(cf), bw, flush=True)
+                got = spmm_capi(fmt, F, Xd, cf, bw)
+                torch.cuda.synchronize()
+                assert_close(got, want, what="%s N=%d native %s bw=%d" % (fmt, N, _capi.unpack_cf(cf), bw), scale=scale)
+    # malformed native values are argument errors
+    p = _capi.ptr
+    x = torch.zeros(4, 16, device="cuda")
+    rp = torch.zeros(5, dtype=torch.int32, device="cuda")
+    for bad in (_capi.CF_NATIVE | (7 << 3), _capi.CF_NATIVE | (1 << 13), _capi.pack_cf(4, 8, 2) | (3 << 6),
+                _capi.CF_NATIVE | (2 << 6) | (1 << 3)):
+        assert _capi.lib.psp_spmm_csr_f32(p(rp), None, None, p(x), p(x), 4, 16, 4, bad, 4, None) == -1

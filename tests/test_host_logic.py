@@ -42,9 +42,23 @@ def test_spmm_plan_mapping():
                 assert p["rows_per_wave"] * p["lanes_per_row"] == 64
                 assert 1 <= p["unroll"] <= p["lanes_per_row"]
     assert _capi.spmm_plan(50, 1, 4)["vec"] == 2 and _capi.spmm_plan(51, 1, 4)["vec"] == 1
-    for bad in ((16, 0, 4), (16, 9, 4), (16, 1, 6), (0, 1, 4)):
+    for bad in ((16, 0, 4), (16, 9, 4), (16, 1, 6), (0, 1, 4), (64, _capi.CF_NATIVE | (7 << 3), 4),
+                (64, _capi.pack_cf(4, 8, 2) | (3 << 6), 4), (64, _capi.CF_NATIVE | (1 << 14), 4)):
         with pytest.raises(_capi.ParamSpError):
             _capi.spmm_plan(*bad)
+    # native configurations: every field is honoured, vectors per lane are capped by the width
+    p = _capi.spmm_plan(128, _capi.pack_cf(2, 16, 2, 32, even_split=True), 8)
+    assert (p["coarsen"], p["lanes_per_row"], p["rows_per_wave"], p["unroll"], p["col_tiles"], p["log_segs_per_wave"],
+            p["even_split"]) == (2, 16, 4, 2, 1, 5, 1)
+    assert _capi.spmm_plan(16, _capi.pack_cf(4, 8, 2), 4)["coarsen"] == 4
+    assert _capi.spmm_plan(8, _capi.pack_cf(4, 8, 2), 4)["coarsen"] == 2
+    # options
+    assert _capi.get_option("align_pct") == 50 and _capi.get_option("xcd_stripe_rows") == 8192
+    _capi.set_option("align_pct", 25)
+    assert _capi.get_option("align_pct") == 25
+    _capi.set_option("align_pct", 50)
+    with pytest.raises(_capi.ParamSpError):
+        _capi.set_option("no_such_option", 1)
 
 
 @pytest.mark.parametrize("g", [1, 7, 32, 96])
@@ -182,9 +196,9 @@ def test_format_builder_from_arrays_and_synthetic_closed_form(oracle):
 
 def test_cf_search_space_and_decoding_match_reference_integers(oracle):
     from oracle.oracle import CF_TABLE
-    from paramspmm_ae_amd.PCSR import dynamic_CF_prompter, gap_calculator
+    from paramspmm_ae_amd.PCSR import decider_CF_list, dynamic_CF_prompter, gap_calculator
     from paramspmm_ae_amd.decider import SpMMDecider, model_dim_for
-    from paramspmm_ae_amd import sweep
+    from paramspmm_ae_amd import _capi, sweep
 
     for dim in range(1, 300):
         assert dynamic_CF_prompter(dim) == oracle.dynamic_CF_prompter(dim)
@@ -195,13 +209,31 @@ def test_cf_search_space_and_decoding_match_reference_integers(oracle):
         assert dynamic_CF_prompter(dim) == cfs
     d = SpMMDecider("unused/")
     for dim, cfs in CF_TABLE.items():
-        names = sweep.column_names(dim)
+        # the reference's own class space: 8 * |CF_list| codes, decoded with its arithmetic
+        names = sweep.column_names(dim, cfs)
         assert len(names) == 8 * len(cfs)
         for code in range(8 * len(cfs)):
-            got = d.decode_tree(code, dim)
-            assert got == oracle.decode_tree(code, dim) == sweep.decode_column(dim, code)
+            got = d.decode_tree(code, dim, CF_list=cfs)
+            assert got == oracle.decode_tree(code, dim) == sweep.decode_column(dim, code, cfs)
             rep = ["vec1", "vec1_split", "vec2", "vec2_split"][code % 4]
             assert names[code] == "%s_TP_%d%d" % (rep, got[2], got[3])
+        # the widened space: the same arithmetic over the reference's list followed by the native configurations
+        wide = decider_CF_list(dim)
+        assert wide[: len(cfs)] == cfs and all(c & _capi.CF_NATIVE for c in wide[len(cfs):])
+        assert wide == decider_CF_list(dim - 15)  # one list per 32-wide band, like the forests (decider.py:52-55)
+        names = sweep.column_names(dim)
+        assert len(names) == len(set(names)) == 8 * len(wide)
+        for code in range(8 * len(wide)):
+            if_split, vec, cf, bw = d.decode_tree(code, dim)
+            assert (if_split, vec, cf, bw) == sweep.decode_column(dim, code)
+            assert (if_split, vec) == ((code % 2), (1, 2)[code // 2 % 2]) and cf == wide[code // 4 % len(wide)]
+            assert bw == (4, 8)[code // (4 * len(wide))]
+            plan = _capi.spmm_plan(dim, cf, bw)  # every class is a configuration the library accepts
+            assert plan["lanes_per_row"] * plan["coarsen"] * plan["vec"] * plan["col_tiles"] >= dim
+            if cf & _capi.CF_NATIVE:
+                c, lanes, unroll, segs, even = _capi.unpack_cf(cf)
+                assert (plan["coarsen"], plan["lanes_per_row"], plan["unroll"], bool(plan["even_split"])) == (c, lanes, unroll, even)
+                assert _capi.pack_cf(c, lanes, unroll, segs, even) == cf
     assert [model_dim_for(x) for x in (16, 24, 32, 40, 48, 100, 128, 250)] == [16, 16, 32, 48, 48, 112, 128, 240]
 
 
@@ -233,8 +265,21 @@ def test_decider_round_trip_with_a_forest_trained_in_test(tmp_path):
     d.gen_model_dict([64, 40, 48])  # 40 and 48 share the forest of 48
     assert d.model_dict[40] is d.model_dict[48]
     lo, hi = np.full(15, 0.1), np.full(15, 0.9)
-    assert d.config_PCSR(G(lo), 64) == d.decode_tree(1, 64) == (1, 1, 1, 4)
-    assert d.config_PCSR(G(hi), 64) == d.decode_tree(6, 64) == (0, 2, 2, 4)
+    # a forest without a recorded CF axis was trained on the reference's table
+    assert d.config_PCSR(G(lo), 64) == d.decode_tree(1, 64, CF_list=[1, 2]) == (1, 1, 1, 4)
+    assert d.config_PCSR(G(hi), 64) == d.decode_tree(6, 64, CF_list=[1, 2]) == (0, 2, 2, 4)
+    # one that records the widened axis decodes over it: class 38 = blkWarpNum 8, fifth CF of the list, vec2
+    from paramspmm_ae_amd.PCSR import decider_CF_list
+
+    wide = decider_CF_list(64)
+    clf2 = RandomForestClassifier(n_estimators=5, random_state=0).fit(X, np.where(X[:, 0] > 0.5, 38, 9))
+    clf2.psp_cf_list_ = wide
+    with open(tmp_path / "rnd_tree_64.pkl", "wb") as f:
+        pickle.dump(clf2, f)
+    d2 = SpMMDecider(str(tmp_path) + os.sep)
+    d2.gen_model_dict([64])
+    assert d2.config_PCSR(G(hi), 64) == (0, 2, wide[4], 8)
+    assert d2.config_PCSR(G(lo), 64) == (1, 1, wide[2], 4)
     with pytest.raises(ValueError, match="not found in model_dict"):
         d.config_PCSR(G(lo), 128)
 
@@ -318,7 +363,7 @@ def test_sddmm_harness_checks_and_column_orders():
     """compare / compare_2d (SDDMM.py:19-43) and the column orders of the two sweep tables"""
     import torch
     from paramspmm_ae_amd import SDDMM as S
-    from paramspmm_ae_amd import sweep
+    from paramspmm_ae_amd import _capi, sweep
     from paramspmm_ae_amd.PCSR import dynamic_CF_prompter
 
     ref = torch.tensor([32.0, 32.0, 32.0])
@@ -340,4 +385,5 @@ def test_sddmm_harness_checks_and_column_orders():
         names = sweep.column_names(dim)
         for col, name in enumerate(names):
             if_split, vec_size, cf, bw = sweep.decode_column(dim, col)
-            assert name == "vec%d%s_TP_%d%d" % (vec_size, "_split" if if_split else "", cf, bw)
+            assert name == "vec%d%s_TP_%s%d" % (vec_size, "_split" if if_split else "", sweep.cf_label(cf), bw)
+    assert sweep.cf_label(3) == "3" and sweep.cf_label(_capi.pack_cf(2, 16, 2, 8, even_split=True)) == "c2l16u2w8e"
