@@ -8,14 +8,22 @@ sweep over the PCSR configurations, or the trained decider's pick with --pick de
 in HBM before the timed region.  value = sum(2*nnz*N) * steps / wall time, in GFLOP/s.
 
 The JSON line also carries
-  roofline      for the width that takes the most time: algorithmic bytes
-                4(M+1) + 8 nnz + 4 n N + 4 M N (CSR; split adds 8 S + 4, blocks use 4(Mb+1) + 12 nblk)
-                divided by that launch's mean duration (HIP events on the launching stream), against 8 TB/s;
-  sweep         the same numbers for every width;
-  cpu_baseline  the oracle's scalar C port of the CSR kernel on a bounded sample of the widths (it also checks the GPU
-                result there); cpu_torch_sparse_mm is the host product the reference verifies against, for scale.
+  roofline         for the kernel symbol that takes the most time: algorithmic bytes
+                   4(M+1) + 8 nnz + 4 n N + 4 M N (CSR; split adds 8 S + 4, blocks use 4(Mb+1) + 12 nblk)
+                   divided by that launch's mean duration (HIP events on the launching stream), against 8 TB/s;
+                   gather_ceiling_frac = duration of the bare gathers of the same pattern and width
+                   (psp_probe_gather_f32: same colIdx stream, same X row tiles, no rows, no FMAs) / kernel duration;
+  sweep            the same numbers for every width;
+  decider_vs_best  t(decider's pick) / t(best swept configuration) per width, from a short sweep of every
+                   <representation, CF, blkWarpNum> after the timed region (PCSR.py:754-788, rnd_tree.ipynb cell 4);
+  sddmm            one SDDMM width (K = 64) on the same pattern with its own roofline;
+  gcn_epoch_ms     20 GCN training epochs (5 layers, hidden 16, 16 classes) on the 1M-node block model (GNN.py:126-151);
+  cpu_baseline     torch.sparse.mm on the host cores (the product the reference verifies against, verification.py:18-46)
+                   on a bounded sample of the widths; cpu_scalar_port is the oracle's one-thread C restatement, which also
+                   checks the GPU result at those widths.
 """
 import argparse
+import contextlib
 import json
 import os
 import sys
@@ -27,6 +35,7 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+DEFAULT_DIMS = ",".join(str(d) for d in range(16, 257, 16))
 
 
 def algorithmic_bytes(fmt, F, n_x_rows, N):
@@ -64,6 +73,79 @@ def measured_traffic(graph, rows_of):
             return None
         total += table[key]
     return int(total / len(rows_of))
+
+
+def gather_probe_ms(colIdx_dev, nnz, X, lanes, reps=5):
+    """Best duration (ms) of the bare gathers of this pattern at X's width: psp_probe_gather_f32 over a few shapes."""
+    import torch
+    from paramspmm_ae_amd import _capi
+
+    L, p = _capi.lib, _capi.ptr
+    N = X.shape[1]
+    stream = torch.cuda.current_stream().cuda_stream
+    best = None
+    for unroll in (4, 8):
+        if unroll > lanes:
+            continue
+        for per_wave in (512, 2048):
+            need = L.psp_probe_gather_out_floats(nnz, N, lanes, per_wave)
+            out = torch.empty(need, device="cuda")
+            call = lambda: L.psp_probe_gather_f32(p(colIdx_dev), nnz, p(X), N, lanes, unroll, per_wave, p(out), need, stream)
+            _capi.check(call())
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(reps):
+                call()
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1) / reps
+            if best is None or ms < best[0]:
+                best = (ms, unroll, per_wave)
+    return best
+
+
+def bench_gather(args):
+    """The gather ceiling next to the kernel: for each width the bare gathers of the pattern (no rows, no FMAs, one
+    store per lane and wavefront) and the SpMM in the decider's configuration; GB/s of gathered bytes (nnz * N * 4)."""
+    import torch
+
+    from paramspmm_ae_amd import _capi, synth, sweep
+    from paramspmm_ae_amd.decider import SpMMDecider
+    from paramspmm_ae_amd.graph_input import graph_input
+
+    dims = [int(d) for d in args.dims.split(",")] if args.dims != DEFAULT_DIMS else [16, 64, 128]
+    rowPtr, colIdx, val, n = synth.config_graph(args.graph)
+    graph = graph_input(args.graph, "")
+    graph.verbose = False
+    graph.load_from_csr(rowPtr, colIdx, val)
+    nnz = graph.mtx_edges
+    ops = sweep.operators_of(graph)
+    dec = SpMMDecider()
+    dec.gen_model_dict(dims)
+    rows = (n + 1) // 2 * 2
+    ci = ops[0].colIdx
+    table = []
+    for d in dims:
+        X = torch.randn(rows, d, device="cuda", generator=torch.Generator(device="cuda").manual_seed(d))
+        if_split, vec, cf, bw = (int(v) for v in dec.config_PCSR(graph, d))
+        op = ops[(1 if if_split else 0) + (2 if vec == 2 else 0)]
+        k_ms = op.time_ms(X, CF=cf, blkWarpNum=bw, warmup=3, iters=10)
+        plan = _capi.spmm_plan(d, cf, bw)
+        row = {"dim": d, "kernel_ms": round(k_ms, 5), "pick": [if_split, vec, sweep.cf_label(cf), bw], "probes": {}}
+        gathered = 4.0 * nnz * d
+        for lanes in sorted({plan["lanes_per_row"], min(8, d // 4), min(32, d // 4)}):
+            ms, unroll, per_wave = gather_probe_ms(ci, nnz, X, lanes)
+            row["probes"]["lanes%d" % lanes] = {"ms": round(ms, 5), "unroll": unroll, "entries_per_wave": per_wave,
+                                                "gathered_GBps": round(gathered / ms / 1e6, 1)}
+        best = min(v["ms"] for v in row["probes"].values())
+        row["kernel_gathered_GBps"] = round(gathered / k_ms / 1e6, 1)
+        row["gather_ceiling_frac"] = round(best / k_ms, 4)
+        table.append(row)
+    print(json.dumps({"metric": "gather ceiling: bare gathers of the pattern vs the SpMM kernel", "unit": "ratio",
+                      "value": table[-1]["gather_ceiling_frac"], "n_gpus": 1, "steps": 10, "warmup": 3,
+                      "ms_per_step": table[-1]["kernel_ms"], "higher_is_better": True, "scaling": "weak",
+                      "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": "%s gather ceiling" % args.graph, "nodes": n, "nnz": nnz}, "per_dim": table}))
 
 
 def bench_agnn(args):
@@ -354,7 +436,7 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--graph", default="C2", help="C1, C2, C3, C3s, C5, C5p (synth.config_graph)")
-    ap.add_argument("--dims", default=",".join(str(d) for d in range(16, 257, 16)))
+    ap.add_argument("--dims", default=DEFAULT_DIMS)
     ap.add_argument("--pick", default="auto",
                     help="auto (decider if its forests are built, else sweep) | sweep | decider | "
                          "fixed:<csr|csr_split|bcsr|bcsr_split>:<CF>:<blkWarpNum>")
@@ -363,7 +445,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-vendor", action="store_true", help="skip the rocSPARSE comparison leg")
     ap.add_argument("--dump", default=None, help="write the full sweep table (every column, every width) as JSON")
-    ap.add_argument("--workload", choices=["spmm", "agnn", "gcn", "build", "sddmm"], default="spmm",
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip what follows the timed region: decider check, gather ceiling, SDDMM and GCN legs")
+    ap.add_argument("--workload", choices=["spmm", "agnn", "gcn", "build", "sddmm", "gather"], default="spmm",
                     help="spmm: the headline width sweep; agnn: SDDMM -> row softmax -> SpMM attention layers; "
                          "gcn: GCN / GIN training epochs on the SBM graph; build: PCSR construction, host against device; "
                          "sddmm: SDDMM width sweep over the four formats")
@@ -386,6 +470,8 @@ def main():
         return bench_build(args)
     if args.workload == "sddmm":
         return bench_sddmm(args)
+    if args.workload == "gather":
+        return bench_gather(args)
     from paramspmm_ae_amd import _capi, synth, sweep
     from paramspmm_ae_amd.graph_input import graph_input
 
@@ -428,6 +514,10 @@ def main():
     fixed = None
     if pick.startswith("fixed:"):
         _, f_fmt, f_cf, f_bw = pick.split(":")
+        if "." in f_cf:  # native configuration: vectors.lanes.unroll.segments_per_wave[.e]  (0 segments = automatic)
+            parts = f_cf.split(".")
+            c_, l_, u_, w_ = (int(v) for v in parts[:4])
+            f_cf = _capi.pack_cf(c_, l_, u_, w_ or None, even_split=parts[-1] == "e")
         fixed = (int("split" in f_fmt), 2 if f_fmt.startswith("bcsr") else 1, int(f_cf), int(f_bw))
     for d in dims:
         if pick == "sweep" or args.dump:
@@ -502,7 +592,7 @@ def main():
         # no-reuse gather volume: every stored entry fetches its row of X (what a matrix without locality moves)
         stored = F["nblk"] if fmt.startswith("bcsr") else nnz
         b_gather = b_alg - 4 * n * d + 4 * stored * d
-        per_dim.append({"dim": d, "format": fmt, "CF": cf, "blkWarpNum": bw, "ms": round(ms, 5),
+        per_dim.append({"dim": d, "format": fmt, "CF": cf, "config": sweep.cf_label(cf), "blkWarpNum": bw, "ms": round(ms, 5),
                         "gflops": round(2.0 * nnz * d / (ms * 1e-3) / 1e9, 1), "alg_bytes": b_alg,
                         "alg_GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
                         "gather_bytes": int(b_gather),
@@ -541,6 +631,75 @@ def main():
         "sweep": per_dim,
     }
 
+    if not args.no_extras:
+        # ---- gather ceiling of the dominant width: the bare gathers of the same pattern and X row tiles ----------
+        dom = max(rows_of, key=lambda r: r["ms"])
+        plan = _capi.spmm_plan(dom["dim"], dom["CF"], dom["blkWarpNum"])
+        dom_op = ops[fmt_names.index(dom["format"])]
+        stored = dom_op.colIdx.numel()
+        probe_ms, probe_unroll, probe_per_wave = gather_probe_ms(dom_op.colIdx, stored, Xs[dom["dim"]], plan["lanes_per_row"])
+        roofline["gather_ceiling"] = {"dim": dom["dim"], "probe_ms": round(probe_ms, 5), "kernel_ms": dom["ms"],
+                                      "probe_gathered_GBps": round(4.0 * stored * dom["dim"] / probe_ms / 1e6, 1),
+                                      "lanes_per_row": plan["lanes_per_row"], "unroll": probe_unroll,
+                                      "entries_per_wave": probe_per_wave}
+        roofline["gather_ceiling_frac"] = round(probe_ms / dom["ms"], 4)
+
+        # ---- the decider's pick against the best swept configuration, per width --------------------------------
+        if pick == "decider":
+            checks = []
+            for d in dims:
+                ms_all, _ = sweep.sweep_dim(ops, d, nnz, n, warmup=1, iters=3, X=Xs[d])
+                names = sweep.column_names(d)
+                if_split, vec, cf, bw = chosen[d]
+                col = [c for c in range(len(names)) if sweep.decode_column(d, c) == (if_split, vec, cf, bw)][0]
+                best = int(np.argmin(ms_all))
+                checks.append({"dim": d, "pick": names[col], "best": names[best], "t_pick_over_t_best": round(float(ms_all[col] / ms_all[best]), 3),
+                               "ms_pick": round(float(ms_all[col]), 5), "ms_best": round(float(ms_all[best]), 5)})
+            ratios = np.array([c["t_pick_over_t_best"] for c in checks])
+            out["decider_vs_best"] = {"per_dim": checks, "share_within_10pct": round(float(np.mean(ratios <= 1.10)), 3),
+                                      "mean_normalised_performance": round(float(np.mean(1.0 / ratios)), 4),
+                                      "worst_t_pick_over_t_best": round(float(ratios.max()), 3),
+                                      "columns_swept": int(sum(len(sweep.column_names(d)) for d in dims))}
+
+        # ---- SDDMM at K = 64 on the same pattern ----------------------------------------------------------------
+        import ParamSDDMM
+
+        K = 64
+        A = torch.randn(rows, K, device="cuda", generator=gen)
+        Bm = torch.randn(rows, K, device="cuda", generator=gen)
+        c_, b_ = ops[0], ops[2]
+        cs_, bs_ = ops[1], ops[3]
+        sd = {}
+        for bw in (4, 8):
+            sd[("csr", bw)] = lambda bw=bw: ParamSDDMM.csr_sddmm(A, Bm, c_.rowPtr, c_.colIdx, c_.val, 2, bw)
+            sd[("csr_split", bw)] = lambda bw=bw: ParamSDDMM.csr_split_sddmm(A, Bm, cs_.rowPtr, cs_.colIdx, cs_.val, cs_.target_row, 2, bw)
+            sd[("bcsr", bw)] = lambda bw=bw: ParamSDDMM.bcsr_sddmm(A, Bm, b_.rowPtr, b_.colIdx, b_.val, 2, bw)
+            sd[("bcsr_split", bw)] = lambda bw=bw: ParamSDDMM.bcsr_split_sddmm(A, Bm, bs_.rowPtr, bs_.colIdx, bs_.val, bs_.target_row, 2, bw)
+        sd_ms = {}
+        for key, fn in sd.items():
+            fn()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(5):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            sd_ms[key] = e0.elapsed_time(e1) / 5
+        (sfmt, sbw), sms = min(sd_ms.items(), key=lambda kv: kv[1])
+        if sfmt.startswith("bcsr"):
+            salg = 4 * (F["Sb"] + 1 if "split" in sfmt else F["Mb"] + 1) + 12 * F["nblk"] + 8 * n * K + 8 * F["nblk"]
+            salg += 4 * F["Sb"] if "split" in sfmt else 0
+        else:
+            salg = 4 * (F["S"] + 1 if "split" in sfmt else n + 1) + 4 * nnz + 8 * n * K + 4 * nnz
+            salg += 4 * F["S"] if "split" in sfmt else 0
+        out["sddmm"] = {"K": K, "format": sfmt, "blkWarpNum": sbw, "ms": round(sms, 5), "gflops": round(2.0 * nnz * K / sms / 1e6, 1),
+                        "all_ms": {"%s/%d" % k: round(v, 5) for k, v in sd_ms.items()},
+                        "roofline": {"bound": "hbm", "achieved": round(salg / sms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                     "frac": round(salg / sms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None,
+                                     "kernel": "psp_sddmm_kernel, K = 64, %s, %d wavefronts per workgroup" % (sfmt, sbw),
+                                     "alg_bytes_per_launch": int(salg), "ms_per_launch": round(sms, 5)}}
+        del A, Bm
+
     if not args.no_vendor:
         # vendor library beside it: rocSPARSE CSR SpMM (default algorithm), the counterpart of the cuSPARSE baseline
         # the reference quotes its speed-ups against (SpMM/Baseline_kernel.cu:24-169)
@@ -558,28 +717,12 @@ def main():
                                   "mean_speedup": round(float(np.mean(speedups)), 2)}
 
     if not args.no_cpu:
-        # cpu_baseline: the C restatement of the reference's CSR kernel (oracle/paramsp_oracle.c, one scalar thread) on a
-        # bounded sample of the sweep's widths; it doubles as the checker of the GPU result at those widths
-        from oracle import oracle as orc
-
-        rp_h, ci_h, v_h = (graph.csr_data.rowPtr.numpy(), graph.csr_data.colIdx.numpy(), graph.csr_data.val.numpy())
-        sample_dims = [d for d in (16, 64, 128) if d in dims] or dims[:1]
-        flops, secs, err = 0.0, 0.0, 0.0
-        for d in sample_dims:
-            Xc = Xs[d][:n].cpu().numpy()
-            t1 = time.perf_counter()
-            yo = orc.spmm_csr(rp_h, ci_h, v_h, Xc)
-            secs += time.perf_counter() - t1
-            flops += 2.0 * nnz * d
-            err = max(err, float(np.abs(Ys[d][:n].cpu().numpy() - yo).max()))
-        out["cpu_baseline"] = {"value": round(flops / secs / 1e9, 3), "unit": "GFLOP/s", "cores": 1, "kind": "port",
-                               "sample": "oracle orc_spmm_csr (scalar C, fp32 FMA chain per row) on the same graph, widths %s, one pass each (%.1f s); max |gpu-oracle| = %.2e"
-                                         % (sample_dims, secs, err)}
-        # beside it, the product the reference itself checks against on the host: torch.sparse.mm of the CSR tensor
-        # (verification.py:18-46), all host threads
+        # cpu_baseline: the product the reference itself checks against on the host, torch.sparse.mm of the CSR tensor
+        # (verification.py:18-46), on all host threads, on a bounded sample of the widths
         s = torch.sparse_csr_tensor(graph.csr_data.rowPtr, graph.csr_data.colIdx, graph.csr_data.val, size=(n, n))
-        flops, secs = 0.0, 0.0
-        for d in [d for d in (16, 64, 128) if d in dims] or dims[:1]:
+        sample_dims = [d for d in (16, 64, 128) if d in dims] or dims[:1]
+        flops, secs, total_reps = 0.0, 0.0, 0
+        for d in sample_dims:
             Xc = Xs[d][:n].cpu()
             torch.sparse.mm(s, Xc)  # warm-up
             reps = 0
@@ -589,7 +732,44 @@ def main():
                 reps += 1
             secs += time.perf_counter() - t1
             flops += 2.0 * nnz * d * reps
-        out["cpu_torch_sparse_mm"] = {"value": round(flops / secs / 1e9, 2), "unit": "GFLOP/s", "cores": torch.get_num_threads()}
+            total_reps += reps
+        out["cpu_baseline"] = {"value": round(flops / secs / 1e9, 2), "unit": "GFLOP/s", "cores": torch.get_num_threads(),
+                               "kind": "reference",
+                               "sample": "torch.sparse.mm(torch.sparse_csr_tensor(A), X) on the host, the product the reference verifies "
+                                         "against (verification.py:18-46), same graph, widths %s, %d products in %.1f s"
+                                         % (sample_dims, total_reps, secs)}
+        # beside it the C restatement of the reference's CSR kernel (oracle/paramsp_oracle.c, one scalar thread); it
+        # doubles as the checker of the GPU result at those widths
+        from oracle import oracle as orc
+
+        rp_h, ci_h, v_h = (graph.csr_data.rowPtr.numpy(), graph.csr_data.colIdx.numpy(), graph.csr_data.val.numpy())
+        port_dims = [d for d in (16, 64) if d in dims] or dims[:1]
+        flops, secs, err = 0.0, 0.0, 0.0
+        for d in port_dims:
+            Xc = Xs[d][:n].cpu().numpy()
+            t1 = time.perf_counter()
+            yo = orc.spmm_csr(rp_h, ci_h, v_h, Xc)
+            secs += time.perf_counter() - t1
+            flops += 2.0 * nnz * d
+            err = max(err, float(np.abs(Ys[d][:n].cpu().numpy() - yo).max()))
+        out["cpu_scalar_port"] = {"value": round(flops / secs / 1e9, 3), "unit": "GFLOP/s", "cores": 1, "kind": "port",
+                                  "sample": "oracle orc_spmm_csr (scalar C, fp32 FMA chain per row), widths %s, one pass each (%.1f s)" % (port_dims, secs),
+                                  "max_abs_gpu_minus_oracle": err}
+
+    if not args.no_extras and args.graph == "C2":
+        # ---- GCN training epochs on the 1M-node block model (the metric's second half) ------------------------------
+        for d in list(Xs):
+            del Xs[d], Ys[d]
+        torch.cuda.empty_cache()
+        from paramspmm_ae_amd import GNN
+
+        with contextlib.redirect_stdout(sys.stderr):
+            res = GNN.main(["--net", "GCN", "--synthetic", "C5", "--hidden_list", "16", "--num_classes", "16",
+                            "--num_features", "32", "--num_epoches", "20"])
+        out["gcn_epoch_ms"] = {"value": round(float(list(res.values())[0]), 3), "unit": "ms per epoch", "epochs": 20,
+                               "config": "GCN, 5 layers, hidden 16, 16 classes, 32 features, fwd+bwd+Adam, SBM 1M nodes "
+                                         "(community order), decider-picked operators"}
+
     print(json.dumps(out))
 
 

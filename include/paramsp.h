@@ -67,7 +67,7 @@ int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan);
  *   "xcd_stripe_rows"  rows (segments) dealt to one XCD at a time by the SpMM kernels (default 8192),
  *   "align_pct"        lane groups take whole segments when that costs at most this many percent more steps than
  *                      the even division of a wavefront's entries (default 50),
- *   "split_clear_min"  row-split outputs of at least this many floats are cleared selectively (default 32 Mi).
+ *   "split_clear_min"  row-split outputs of at least this many floats are cleared selectively (default 4 Mi).
  * The environment (PSP_XCD_STRIPE_ROWS, PSP_ALIGN_PCT, PSP_SPLIT_CLEAR_MIN) sets the initial values, once.
  * psp_get_option returns the value, or a negative psp_status for an unknown name.  Not synchronised with running
  * launches: set options before the calls they should affect. */
@@ -333,6 +333,18 @@ int psp_sddmm_f64(const int *rowPtr, const int *colIdx, const double *val_b, con
  * ------------------------------------------------------------------------------------------- */
 int psp_baseline_rowcache_spmm_f32(const int *rowPtr, const int *colIdx, const float *val, const float *X,
                                    float *Y, int M, int N, psp_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * DEVICE: measurement aid, no counterpart in the reference.  The gathers of an SpMM without the SpMM: for every
+ * stored entry and every column tile (lanes_per_row lanes x float4) the X row tile is loaded and added up per
+ * lane; there is no row structure, no multiplication and one 16-byte store per lane and wavefront.  Its duration
+ * is the floor the memory system sets for any SpMM on the pattern (bench.py reports the kernel's time against it).
+ * entries_per_wave: stored entries one wavefront walks (a multiple of 64); unroll: loads in flight per lane
+ * (1, 2, 4, 8).  out: psp_probe_gather_out_floats(...) floats of device memory, overwritten.
+ * ------------------------------------------------------------------------------------------- */
+long long psp_probe_gather_out_floats(long long nnz, int N, int lanes_per_row, int entries_per_wave);
+int psp_probe_gather_f32(const int *colIdx, long long nnz, const float *X, int N, int lanes_per_row, int unroll,
+                         int entries_per_wave, float *out, long long out_floats, psp_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -82,6 +82,8 @@ SIGNATURES = {
     "psp_baseline_rowcache_spmm_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
     "psp_nll_loss_mean_f32": [_vp, _vp, ctypes.c_longlong, _i, _vp, _vp, _vp],
     "psp_nll_loss_mean_backward_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _vp, _vp],
+    "psp_probe_gather_out_floats": [ctypes.c_longlong, _i, _i, _i],
+    "psp_probe_gather_f32": [_vp, ctypes.c_longlong, _vp, _i, _i, _i, _i, _vp, ctypes.c_longlong, _vp],
     "psp_gemm_xw_supported": [_i, _i],
     "psp_gemm_xw_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _i, _vp],
     "psp_gemm_atb_supported": [_i, _i],
@@ -90,7 +92,8 @@ SIGNATURES = {
     "psp_gemm_atb_ws_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _vp, ctypes.c_longlong, _vp],
 }
 # the entries that do not return int
-RESTYPES = {"psp_gemm_atb_workspace_floats": ctypes.c_longlong, "psp_get_option": ctypes.c_longlong}
+RESTYPES = {"psp_gemm_atb_workspace_floats": ctypes.c_longlong, "psp_get_option": ctypes.c_longlong,
+            "psp_probe_gather_out_floats": ctypes.c_longlong}
 
 for _name, _args in SIGNATURES.items():
     _fn = getattr(lib, _name)

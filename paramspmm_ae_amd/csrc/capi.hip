@@ -32,7 +32,7 @@ psp_options &psp_opts(void)
         psp_options d;
         d.stripe_rows = 8192;
         d.align_pct = 50;
-        d.split_clear_min = (long long)32 << 20;
+        d.split_clear_min = (long long)4 << 20;
         if (const char *e = getenv("PSP_XCD_STRIPE_ROWS")) {
             if (atoi(e) > 0) d.stripe_rows = atoi(e);
         }

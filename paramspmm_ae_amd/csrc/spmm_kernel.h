@@ -12,8 +12,9 @@
 //   * every lane owns C column vectors of V floats (V = 4 -> global_load_dwordx4); vector i of lane s
 //     covers columns tile*L*C*V + (i*L + s)*V .. +V, so the L lanes of a group read L*V*4 contiguous bytes
 //     of an X row per load;
-//   * colIdx / values are read once per L entries, coalesced (lane s takes entry base+s), and handed
-//     round the group with ds_bpermute; the next L are prefetched while the current ones are consumed;
+//   * colIdx / values are read once per L*U entries: lane s of a group takes the U consecutive entries
+//     base + s*U .. in one 4U-byte load per array (a group reads whole 128-byte lines), the pairs are handed
+//     round the group with ds_bpermute, and the next L*U are prefetched while the current ones are consumed;
 //   * the walk is software-pipelined over batches of U entries, whatever rows they belong to: the U*C
 //     feature loads of batch t+1 are issued before batch t is added (two register sets alternate), so every
 //     lane group issues the same loads at the same time and only the closing of a row -- a store where a row
@@ -48,6 +49,27 @@ template <int V> __device__ __forceinline__ void psp_store_vec(float *p, const f
     // Y is written once and not read again by this kernel: the streaming hint keeps it from displacing rows of X
     // in the L2 (measured 1-5 % faster; the same hint on colIdx / val loads is slower, other column tiles re-read them)
     __builtin_nontemporal_store(t, (typename psp_vec<V>::type *)p);
+}
+
+// COUNT consecutive 4-byte words starting at a 4-byte aligned address, fetched in the widest pieces (16, 8, 4 bytes)
+typedef int psp_i32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+typedef int psp_i32x2_a4 __attribute__((ext_vector_type(2), aligned(4)));
+template <int COUNT> __device__ __forceinline__ void psp_load_words(const int *p, int (&out)[COUNT])
+{
+    int done = 0;
+#pragma unroll
+    for (; done + 4 <= COUNT; done += 4) {
+        const psp_i32x4_a4 t = *(const psp_i32x4_a4 *)(p + done);
+#pragma unroll
+        for (int e = 0; e < 4; e++) out[done + e] = t[e];
+    }
+    if constexpr ((COUNT & 2) != 0) {
+        const psp_i32x2_a4 t = *(const psp_i32x2_a4 *)(p + done);
+        out[done] = t[0];
+        out[done + 1] = t[1];
+        done += 2;
+    }
+    if constexpr ((COUNT & 1) != 0) out[done] = p[done];
 }
 
 __device__ __forceinline__ int psp_bperm_i(int src_lane, int v) { return __builtin_amdgcn_ds_bpermute(src_lane << 2, v); }
@@ -252,33 +274,42 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         }
     }
 
-    // lane `sub` of the group picks up entry base+sub; past the end of the range: (last column, 0)
-#define PSP_FETCH(base, c_out, v_out)                                      \
-    {                                                                      \
-        const int p_ = (base) + sub;                                       \
-        const bool ok_ = p_ < b;                                           \
-        const int pp_ = ok_ ? p_ : b - 1;                                  \
-        c_out = colIdx[pp_];                                               \
-        if constexpr (NR == 2) {                                           \
-            const psp_f32x2 t_ = ((const psp_f32x2 *)val)[pp_];            \
-            v_out[0] = ok_ ? t_[0] : 0.0f;                                 \
-            v_out[1] = ok_ ? t_[1] : 0.0f;                                 \
-        } else if constexpr (NR > 2) {                                     \
-            _Pragma("unroll") for (int r_ = 0; r_ < NR; r_++)              \
-            {                                                              \
-                const float t_ = val[(size_t)pp_ * NR + r_];               \
-                v_out[r_] = ok_ ? t_ : 0.0f;                               \
-            }                                                              \
-        } else {                                                           \
-            const float t_ = val[pp_];                                     \
-            v_out[0] = ok_ ? t_ : 0.0f;                                    \
-        }                                                                  \
+    // Lane `sub` of the group picks up the U consecutive entries base + sub*U ..: one 4U-byte load of column
+    // indices and one of 4U*NR bytes of values, so a group reads L*U*4 contiguous bytes of each array at a time
+    // (whole 128-byte lines for 8 lanes x 4 entries).  Entries past the end of the range: (last column, 0), taken
+    // one by one so that nothing past the arrays is touched.
+#define PSP_FETCH(base, c_out, v_out)                                                        \
+    {                                                                                        \
+        const int p0_ = (base) + sub * U;                                                    \
+        if (p0_ + U <= b) {                                                                  \
+            psp_load_words<U>(colIdx + p0_, c_out);                                          \
+            int w_[U * NR];                                                                  \
+            psp_load_words<U * NR>((const int *)val + (size_t)p0_ * NR, w_);                 \
+            _Pragma("unroll") for (int u_ = 0; u_ < U; u_++)                                 \
+                _Pragma("unroll") for (int r_ = 0; r_ < NR; r_++) v_out[u_][r_] = __int_as_float(w_[u_ * NR + r_]); \
+        } else {                                                                             \
+            _Pragma("unroll") for (int u_ = 0; u_ < U; u_++)                                 \
+            {                                                                                \
+                const bool ok_ = p0_ + u_ < b;                                               \
+                const int pp_ = ok_ ? p0_ + u_ : b - 1;                                      \
+                c_out[u_] = colIdx[pp_];                                                     \
+                _Pragma("unroll") for (int r_ = 0; r_ < NR; r_++)                            \
+                {                                                                            \
+                    const float t_ = val[(size_t)pp_ * NR + r_];                             \
+                    v_out[u_][r_] = ok_ ? t_ : 0.0f;                                         \
+                }                                                                            \
+            }                                                                                \
+        }                                                                                    \
     }
 
-    int c_cur = 0;
-    float v_cur[NR];
+    int c_cur[U], c_nxt[U];
+    float v_cur[U][NR], v_nxt[U][NR];
 #pragma unroll
-    for (int r = 0; r < NR; r++) v_cur[r] = 0.0f;
+    for (int u = 0; u < U; u++) {
+        c_cur[u] = c_nxt[u] = 0;
+#pragma unroll
+        for (int r = 0; r < NR; r++) v_cur[u][r] = v_nxt[u][r] = 0.0f;
+    }
     if (busy) PSP_FETCH(a, c_cur, v_cur);
 
     // The entry just added closed its segment and the group's range goes on: move to the next filled segment
@@ -321,12 +352,10 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     // part diverges between groups.  Entries past the group's range (last, partial batch) are loaded from a valid
     // address but never added, so values of other rows cannot leak in.
     int pos = a;      // first entry of the next batch to gather
-    int cbase = a;    // first entry of the chunk c_cur / v_cur hold (lane `sub` holds entry cbase + sub)
-    int c_nxt = 0;
-    float v_nxt[NR];
-#pragma unroll
-    for (int r = 0; r < NR; r++) v_nxt[r] = 0.0f;
-    if (busy && a + L < b) PSP_FETCH(a + L, c_nxt, v_nxt);
+    int cbase = a;    // first entry of the chunk c_cur / v_cur hold (lane `sub` holds entries cbase + sub*U ..)
+    int jb = 0;       // batch of that chunk the next gather takes: the one lane `jb` of the group holds
+    const int chunk = L * U;
+    if (busy && a + chunk < b) PSP_FETCH(a + chunk, c_nxt, v_nxt);
 
 #define PSP_DECLARE(S)      \
     int S##_ck[U], S##_pos; \
@@ -334,20 +363,22 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     vec_t S##_x[U][C];
 #define PSP_GATHER(S)                                                                                  \
     {                                                                                                  \
-        int k_ = pos - cbase;                                                                          \
-        if (k_ == L) { /* the chunk is used up: the prefetched one becomes current, the next is requested */ \
-            c_cur = c_nxt;                                                                             \
-            _Pragma("unroll") for (int r = 0; r < NR; r++) v_cur[r] = v_nxt[r];                        \
-            cbase += L;                                                                                \
-            if (cbase + L < b) PSP_FETCH(cbase + L, c_nxt, v_nxt);                                     \
-            k_ = 0;                                                                                    \
+        if (jb == L) { /* the chunk is used up: the prefetched one becomes current, the next is requested */ \
+            _Pragma("unroll") for (int u = 0; u < U; u++)                                              \
+            {                                                                                          \
+                c_cur[u] = c_nxt[u];                                                                   \
+                _Pragma("unroll") for (int r = 0; r < NR; r++) v_cur[u][r] = v_nxt[u][r];              \
+            }                                                                                          \
+            cbase += chunk;                                                                            \
+            if (cbase + chunk < b) PSP_FETCH(cbase + chunk, c_nxt, v_nxt);                             \
+            jb = 0;                                                                                    \
         }                                                                                              \
         S##_pos = pos;                                                                                 \
+        const int src = grp_base + jb;                                                                 \
         _Pragma("unroll") for (int u = 0; u < U; u++)                                                  \
         {                                                                                              \
-            const int src = grp_base + min(k_ + u, L - 1);                                             \
-            S##_ck[u] = psp_bperm_i(src, c_cur);                                                       \
-            _Pragma("unroll") for (int r = 0; r < NR; r++) S##_vk[u][r] = psp_bperm_f(src, v_cur[r]);  \
+            S##_ck[u] = psp_bperm_i(src, c_cur[u]);                                                    \
+            _Pragma("unroll") for (int r = 0; r < NR; r++) S##_vk[u][r] = psp_bperm_f(src, v_cur[u][r]); \
         }                                                                                              \
         _Pragma("unroll") for (int u = 0; u < U; u++)                                                  \
         {                                                                                              \
@@ -355,6 +386,7 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
             _Pragma("unroll") for (int i = 0; i < C; i++) S##_x[u][i] = *(const vec_t *)(xr + off[i]); \
         }                                                                                              \
         pos += U;                                                                                      \
+        jb++;                                                                                          \
     }
 #define PSP_CONSUME(S)                                                                                 \
     {                                                                                                  \
