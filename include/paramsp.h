@@ -292,6 +292,10 @@ int psp_gemm_atb_f32(const float *A, const float *B, float *C, long long n, int 
 long long psp_gemm_atb_workspace_floats(long long n, int K1, int K2);
 int psp_gemm_atb_ws_f32(const float *A, const float *B, float *C, long long n, int K1, int K2, float *workspace,
                         long long workspace_floats, psp_stream_t stream);
+/* relu_a != 0: A enters the product as max(a, 0): the weight gradient of a layer that reads the previous layer's
+ * output through a ReLU (GNN.py:43-61 applies F.relu between the layers) without that activation being stored. */
+int psp_gemm_atb_ws_act_f32(const float *A, const float *B, float *C, long long n, int K1, int K2, int relu_a,
+                            float *workspace, long long workspace_floats, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: Y[n,K2] = X[n,K1] * W (transW = 0, W is [K1,K2] row-major) or X * W^T (transW != 0, W is [K2,K1]) for
@@ -302,6 +306,13 @@ int psp_gemm_atb_ws_f32(const float *A, const float *B, float *C, long long n, i
 int psp_gemm_xw_supported(int K1, int K2);
 int psp_gemm_xw_f32(const float *X, const float *W, float *Y, long long n, int K1, int K2, int transW,
                     psp_stream_t stream);
+/* The same products with the ReLU between two GCN layers (F.relu in GNN.py:43-61) folded in, so that neither the
+ * activation nor its backward is a pass of its own:
+ *   relu_x != 0 (transW == 0 only): Y = max(X, 0) * W -- the layer reads the previous layer's output through the ReLU;
+ *   mask != NULL (transW != 0 only): Y = (X * W^T) where mask > 0, else 0; mask is [n, K2] -- the gradient with respect
+ *   to the pre-activation values the layer was given. */
+int psp_gemm_xw_act_f32(const float *X, const float *W, float *Y, long long n, int K1, int K2, int transW, int relu_x,
+                        const float *mask, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: mean negative log-likelihood, the loss of the reference's training step (F.nll_loss(model(), labels),

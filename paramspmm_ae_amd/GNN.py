@@ -33,12 +33,19 @@ class Net_5layers(torch.nn.Module):
         self.conv1, self.conv2, self.conv3, self.conv4, self.conv5 = (
             GCNConv(widths[i], widths[i + 1]) for i in range(5)
         )
+        self.fuse_relu = True  # False: F.relu between the layers as separate passes, as the reference's driver does
 
     def forward(self):
-        x = self.x
-        for conv in (self.conv1, self.conv2, self.conv3, self.conv4):
-            x = F.relu(conv(x, self.spmm_dict))
-        return F.log_softmax(self.conv5(x, self.spmm_dict), dim=1)
+        if not self.fuse_relu:
+            x = self.x
+            for conv in (self.conv1, self.conv2, self.conv3, self.conv4):
+                x = F.relu(conv(x, self.spmm_dict))
+            return F.log_softmax(self.conv5(x, self.spmm_dict), dim=1)
+        # the same network with every ReLU applied by the layer that reads it (no activation passes)
+        z = self.conv1(self.x, self.spmm_dict)
+        for conv in (self.conv2, self.conv3, self.conv4, self.conv5):
+            z = conv(z, self.spmm_dict, relu_input=True)
+        return F.log_softmax(z, dim=1)
 
 
 class GIN(torch.nn.Module):
@@ -218,6 +225,8 @@ def main(argv=None):
     p.add_argument("--synthetic", type=str, default=None, help="C1, C2, C3, C3s, C5 or C5p instead of a .mtx file")
     p.add_argument("--hip_graph", action="store_true",
                    help="record the training step in a HIP graph and replay it per epoch (an addition of this build)")
+    p.add_argument("--no_fuse_relu", action="store_true",
+                   help="GCN: apply F.relu between the layers as passes of their own, as the reference's driver does")
     p.add_argument("--config", nargs=4, type=int, default=None, metavar=("IF_SPLIT", "VEC", "CF", "BW"),
                    help="skip the decider and use this configuration for every layer width")
     args = p.parse_args(argv)
@@ -247,6 +256,8 @@ def main(argv=None):
                                       None if args.config is None else tuple(args.config))
             print("SpMM-decider config time: {:.3f} (ms)".format((time.perf_counter() - t1) * 1e3))
             model = build_model(args.net, graph, ops, hidden, args.num_features, args.num_classes, args.num_layers)
+            if args.no_fuse_relu and hasattr(model, "fuse_relu"):
+                model.fuse_relu = False
             torch.cuda.synchronize()
             results[(name, hidden)] = train_profiling(model, graph.y, args.num_epoches, verbose=args.verbose == "True",
                                                      hip_graph=args.hip_graph)

@@ -86,6 +86,8 @@ SIGNATURES = {
     "psp_probe_gather_f32": [_vp, ctypes.c_longlong, _vp, _i, _i, _i, _i, _vp, ctypes.c_longlong, _vp],
     "psp_gemm_xw_supported": [_i, _i],
     "psp_gemm_xw_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _i, _vp],
+    "psp_gemm_xw_act_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _i, _i, _vp, _vp],
+    "psp_gemm_atb_ws_act_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _i, _vp, ctypes.c_longlong, _vp],
     "psp_gemm_atb_supported": [_i, _i],
     "psp_gemm_atb_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _i, _vp],
     "psp_gemm_atb_workspace_floats": [ctypes.c_longlong, _i, _i],

@@ -13,7 +13,9 @@
 #include "psp_common.h"
 #include "spmm_kernel.h"
 
-template <int K1, int K2>
+// RELU_A (both kernels): A enters the product as max(a, 0) -- the weight gradient of a layer whose input is the
+// activation of the previous layer's output, without that activation ever being stored.
+template <int K1, int K2, bool RELU_A>
 __global__ void __launch_bounds__(256)
 psp_atb_kernel(const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, long long n,
                long long rows_per_block)
@@ -38,6 +40,10 @@ psp_atb_kernel(const float *__restrict__ A, const float *__restrict__ B, float *
             const int r = v / (K1 / 4), c4 = v % (K1 / 4);
             psp_f32x4 x = {0.f, 0.f, 0.f, 0.f};
             if (base + r < r_end) x = *(const psp_f32x4 *)(A + (base + r) * K1 + c4 * 4);
+            if constexpr (RELU_A) {
+#pragma unroll
+                for (int e = 0; e < 4; e++) x[e] = x[e] < 0.0f ? 0.0f : x[e];
+            }
             *(psp_f32x4 *)&sA[r][c4 * 4] = x;
         }
         for (int v = t; v < ATB_ROWS * K2 / 4; v += 256) {
@@ -94,7 +100,7 @@ template <int V> __device__ __forceinline__ void psp_atb_load(const float *p, fl
 // column of a (sub)matrix that index i of tile m stands for
 template <int V> __device__ __forceinline__ int psp_atb_col(int m, int i) { return (m / V) * 16 * V + V * i + (m % V); }
 
-template <int K1, int K2, int JSPLIT>
+template <int K1, int K2, int JSPLIT, bool RELU_A>
 __global__ void __launch_bounds__(256)
 psp_atb_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, long long n,
                     float *__restrict__ partial)
@@ -125,6 +131,10 @@ psp_atb_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B, fl
             const long long row = (g + u) * 4 + kk;
 #pragma unroll
             for (int t = 0; t < RM / VA; t++) psp_atb_load<VA>(A + row * K1 + t * 16 * VA + VA * c, &fa[u][t * VA]);
+            if constexpr (RELU_A) {
+#pragma unroll
+                for (int m = 0; m < RM; m++) fa[u][m] = fa[u][m] < 0.0f ? 0.0f : fa[u][m];
+            }
 #pragma unroll
             for (int t = 0; t < RNW / VB; t++) psp_atb_load<VB>(B + row * K2 + col0 + t * 16 * VB + VB * c, &fb[u][t * VB]);
         }
@@ -172,7 +182,10 @@ psp_atb_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B, fl
         for (int u = 0; u < U; u++) {
             const long long row = (gt + u) * 4 + kk;
 #pragma unroll
-            for (int m = 0; m < RM; m++) a0[u][m] = row < n ? A[row * K1 + psp_atb_col<VA>(m, c)] : 0.f;
+            for (int m = 0; m < RM; m++) {
+                a0[u][m] = row < n ? A[row * K1 + psp_atb_col<VA>(m, c)] : 0.f;
+                if (RELU_A) a0[u][m] = a0[u][m] < 0.0f ? 0.0f : a0[u][m];
+            }
 #pragma unroll
             for (int q = 0; q < RNW; q++) b0[u][q] = row < n ? B[row * K2 + col0 + psp_atb_col<VB>(q, c)] : 0.f;
         }
@@ -246,10 +259,10 @@ psp_atb_reduce_kernel(const float *__restrict__ partial, float *__restrict__ C, 
 typedef void (*psp_atb_kernel_t)(const float *, const float *, float *, long long, long long);
 typedef void (*psp_atb_mfma_kernel_t)(const float *, const float *, float *, long long, float *);
 
-static psp_atb_kernel_t atb_lookup(int K1, int K2)
+static psp_atb_kernel_t atb_lookup(int K1, int K2, bool relu_a = false)
 {
 #define ATB_CASE(a, b) \
-    if (K1 == a && K2 == b) return psp_atb_kernel<a, b>;
+    if (K1 == a && K2 == b) return relu_a ? psp_atb_kernel<a, b, true> : psp_atb_kernel<a, b, false>;
 #define ATB_ROW(a) ATB_CASE(a, 16) ATB_CASE(a, 32) ATB_CASE(a, 48) ATB_CASE(a, 64) ATB_CASE(a, 80) ATB_CASE(a, 96) ATB_CASE(a, 112) ATB_CASE(a, 128)
     ATB_ROW(16) ATB_ROW(32) ATB_ROW(48) ATB_ROW(64) ATB_ROW(80) ATB_ROW(96) ATB_ROW(112) ATB_ROW(128)
 #undef ATB_ROW
@@ -258,11 +271,11 @@ static psp_atb_kernel_t atb_lookup(int K1, int K2)
 }
 
 // *jsplit receives the kernel's JSPLIT
-static psp_atb_mfma_kernel_t atb_mfma_lookup(int K1, int K2, int *jsplit)
+static psp_atb_mfma_kernel_t atb_mfma_lookup(int K1, int K2, int *jsplit, bool relu_a = false)
 {
     *jsplit = 1;
 #define ATB_MFMA(a, b) \
-    if (K1 == a && K2 == b) return psp_atb_mfma_kernel<a, b, 1>;
+    if (K1 == a && K2 == b) return relu_a ? psp_atb_mfma_kernel<a, b, 1, true> : psp_atb_mfma_kernel<a, b, 1, false>;
     ATB_MFMA(16, 16) ATB_MFMA(16, 32) ATB_MFMA(16, 48) ATB_MFMA(16, 64) ATB_MFMA(16, 80) ATB_MFMA(16, 96) ATB_MFMA(16, 112) ATB_MFMA(16, 128)
     ATB_MFMA(32, 16) ATB_MFMA(32, 32) ATB_MFMA(32, 48) ATB_MFMA(32, 64) ATB_MFMA(32, 80) ATB_MFMA(32, 96) ATB_MFMA(32, 112) ATB_MFMA(32, 128)
     ATB_MFMA(48, 16) ATB_MFMA(48, 32) ATB_MFMA(48, 48) ATB_MFMA(48, 64) ATB_MFMA(48, 80)
@@ -272,7 +285,7 @@ static psp_atb_mfma_kernel_t atb_mfma_lookup(int K1, int K2, int *jsplit)
 #undef ATB_MFMA
     *jsplit = 4;
 #define ATB_MFMA4(a, b) \
-    if (K1 == a && K2 == b) return psp_atb_mfma_kernel<a, b, 4>;
+    if (K1 == a && K2 == b) return relu_a ? psp_atb_mfma_kernel<a, b, 4, true> : psp_atb_mfma_kernel<a, b, 4, false>;
     ATB_MFMA4(64, 128) ATB_MFMA4(80, 64) ATB_MFMA4(96, 64) ATB_MFMA4(112, 64) ATB_MFMA4(128, 64)
     ATB_MFMA4(80, 128) ATB_MFMA4(96, 128) ATB_MFMA4(112, 128) ATB_MFMA4(128, 128)
 #undef ATB_MFMA4
@@ -291,19 +304,18 @@ static long long atb_mfma_grid(long long n, int jsplit, int E)
 
 PSP_EXPORT int psp_gemm_atb_supported(int K1, int K2) { return atb_lookup(K1, K2) != nullptr; }
 
-PSP_EXPORT int psp_gemm_atb_f32(const float *A, const float *B, float *C, long long n, int K1, int K2,
-                                psp_stream_t stream)
+static int atb_atomic(const float *A, const float *B, float *C, long long n, int K1, int K2, bool relu_a, hipStream_t stream)
 {
     PSP_REQUIRE(n >= 0 && K1 >= 1 && K2 >= 1, "gemm_atb: bad size");
-    psp_atb_kernel_t k = atb_lookup(K1, K2);
+    psp_atb_kernel_t k = atb_lookup(K1, K2, relu_a);
     PSP_REQUIRE(k != nullptr, "gemm_atb: K1 and K2 must be multiples of 16 up to 128 (got %d, %d)", K1, K2);
     PSP_REQUIRE(C != nullptr && (n == 0 || (A && B)), "gemm_atb: null pointer");
-    int rc = psp_zero_f32(C, (size_t)K1 * K2, (hipStream_t)stream);
+    int rc = psp_zero_f32(C, (size_t)K1 * K2, stream);
     if (rc != PSP_OK || n == 0) return rc;
     int jsplit = 1;
-    if (psp_atb_mfma_kernel_t km = atb_mfma_lookup(K1, K2, &jsplit)) {
+    if (psp_atb_mfma_kernel_t km = atb_mfma_lookup(K1, K2, &jsplit, relu_a)) {
         const long long wgs = atb_mfma_grid(n, jsplit, K1 * K2);
-        hipLaunchKernelGGL(km, dim3((unsigned)wgs), dim3(256), 0, (hipStream_t)stream, A, B, C, n, (float *)nullptr);
+        hipLaunchKernelGGL(km, dim3((unsigned)wgs), dim3(256), 0, stream, A, B, C, n, (float *)nullptr);
         return psp_check_launch("gemm_atb mfma kernel");
     }
     // about 8 workgroups per CU, each on a contiguous band of whole 64-row tiles
@@ -312,8 +324,14 @@ PSP_EXPORT int psp_gemm_atb_f32(const float *A, const float *B, float *C, long l
     if (blocks > 2048) blocks = 2048;
     long long rows_per_block = ((n + blocks - 1) / blocks + ATB_ROWS - 1) / ATB_ROWS * ATB_ROWS;
     blocks = (n + rows_per_block - 1) / rows_per_block;
-    hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, A, B, C, n, rows_per_block);
+    hipLaunchKernelGGL(k, dim3((unsigned)blocks), dim3(256), 0, stream, A, B, C, n, rows_per_block);
     return psp_check_launch("gemm_atb kernel");
+}
+
+PSP_EXPORT int psp_gemm_atb_f32(const float *A, const float *B, float *C, long long n, int K1, int K2,
+                                psp_stream_t stream)
+{
+    return atb_atomic(A, B, C, n, K1, K2, false, (hipStream_t)stream);
 }
 
 PSP_EXPORT long long psp_gemm_atb_workspace_floats(long long n, int K1, int K2)
@@ -323,12 +341,12 @@ PSP_EXPORT long long psp_gemm_atb_workspace_floats(long long n, int K1, int K2)
     return atb_mfma_grid(n, jsplit, K1 * K2) * K1 * K2;
 }
 
-PSP_EXPORT int psp_gemm_atb_ws_f32(const float *A, const float *B, float *C, long long n, int K1, int K2,
-                                   float *workspace, long long workspace_floats, psp_stream_t stream)
+PSP_EXPORT int psp_gemm_atb_ws_act_f32(const float *A, const float *B, float *C, long long n, int K1, int K2, int relu_a,
+                                       float *workspace, long long workspace_floats, psp_stream_t stream)
 {
     int jsplit = 1;
-    psp_atb_mfma_kernel_t km = atb_mfma_lookup(K1, K2, &jsplit);
-    if (!km || n <= 0) return psp_gemm_atb_f32(A, B, C, n, K1, K2, stream);  // shapes of the LDS-tiled kernel; n = 0
+    psp_atb_mfma_kernel_t km = atb_mfma_lookup(K1, K2, &jsplit, relu_a != 0);
+    if (!km || n <= 0) return atb_atomic(A, B, C, n, K1, K2, relu_a != 0, (hipStream_t)stream);  // shapes of the LDS-tiled kernel; n = 0
     PSP_REQUIRE(A && B && C, "gemm_atb_ws: null pointer");
     const long long wgs = atb_mfma_grid(n, jsplit, K1 * K2);
     PSP_REQUIRE(workspace && workspace_floats >= wgs * K1 * K2, "gemm_atb_ws: the workspace holds %lld floats, %lld needed",
@@ -340,4 +358,10 @@ PSP_EXPORT int psp_gemm_atb_ws_f32(const float *A, const float *B, float *C, lon
     hipLaunchKernelGGL(psp_atb_reduce_kernel, dim3((unsigned)((K1 * K2 + 15) / 16)), dim3(1024), 0, st, workspace, C, (int)wgs,
                        K1 * K2);
     return psp_check_launch("gemm_atb reduce kernel");
+}
+
+PSP_EXPORT int psp_gemm_atb_ws_f32(const float *A, const float *B, float *C, long long n, int K1, int K2,
+                                   float *workspace, long long workspace_floats, psp_stream_t stream)
+{
+    return psp_gemm_atb_ws_act_f32(A, B, C, n, K1, K2, 0, workspace, workspace_floats, stream);
 }

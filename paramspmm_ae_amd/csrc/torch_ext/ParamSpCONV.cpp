@@ -60,6 +60,75 @@ static Tensor dense_xw(const Tensor &X, const Tensor &W, bool transW)
     return Y;
 }
 
+// The same two products with the ReLU between two layers folded in (psp_gemm_xw_act_f32 / psp_gemm_atb_ws_act_f32);
+// shapes the library does not cover apply the activation with PyTorch and multiply with torch::mm.
+static Tensor dense_relu_xw(const Tensor &Z, const Tensor &W)
+{
+    const long K1 = Z.dim() == 2 ? Z.size(1) : -1;
+    const bool shapes = Z.dim() == 2 && W.dim() == 2 && W.size(0) == K1;
+    const bool narrow = shapes && Z.size(0) >= 16384 && Z.scalar_type() == torch::kFloat32 && W.scalar_type() == torch::kFloat32 &&
+                        psp_gemm_xw_supported((int)K1, (int)W.size(1));
+    if (!narrow) return torch::mm(torch::relu(Z), W);
+    Tensor Zc = Z.contiguous(), Wc = W.contiguous();
+    DeviceGuard guard(Zc.device());
+    Tensor Y = torch::empty({Zc.size(0), Wc.size(1)}, Zc.options());
+    ok(psp_gemm_xw_act_f32(fp(Zc), fp(Wc), fpw(Y), Zc.size(0), (int)K1, (int)Wc.size(1), 0, 1, nullptr, stream_of(Zc)));
+    return Y;
+}
+// (AG * W^T) where Z > 0, else 0
+static Tensor dense_xwt_masked(const Tensor &AG, const Tensor &W, const Tensor &Z)
+{
+    const long K1 = AG.dim() == 2 ? AG.size(1) : -1;
+    const bool shapes = AG.dim() == 2 && W.dim() == 2 && W.size(1) == K1 && Z.dim() == 2 && Z.size(0) == AG.size(0) &&
+                        Z.size(1) == W.size(0);
+    const bool narrow = shapes && AG.size(0) >= 16384 && AG.scalar_type() == torch::kFloat32 && W.scalar_type() == torch::kFloat32 &&
+                        Z.scalar_type() == torch::kFloat32 && psp_gemm_xw_supported((int)K1, (int)W.size(0));
+    if (!narrow) return at::threshold_backward(torch::mm(AG, W.t()), Z, 0);  // what F.relu's backward runs
+    Tensor Gc = AG.contiguous(), Wc = W.contiguous(), Zc = Z.contiguous();
+    DeviceGuard guard(Gc.device());
+    Tensor Y = torch::empty({Gc.size(0), Wc.size(0)}, Gc.options());
+    ok(psp_gemm_xw_act_f32(fp(Gc), fp(Wc), fpw(Y), Gc.size(0), (int)K1, (int)Wc.size(0), 1, 0, fp(Zc), stream_of(Gc)));
+    return Y;
+}
+// relu(Z)^T * AG
+static Tensor weight_gradient_relu(const Tensor &Z, const Tensor &AG)
+{
+    const bool narrow = Z.dim() == 2 && AG.dim() == 2 && Z.size(0) == AG.size(0) && Z.size(0) >= 16384 &&
+                        Z.scalar_type() == torch::kFloat32 && AG.scalar_type() == torch::kFloat32 &&
+                        psp_gemm_atb_supported((int)Z.size(1), (int)AG.size(1));
+    if (!narrow) return torch::mm(torch::relu(Z).t(), AG);
+    Tensor Zc = Z.contiguous(), Gc = AG.contiguous();
+    DeviceGuard guard(Zc.device());
+    Tensor dW = torch::empty({Zc.size(1), Gc.size(1)}, Zc.options());
+    const long long ws_floats = psp_gemm_atb_workspace_floats(Zc.size(0), (int)Zc.size(1), (int)Gc.size(1));
+    Tensor ws = torch::empty({(long)ws_floats}, Zc.options());
+    ok(psp_gemm_atb_ws_act_f32(fp(Zc), fp(Gc), fpw(dW), Zc.size(0), (int)Zc.size(1), (int)Gc.size(1), 1, fpw(ws), ws_floats,
+                               stream_of(Zc)));
+    return dW;
+}
+
+// GCN layer that reads its input through a ReLU: A * (relu(Z) * W).  fmt: 0 csr, 1 csr_split, 2 bcsr, 3 bcsr_split.
+// No counterpart among the reference's bindings: its driver applies F.relu between the layers as a pass of its own
+// (GNN.py:43-61); the algebra of the layer itself is SpCONV/SpCONV.h:43-71.
+static Tensor relu_input_forward(int fmt, Tensor Z, Tensor W, Tensor rowPtr, Tensor colIdx, Tensor values,
+                                 c10::optional<Tensor> target_row, int CF, int bw)
+{
+    need_gpu(Z, "input");
+    need_gpu(W, "weight");
+    TORCH_CHECK(fmt >= 0 && fmt <= 3 && ((fmt & 1) != 0) == target_row.has_value(), "format code and target_row disagree");
+    return aggregate(fmt, dense_relu_xw(Z, W), rowPtr, colIdx, values, target_row ? &*target_row : nullptr, CF, bw);
+}
+// [dZ, dW] = [ ((A dY) W^T) where Z > 0,  relu(Z)^T (A dY) ]
+static std::vector<Tensor> relu_input_backward(int fmt, Tensor dY, Tensor Z, Tensor W, Tensor rowPtr, Tensor colIdx,
+                                               Tensor values, c10::optional<Tensor> target_row, int CF, int bw)
+{
+    need_gpu(Z, "input");
+    need_gpu(W, "weight");
+    TORCH_CHECK(fmt >= 0 && fmt <= 3 && ((fmt & 1) != 0) == target_row.has_value(), "format code and target_row disagree");
+    Tensor AG = aggregate(fmt, dY, rowPtr, colIdx, values, target_row ? &*target_row : nullptr, CF, bw);
+    return {dense_xwt_masked(AG, W, Z), weight_gradient_relu(Z, AG)};
+}
+
 static Tensor forward_impl(int fmt, const Tensor &H, const Tensor &W, const Tensor &rowPtr, const Tensor &colIdx,
                            const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
 {
@@ -161,6 +230,10 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     }, "X * W (transW false) or X * W^T for tall-skinny X: (X, W, transW)");
     m.def("nll_loss_mean", &nll_loss_mean, "[loss, stats] of the mean negative log-likelihood (log-probabilities, int64 labels)");
     m.def("nll_loss_mean_backward", &nll_loss_mean_backward, "gradient w.r.t. the log-probabilities: (labels, grad_loss, stats, n, C)");
+    m.def("relu_input_forward", &relu_input_forward,
+          "A*(relu(Z)*W): (fmt 0..3, Z, W, rowPtr, colIdx, values, target_row or None, CF, blkWarpNum)");
+    m.def("relu_input_backward", &relu_input_backward,
+          "[dZ, dW] of relu_input_forward: (fmt, dY, Z, W, rowPtr, colIdx, values, target_row or None, CF, blkWarpNum)");
     m.def("csr_spmm_forward", &csr_spmm_forward, "A*(H*W), CSR");
     m.def("csr_spmm_backward", &csr_spmm_backward, "[dH, dW], CSR");
     m.def("csr_split_spmm_forward", &csr_split_spmm_forward, "A*(H*W), row-split CSR");

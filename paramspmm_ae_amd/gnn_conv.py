@@ -67,6 +67,31 @@ class GCNFunction(torch.autograd.Function):
         return d_input, d_weight, None
 
 
+class GCNReLUInputFunction(torch.autograd.Function):
+    """The GCN layer reading its input through a ReLU, A (relu(Z) W), as one function of the pre-activation values
+    Z: forward relu(Z) W with the activation applied as Z is read; backward dZ = ((A dY) W^T) where Z > 0 and
+    dW = relu(Z)^T (A dY), again without a pass for the activation.  Five layers with F.relu between them
+    (GNN.py:43-61) are conv1(x), then four of these."""
+
+    @staticmethod
+    def forward(ctx, Z, weight, ParamSpMM):
+        ctx.save_for_backward(Z, weight)
+        ctx.ParamSpMM = ParamSpMM
+        op = ParamSpMM
+        fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
+        return SpCONV.relu_input_forward(fmt, Z, weight, op.rowPtr, op.colIdx, op.val,
+                                         op.target_row if op.if_split else None, op.CF, op.blkWarpNum)
+
+    @staticmethod
+    def backward(ctx, d_output):
+        Z, weight = ctx.saved_tensors
+        op = ctx.ParamSpMM
+        fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
+        d_input, d_weight = SpCONV.relu_input_backward(fmt, d_output.contiguous(), Z, weight, op.rowPtr, op.colIdx, op.val,
+                                                       op.target_row if op.if_split else None, op.CF, op.blkWarpNum)
+        return d_input, d_weight, None
+
+
 class _Layer(torch.nn.Module):
     def __init__(self, input_dim, output_dim):
         super().__init__()
@@ -85,8 +110,11 @@ class _Layer(torch.nn.Module):
 
 
 class GCNConv(_Layer):
-    def forward(self, H, spmm_dict):
-        return GCNFunction.apply(H, self.weights, self._operator(spmm_dict))
+    def forward(self, H, spmm_dict, relu_input=False):
+        """``relu_input``: H holds pre-activation values and the layer computes A (relu(H) W); the activation and its
+        backward are folded into the dense products around the sparse one."""
+        fn = GCNReLUInputFunction if relu_input else GCNFunction
+        return fn.apply(H, self.weights, self._operator(spmm_dict))
 
 
 class AGNNFunction(torch.autograd.Function):

@@ -152,6 +152,7 @@ def test_row_caching_baseline_matches_oracle(oracle, N):
 
 
 def test_spconv_forward_backward(oracle):
+    import paramspmm_ae_amd  # noqa: F401
     import ParamSpCONV
     from paramspmm_ae_amd.PCSR import pcsr_spmm
 
@@ -198,6 +199,61 @@ def test_gcn_and_gin_layers_match_dense_autograd(vec, split):
         torch.testing.assert_close(layer.weights.grad, Wr.grad, rtol=1e-3, atol=1e-3)
     with pytest.raises(ValueError):
         GCNConv(32, 24).cuda()(X, {16: op})
+
+
+@pytest.mark.parametrize("vec,split", VARIANTS)
+@pytest.mark.parametrize("n,width_in,width_out", [(300, 24, 40), (20000, 32, 16), (20000, 16, 32), (17000, 128, 16), (16400, 128, 128)])
+def test_gcn_layer_with_relu_on_its_input(vec, split, n, width_in, width_out):
+    """A (relu(Z) W) as one function of Z against PyTorch autograd of the same expression (torch.sparse.mm): small
+    graphs and unsupported widths take the PyTorch path, 16384 rows and more with widths the library covers run the
+    activation inside the dense kernels."""
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from paramspmm_ae_amd.gnn_conv import GCNConv
+
+    g, rowPtr, colIdx, val = sym_graph(n, 5)
+    S = torch.sparse_csr_tensor(torch.from_numpy(rowPtr).cuda(), torch.from_numpy(colIdx).cuda(), torch.from_numpy(val).cuda(),
+                                size=(n, n))
+    op = pcsr_spmm(g, vec_size=vec, if_split=split, CF=1, blkWarpNum=4)
+    torch.manual_seed(3)
+    layer = GCNConv(width_in, width_out).cuda()
+    Z = torch.randn(n, width_in, device="cuda", requires_grad=True)
+    y = layer(Z, {width_out: op}, relu_input=True)
+    dY = torch.randn_like(y)
+    y.backward(dY)
+    Zr = Z.detach().clone().requires_grad_(True)
+    Wr = layer.weights.detach().clone().requires_grad_(True)
+    yr = torch.sparse.mm(S, torch.relu(Zr) @ Wr)
+    yr.backward(dY)
+    torch.testing.assert_close(y, yr, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(Z.grad, Zr.grad, rtol=1e-3, atol=1e-4)
+    torch.testing.assert_close(layer.weights.grad, Wr.grad, rtol=2e-3, atol=2e-3)
+    assert bool((Z.grad[Z.detach() <= 0] == 0).all())
+
+
+def test_gcn_network_with_folded_relu_equals_the_plain_one():
+    """Net_5layers with the activations folded into the layers gives the loss and the gradients of the network with
+    F.relu between the layers (GNN.py:43-61)."""
+    from paramspmm_ae_amd import GNN
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from paramspmm_ae_amd.gnn_conv import nll_loss_mean
+
+    n = 20000
+    g, rowPtr, colIdx, val = sym_graph(n, 8)
+    ops = {16: pcsr_spmm(g, vec_size=1, if_split=False, CF=1, blkWarpNum=4)}
+    torch.manual_seed(0)
+    x = torch.randn(n, 32, device="cuda")
+    labels = torch.randint(0, 16, (n,), device="cuda")
+    model = GNN.Net_5layers(16, 32, x, ops, 16).cuda()
+    grads = {}
+    for fused in (True, False):
+        model.fuse_relu = fused
+        model.zero_grad(set_to_none=True)
+        loss = nll_loss_mean(model(), labels)
+        loss.backward()
+        grads[fused] = (loss.item(), [p.grad.clone() for p in model.parameters()])
+    assert abs(grads[True][0] - grads[False][0]) <= 1e-5 * abs(grads[False][0])
+    for a, b in zip(grads[True][1], grads[False][1]):
+        torch.testing.assert_close(a, b, rtol=1e-3, atol=1e-5)
 
 
 @pytest.mark.parametrize("vec,split", VARIANTS)
