@@ -445,6 +445,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-vendor", action="store_true", help="skip the rocSPARSE comparison leg")
     ap.add_argument("--dump", default=None, help="write the full sweep table (every column, every width) as JSON")
+    ap.add_argument("--reorder", choices=["community", "degree"], default=None,
+                    help="spmm workload: permute rows and columns together at load time (paramspmm_ae_amd/reorder.py)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip what follows the timed region: decider check, gather ceiling, SDDMM and GCN legs")
     ap.add_argument("--workload", choices=["spmm", "agnn", "gcn", "build", "sddmm", "gather"], default="spmm",
@@ -480,7 +482,9 @@ def main():
     rowPtr, colIdx, val, n = synth.config_graph(args.graph)
     graph = graph_input(mtx_name=args.graph, path="")
     graph.verbose = False
-    graph.load_from_csr(rowPtr, colIdx, val)
+    t_re = time.time()
+    graph.load_from_csr(rowPtr, colIdx, val, reorder=args.reorder)
+    load_s = time.time() - t_re
     nnz = graph.mtx_edges
     ops = sweep.operators_of(graph)  # vec1, vec1_split, vec2, vec2_split on the GPU
     fmt_names = ["csr", "csr_split", "bcsr", "bcsr_split"]
@@ -537,9 +541,9 @@ def main():
     p = _capi.ptr
     L = _capi.lib
 
-    def launcher(d):
-        if_split, vec, cf, bw = chosen[d]
-        op = ops[(1 if if_split else 0) + (2 if vec == 2 else 0)]
+    def launcher(d, ops_, chosen_):
+        if_split, vec, cf, bw = chosen_[d]
+        op = ops_[(1 if if_split else 0) + (2 if vec == 2 else 0)]
         X, Y = Xs[d], Ys[d]
         a = (p(op.rowPtr), p(op.colIdx), p(op.val))
         nrows = op.rowPtr.numel() - 1
@@ -551,33 +555,38 @@ def main():
             return lambda: L.psp_spmm_bcsr_f32(*a, p(X), p(Y), nrows, d, rows, cf, bw, stream)
         return lambda: L.psp_spmm_bcsr_split_f32(*a, p(op.target_row), p(X), p(Y), nrows, d, rows, cf, bw, stream)
 
-    launch = {d: launcher(d) for d in dims}
+    def timed_steps(ops_, chosen_):
+        """args.warmup untimed steps, then args.steps timed ones bracketed by synchronisation; one step = one SpMM per
+        width.  Returns (wall seconds, {width: [(start event, stop event)]})."""
+        launch = {d: launcher(d, ops_, chosen_) for d in dims}
 
-    def step(events=None):
-        for d in dims:
-            if events is not None:
-                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                e0.record()
-            rc = launch[d]()
-            if events is not None:
-                e1.record()
-                events[d].append((e0, e1))
-            if rc != 0:
-                _capi.check(rc)
+        def step(events=None):
+            for d in dims:
+                if events is not None:
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                rc = launch[d]()
+                if events is not None:
+                    e1.record()
+                    events[d].append((e0, e1))
+                if rc != 0:
+                    _capi.check(rc)
+
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        events_ = {d: [] for d in dims}
+        t0_ = time.perf_counter()
+        for _ in range(args.steps):
+            step(events_)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0_, events_
 
     if args.calibrate_copy:
         d0 = dims[-1]
         Ys[d0].copy_(Xs[d0])  # moves 2 * rows * d0 * 4 bytes
         print("calibration copy: %d bytes read, %d bytes written" % (rows * d0 * 4, rows * d0 * 4), file=sys.stderr)
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    events = {d: [] for d in dims}
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step(events)
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
+    wall, events = timed_steps(ops, chosen)
 
     flops_step = sum(2.0 * nnz * d for d in dims)
     value = flops_step * args.steps / wall / 1e9
@@ -626,7 +635,8 @@ def main():
         "ms_per_step": round(wall * 1e3 / args.steps, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: R-MAT 2^20 nodes SpMM width sweep" % args.graph if args.graph == "C2" else args.graph,
-                   "nodes": n, "nnz": nnz, "dims": dims, "pick": pick, "setup_s": round(setup_s, 1)},
+                   "nodes": n, "nnz": nnz, "dims": dims, "pick": pick, "setup_s": round(setup_s, 1),
+                   "reorder": args.reorder, "load_s": round(load_s, 2)},
         "roofline": roofline,
         "sweep": per_dim,
     }
@@ -699,6 +709,33 @@ def main():
                                      "kernel": "psp_sddmm_kernel, K = 64, %s, %d wavefronts per workgroup" % (sfmt, sbw),
                                      "alg_bytes_per_launch": int(salg), "ms_per_launch": round(sms, 5)}}
         del A, Bm
+
+    if not args.no_extras and args.reorder is None and pick == "decider":
+        # ---- the same sweep after the community reordering pass (rows and columns permuted together at load time,
+        # paramspmm_ae_amd/reorder.py; the reference's inputs arrive Rabbit-ordered, README.md:14-16) ---------------
+        t1 = time.time()
+        graph_r = graph_input(mtx_name=args.graph, path="")
+        graph_r.verbose = False
+        graph_r.load_from_csr(rowPtr, colIdx, val, reorder="community")
+        load_r = time.time() - t1
+        ops_r = sweep.operators_of(graph_r)
+        chosen_r = {d: tuple(int(v) for v in decider.config_PCSR(graph_r, d)) for d in dims}
+        wall_r, events_r = timed_steps(ops_r, chosen_r)
+        F_r = {"n": n, "nnz": nnz, "S": graph_r.csr_data.target_row.numel(), "Mb": graph_r.bcsr_data.num_nodes,
+               "nblk": graph_r.bcsr_data.colIdx.numel(), "Sb": graph_r.bcsr_data.target_row.numel()}
+        fracs = []
+        for d in dims:
+            ms = float(np.mean([a.elapsed_time(b) for a, b in events_r[d]]))
+            if_split, vec, cf, bw = chosen_r[d]
+            fmt = fmt_names[(1 if if_split else 0) + (2 if vec == 2 else 0)]
+            fracs.append(algorithmic_bytes(fmt, F_r, n, d) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
+        out["reordered"] = {"order": "community (label propagation, vertices sorted by label)",
+                            "value": round(flops_step * args.steps / wall_r / 1e9, 1), "unit": "GFLOP/s",
+                            "ms_per_step": round(wall_r * 1e3 / args.steps, 4), "speedup": round(wall / wall_r, 3),
+                            "mean_frac_over_widths": round(float(np.mean(fracs)), 4),
+                            "load_s_with_reordering": round(load_r, 2), "load_s_without": round(load_s, 2)}
+        del ops_r, graph_r
+        torch.cuda.empty_cache()
 
     if not args.no_vendor:
         # vendor library beside it: rocSPARSE CSR SpMM (default algorithm), the counterpart of the cuSPARSE baseline

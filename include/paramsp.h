@@ -317,10 +317,14 @@ int psp_gemm_xw_act_f32(const float *X, const float *W, float *Y, long long n, i
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: mean negative log-likelihood, the loss of the reference's training step (F.nll_loss(model(), labels),
  * GNN.py:131-146), forward and backward.  logp is [n, C] row-major log-probabilities, labels are int64; rows whose
- * label is outside [0, C) do not count.  loss: one float.  stats: two floats of device memory that the forward
- * call fills (sum, count) and the backward call reads.  grad_loss: one float on the device (the incoming
- * gradient); grad_logp [n, C] is overwritten.  The sum is accumulated with fp32 atomics.
+ * label is outside [0, C) do not count.  loss: one float.  stats: psp_nll_loss_stats_floats() floats of device memory
+ * (contents irrelevant on entry) that the forward call fills -- [0] the sum, [1] the number of rows that count, [2] the
+ * number of labels outside [0, C) other than PyTorch's ignore_index -100 (PyTorch raises for those; check it where
+ * that matters), the rest workspace -- and the backward call reads.  grad_loss: one float on the device (the incoming
+ * gradient); grad_logp [n, C] is overwritten.  The partial sums of the workgroups are added in a fixed order: the
+ * loss repeats bit for bit.
  * ------------------------------------------------------------------------------------------- */
+int psp_nll_loss_stats_floats(void);
 int psp_nll_loss_mean_f32(const float *logp, const long long *labels, long long n, int C, float *loss, float *stats,
                           psp_stream_t stream);
 int psp_nll_loss_mean_backward_f32(const long long *labels, const float *grad_loss, const float *stats, long long n,

@@ -145,7 +145,7 @@ def train_profiling(model, labels, num_epoches, verbose=False, progress=False, h
     return ms
 
 
-def load_graph(net, path=None, mtx_name=None, synthetic=None, verbose=True):
+def load_graph(net, path=None, mtx_name=None, synthetic=None, verbose=True, reorder=None):
     """The per-network loader choices of GNN.py:189-195."""
     graph = graph_input(mtx_name=mtx_name if synthetic is None else synthetic, path=path)
     graph.verbose = verbose
@@ -159,7 +159,7 @@ def load_graph(net, path=None, mtx_name=None, synthetic=None, verbose=True):
             val[colIdx == _row_of(rowPtr)] = 1.5
         else:
             rowPtr, colIdx, val, n = synth.config_graph(synthetic)
-        graph.load_from_csr(rowPtr, colIdx, val, if_mask=(net == "AGNN"))
+        graph.load_from_csr(rowPtr, colIdx, val, if_mask=(net == "AGNN"), reorder=reorder)
     elif net == "GIN":
         graph.load(load_from_mtx=True, GIN_epsilon=0.5)
     elif net == "AGNN":
@@ -225,6 +225,9 @@ def main(argv=None):
     p.add_argument("--synthetic", type=str, default=None, help="C1, C2, C3, C3s, C5 or C5p instead of a .mtx file")
     p.add_argument("--hip_graph", action="store_true",
                    help="record the training step in a HIP graph and replay it per epoch (an addition of this build)")
+    p.add_argument("--reorder", choices=["community", "degree"], default=None,
+                   help="synthetic graphs: permute rows and columns together at load time (reorder.py); features and labels "
+                        "are generated in the new order")
     p.add_argument("--no_fuse_relu", action="store_true",
                    help="GCN: apply F.relu between the layers as passes of their own, as the reference's driver does")
     p.add_argument("--config", nargs=4, type=int, default=None, metavar=("IF_SPLIT", "VEC", "CF", "BW"),
@@ -250,7 +253,7 @@ def main(argv=None):
         for name in names:
             print("-------------mtx: {} hidden_size: {}-------------".format(name, hidden))
             t0 = time.perf_counter()
-            graph = load_graph(args.net, args.path, name, args.synthetic)
+            graph = load_graph(args.net, args.path, name, args.synthetic, reorder=args.reorder)
             t1 = time.perf_counter()
             ops = configure_operators(decider, graph, [hidden, args.num_classes],
                                       None if args.config is None else tuple(args.config))

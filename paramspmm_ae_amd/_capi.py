@@ -80,6 +80,7 @@ SIGNATURES = {
     "psp_spmm_f64": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "psp_sddmm_f64": [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp],
     "psp_baseline_rowcache_spmm_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _vp],
+    "psp_nll_loss_stats_floats": [],
     "psp_nll_loss_mean_f32": [_vp, _vp, ctypes.c_longlong, _i, _vp, _vp, _vp],
     "psp_nll_loss_mean_backward_f32": [_vp, _vp, _vp, ctypes.c_longlong, _i, _vp, _vp],
     "psp_probe_gather_out_floats": [ctypes.c_longlong, _i, _i, _i],

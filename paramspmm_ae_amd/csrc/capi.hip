@@ -216,14 +216,46 @@ psp_split_clear_kernel(const int *__restrict__ rowPtr_split, const int *__restri
     s_targeted[threadIdx.x] = 0;
     s_added[threadIdx.x] = 0;
     if (threadIdx.x == 0) s_count = 0;
-    if (threadIdx.x < 2) {  // first segment whose target is >= t0 (lane 0) / >= t1 (lane 1)
-        const int key = threadIdx.x == 0 ? t0 : t1;
-        int lo = 0, hi = nseg;
-        while (lo < hi) {
-            const int mid = (lo + hi) >> 1;
-            if (target_row[mid] < key) lo = mid + 1; else hi = mid;
+    // first segment whose target is >= t0 (lanes 0..127) / >= t1 (lanes 128..255): a 128-ary search, every round one
+    // independent load per lane instead of a chain of dependent loads in a single lane
+    {
+        __shared__ int s_lo[2], s_hi[2];
+        const int half = threadIdx.x >> 7, t = threadIdx.x & 127;
+        const int key = half == 0 ? t0 : t1;
+        if (t == 0) {
+            s_lo[half] = 0;
+            s_hi[half] = nseg;
         }
-        s_range[threadIdx.x] = lo;
+        __syncthreads();
+        while (true) {  // workgroup-uniform: both halves loop until both ranges are empty
+            const int lo = s_lo[half], hi = s_hi[half];
+            const bool done = s_lo[0] >= s_hi[0] && s_lo[1] >= s_hi[1];
+            __syncthreads();
+            if (done) break;
+            // invariant: target_row[i] < key for i < lo, target_row[i] >= key for i >= hi
+            const int step = (hi - lo + 127) >> 7;  // 0 when the half's range is empty
+            const int i = lo + t * step;
+            // probes are ascending and a probe past the range counts as >= key, so `ge` is false up to some lane and
+            // true from there on
+            const bool ge = step > 0 && (i >= hi || target_row[i] >= key);
+            const unsigned long long m = __ballot(ge);
+            __shared__ unsigned long long s_m[4];
+            if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6] = m;
+            __syncthreads();
+            if (t == 0 && step > 0) {
+                const unsigned long long m0 = s_m[2 * half], m1 = s_m[2 * half + 1];
+                const int first = m0 ? __ffsll((long long)m0) - 1 : (m1 ? 64 + __ffsll((long long)m1) - 1 : 128);
+                // probes before `first` are < key, probe `first` (if any) is >= key
+                int nlo = first == 0 ? lo : lo + (first - 1) * step + 1;
+                int nhi = first == 128 ? hi : lo + first * step;
+                if (nlo > hi) nlo = hi;
+                if (nhi > hi) nhi = hi;
+                s_lo[half] = nlo;
+                s_hi[half] = nhi;
+            }
+            __syncthreads();
+        }
+        if (t == 0) s_range[half] = s_lo[half];
     }
     __syncthreads();
     const int lo = s_range[0], hi = s_range[1];

@@ -4,41 +4,84 @@
 // of a 16-wide GCN epoch.  These run at the speed of reading the labels and writing the gradient.
 //
 // Rows whose label lies outside [0, C) do not count (PyTorch's ignore_index behaves the same way for its one
-// ignored value); the mean is over the rows that count.
+// ignored value, -100, and raises a device assertion for any other stray label); the mean is over the rows that
+// count, and the number of stray labels other than -100 is reported in stats[2] so that a caller can check.
+// No atomics: the result is the same bit for bit on every run.
 #include "psp_common.h"
 
-// stats[0] += sum of logp[i, label_i], stats[1] += number of rows that count
+#define PSP_NLL_MAX_BLOCKS 1024
+// stats layout (floats): [0] sum of logp[i, label_i], [1] number of rows that count, [2] number of labels that are
+// out of range without being PyTorch's ignore_index (-100), then one partial sum and one partial count per workgroup
+#define PSP_NLL_STATS_FLOATS (3 + 3 * PSP_NLL_MAX_BLOCKS)
+
+// every workgroup stores its partial sum, its row count and its count of stray labels in its own slots: no atomics
 __global__ void __launch_bounds__(256) nll_sum_kernel(const float *__restrict__ logp, const long long *__restrict__ labels,
                                                       long long n, int C, float *__restrict__ stats)
 {
-    __shared__ float s_sum[4], s_cnt[4];
-    float sum = 0.0f, cnt = 0.0f;
+    __shared__ float s_sum[4];
+    __shared__ int s_cnt[4], s_bad[4];
+    float sum = 0.0f;
+    int cnt = 0, bad = 0;
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
         const long long y = labels[i];
         if (y >= 0 && y < C) {
             sum += logp[i * C + y];
-            cnt += 1.0f;
+            cnt++;
+        } else if (y != -100) {
+            bad++;
         }
     }
 #pragma unroll
     for (int d = 1; d < PSP_WAVE; d <<= 1) {
         sum += __shfl_xor(sum, d);
         cnt += __shfl_xor(cnt, d);
+        bad += __shfl_xor(bad, d);
     }
     if ((threadIdx.x & 63) == 0) {
         s_sum[threadIdx.x >> 6] = sum;
         s_cnt[threadIdx.x >> 6] = cnt;
+        s_bad[threadIdx.x >> 6] = bad;
     }
     __syncthreads();
     if (threadIdx.x == 0) {
-        atomicAdd(stats, s_sum[0] + s_sum[1] + s_sum[2] + s_sum[3]);
-        atomicAdd(stats + 1, s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3]);
+        stats[3 + blockIdx.x] = (s_sum[0] + s_sum[1]) + (s_sum[2] + s_sum[3]);
+        ((int *)stats)[3 + PSP_NLL_MAX_BLOCKS + blockIdx.x] = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+        ((int *)stats)[3 + 2 * PSP_NLL_MAX_BLOCKS + blockIdx.x] = s_bad[0] + s_bad[1] + s_bad[2] + s_bad[3];
     }
 }
 
-__global__ void nll_finish_kernel(const float *__restrict__ stats, float *__restrict__ loss)
+// one workgroup adds the partial results in a fixed order (the loss repeats bit for bit from run to run and between
+// replays of a recorded step); the row count is an exact integer until it is stored
+__global__ void __launch_bounds__(256) nll_finish_kernel(float *__restrict__ stats, float *__restrict__ loss, int blocks)
 {
-    if (threadIdx.x == 0 && blockIdx.x == 0) *loss = -stats[0] / stats[1];
+    __shared__ float s_sum[256];
+    __shared__ long long s_cnt[256], s_bad[256];
+    float sum = 0.0f;
+    long long cnt = 0, bad = 0;
+    for (int b = threadIdx.x; b < blocks; b += 256) {
+        sum += stats[3 + b];
+        cnt += ((const int *)stats)[3 + PSP_NLL_MAX_BLOCKS + b];
+        bad += ((const int *)stats)[3 + 2 * PSP_NLL_MAX_BLOCKS + b];
+    }
+    s_sum[threadIdx.x] = sum;
+    s_cnt[threadIdx.x] = cnt;
+    s_bad[threadIdx.x] = bad;
+    __syncthreads();
+    for (int d = 128; d >= 1; d >>= 1) {
+        if ((int)threadIdx.x < d) {
+            s_sum[threadIdx.x] += s_sum[threadIdx.x + d];
+            s_cnt[threadIdx.x] += s_cnt[threadIdx.x + d];
+            s_bad[threadIdx.x] += s_bad[threadIdx.x + d];
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) {
+        const double count = (double)s_cnt[0];
+        stats[0] = s_sum[0];
+        stats[1] = (float)count;
+        stats[2] = (float)s_bad[0];
+        *loss = (float)(-(double)s_sum[0] / count);
+    }
 }
 
 // grad[i, c] = -g / count at c = label_i, 0 elsewhere; V consecutive columns per lane
@@ -62,20 +105,21 @@ __global__ void __launch_bounds__(256) nll_backward_kernel(const long long *__re
     }
 }
 
+PSP_EXPORT int psp_nll_loss_stats_floats(void) { return PSP_NLL_STATS_FLOATS; }
+
 PSP_EXPORT int psp_nll_loss_mean_f32(const float *logp, const long long *labels, long long n, int C, float *loss,
                                      float *stats, psp_stream_t stream)
 {
     PSP_REQUIRE(n >= 0 && C >= 1, "nll_loss: bad shape (n %lld, C %d)", n, C);
     PSP_REQUIRE(loss && stats && (n == 0 || (logp && labels)), "nll_loss: null pointer");
     hipStream_t st = (hipStream_t)stream;
-    int rc = psp_zero_f32(stats, 2, st);
-    if (rc != PSP_OK) return rc;
+    int blocks = 0;
     if (n > 0) {
-        int blocks = psp_ceil_div(n, 256 * 4);
-        if (blocks > 2048) blocks = 2048;
+        blocks = psp_ceil_div(n, 256 * 4);
+        if (blocks > PSP_NLL_MAX_BLOCKS) blocks = PSP_NLL_MAX_BLOCKS;
         hipLaunchKernelGGL(nll_sum_kernel, dim3(blocks), dim3(256), 0, st, logp, labels, n, C, stats);
     }
-    hipLaunchKernelGGL(nll_finish_kernel, dim3(1), dim3(64), 0, st, stats, loss);
+    hipLaunchKernelGGL(nll_finish_kernel, dim3(1), dim3(256), 0, st, stats, loss, blocks);
     return psp_check_launch("nll loss kernels");
 }
 

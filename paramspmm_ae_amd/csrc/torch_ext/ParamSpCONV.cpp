@@ -161,12 +161,12 @@ static void check_loss_args(const Tensor &logp, const Tensor &labels)
                 "nll_loss_mean: labels must be a contiguous int64 tensor with one entry per row");
     TORCH_CHECK(logp.device() == labels.device(), "nll_loss_mean: tensors on different devices");
 }
-// returns [loss (0-dim), stats (2 floats: sum, count) for the backward call]
+// returns [loss (0-dim), stats (sum, count, stray labels, workspace) for the backward call]
 static std::vector<Tensor> nll_loss_mean(Tensor logp, Tensor labels)
 {
     check_loss_args(logp, labels);
     DeviceGuard guard(logp.device());
-    Tensor loss = torch::empty({}, logp.options()), stats = torch::empty({2}, logp.options());
+    Tensor loss = torch::empty({}, logp.options()), stats = torch::empty({(long)psp_nll_loss_stats_floats()}, logp.options());
     ok(psp_nll_loss_mean_f32(fp(logp), (const long long *)labels.data_ptr<int64_t>(), logp.size(0), (int)logp.size(1),
                              loss.data_ptr<float>(), stats.data_ptr<float>(), stream_of(logp)));
     return {loss, stats};
@@ -178,7 +178,7 @@ static Tensor nll_loss_mean_backward(Tensor labels, Tensor grad_loss, Tensor sta
     need_gpu(stats, "stats");
     TORCH_CHECK(labels.scalar_type() == torch::kInt64 && labels.is_contiguous() && labels.numel() == n, "bad labels");
     TORCH_CHECK(grad_loss.scalar_type() == torch::kFloat32 && grad_loss.numel() == 1, "grad_loss must hold one float");
-    TORCH_CHECK(stats.scalar_type() == torch::kFloat32 && stats.numel() == 2 && stats.is_contiguous(), "bad stats");
+    TORCH_CHECK(stats.scalar_type() == torch::kFloat32 && stats.numel() >= 2 && stats.is_contiguous(), "bad stats");
     DeviceGuard guard(labels.device());
     Tensor grad = torch::empty({n, C}, stats.options());
     ok(psp_nll_loss_mean_backward_f32((const long long *)labels.data_ptr<int64_t>(), grad_loss.data_ptr<float>(),

@@ -178,7 +178,8 @@ class GINFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, d_output):
         X_agg, weights = ctx.saved_tensors
-        d_weights = SpCONV.weight_gradient(X_agg, d_output.contiguous())  # X_agg^T * d_output
+        d_output = d_output.contiguous()  # an upstream gradient may be a view (expand, transpose, slice)
+        d_weights = SpCONV.weight_gradient(X_agg, d_output)  # X_agg^T * d_output
         d_input = ctx.ParamSpMM.GIN_spmm(SpCONV.dense_xw(d_output, weights, True))
         return d_input, d_weights, None
 

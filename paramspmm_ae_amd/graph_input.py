@@ -246,6 +246,7 @@ class graph_input(object):
         self.csr_data = None
         self.bcsr_data = None
         self.pack_rate = None
+        self.perm = None  # set by load_from_csr(reorder=...): new position -> old vertex
         self.mask = None
         self.verbose = True
 
@@ -282,9 +283,24 @@ class graph_input(object):
         )
 
     def load_from_csr(self, rowPtr, colIdx, val, manual_granularity=None, is_avg_granularity=False, blk_size=2,
-                      if_mask=False, build_on="auto"):
+                      if_mask=False, build_on="auto", reorder=None):
         """Build every format from a square CSR matrix given as arrays (column indices sorted per row).
-        ``build_on``: "host", "device" or "auto" (the GPU when there is one) for the BCSR and row-split arrays."""
+        ``build_on``: "host", "device" or "auto" (the GPU when there is one) for the BCSR and row-split arrays.
+        ``reorder``: None, "community" or "degree" -- rows and columns are permuted together before anything is built
+        (reorder.py); ``self.perm`` (new position -> old vertex) says how, and features, labels and results move
+        with ``permute_rows`` / ``unpermute_rows``.  The reference's inputs are pre-ordered outside its repository
+        (Rabbit order, README.md:14-16)."""
+        self.perm = None
+        if reorder is not None:
+            from . import reorder as ro
+
+            if reorder == "community":
+                self.perm = ro.community_permutation(rowPtr, colIdx)
+            elif reorder == "degree":
+                self.perm = ro.degree_permutation(rowPtr)
+            else:
+                raise ValueError("reorder must be None, 'community' or 'degree'")
+            rowPtr, colIdx, val = ro.permute_csr(rowPtr, colIdx, val, self.perm)
         if blk_size not in (2, 3):
             raise ValueError("blocks of 2x1 and 3x1 are built (blk_size 2 or 3)")
         if if_mask and blk_size != 2:
@@ -340,6 +356,18 @@ class graph_input(object):
         if self.verbose:
             print("data format all preprocess (ms): {:.3f}".format((time.perf_counter() - t0) * 1e3))
         return self
+
+    def permute_rows(self, t):
+        """a per-vertex tensor in the order the graph was loaded in (identity without ``reorder``)"""
+        from . import reorder as ro
+
+        return t if self.perm is None else ro.permute_rows(t, self.perm)
+
+    def unpermute_rows(self, t):
+        """a result computed on the loaded graph back in the caller's vertex order"""
+        from . import reorder as ro
+
+        return t if self.perm is None else ro.unpermute_rows(t, self.perm)
 
     def get_split_csr(self, build_on="auto"):
         self.csr_split_flag = True

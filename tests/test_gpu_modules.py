@@ -437,6 +437,35 @@ def test_nll_loss_mean_matches_torch(n, C):
     (la * 3.0).backward()
     (lb * 3.0).backward()
     torch.testing.assert_close(a.grad, b.grad, rtol=1e-6, atol=0)
+    # fixed summation order: the value repeats bit for bit; stray labels other than -100 are counted for the caller
+    import paramspmm_ae_amd  # noqa: F401
+    import ParamSpCONV
+
+    again = [ParamSpCONV.nll_loss_mean(a.detach(), labels)[0].item() for _ in range(3)]
+    assert again[0] == again[1] == again[2] == la.item()
+    stray = labels.clone()
+    stray[0] = C + 5
+    loss, stats = ParamSpCONV.nll_loss_mean(a.detach(), stray)
+    kept = int(((stray >= 0) & (stray < C)).sum())
+    assert stats[1].item() == kept and stats[2].item() == 1.0
+
+
+def test_gin_backward_accepts_a_gradient_view():
+    """an upstream gradient that is an expanded / transposed view (as torch.mm accepts in the reference's layer)"""
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from paramspmm_ae_amd.gnn_conv import GINConv
+
+    n = 200
+    g, rowPtr, colIdx, val = sym_graph(n, 4)
+    op = pcsr_spmm(g, vec_size=1, if_split=False, CF=1, blkWarpNum=4)
+    layer = GINConv(32, 16).cuda()
+    X = torch.randn(n, 32, device="cuda", requires_grad=True)
+    y = layer(X, {16: op})
+    y.backward(torch.ones(1, 1, device="cuda").expand(n, 16))       # stride-0 view
+    first = X.grad.clone()
+    X.grad = None
+    layer(X, {16: op}).backward(torch.ones(16, n, device="cuda").t())  # transposed view
+    torch.testing.assert_close(X.grad, first)
 
 
 @pytest.mark.parametrize("K1,K2", [(16, 16), (32, 16), (48, 16), (64, 16), (128, 16), (16, 32), (32, 32), (48, 32), (64, 32),

@@ -387,3 +387,42 @@ def test_sddmm_harness_checks_and_column_orders():
             if_split, vec_size, cf, bw = sweep.decode_column(dim, col)
             assert name == "vec%d%s_TP_%s%d" % (vec_size, "_split" if if_split else "", sweep.cf_label(cf), bw)
     assert sweep.cf_label(3) == "3" and sweep.cf_label(_capi.pack_cf(2, 16, 2, 8, even_split=True)) == "c2l16u2w8e"
+
+
+def test_reordering_restores_community_order_and_is_a_similarity_transform():
+    """community_permutation on a randomly permuted block model: members of a planted community end up contiguous
+    (checked through the share of entries close to the diagonal), P A P^T keeps every entry, and results computed on
+    the reordered graph map back with unpermute_rows."""
+    import scipy.sparse as sp
+    from paramspmm_ae_amd import reorder, synth
+
+    r, c, n = synth.sbm(6000, 60, 18, 1.5, seed=4, permute=True)
+    rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+    A = sp.csr_matrix((val, colIdx, rowPtr), shape=(n, n))
+    perm = reorder.community_permutation(rowPtr, colIdx, device="cpu")
+    assert np.array_equal(np.sort(perm), np.arange(n))
+    rp2, ci2, v2 = reorder.permute_csr(rowPtr, colIdx, val, perm, device="cpu")
+    B = sp.csr_matrix((v2, ci2, rp2), shape=(n, n))
+    want = A[perm][:, perm].tocsr()
+    want.sort_indices()
+    assert np.array_equal(rp2, want.indptr) and np.array_equal(ci2, want.indices) and np.array_equal(v2, want.data)
+    assert all(np.all(np.diff(ci2[rp2[i]:rp2[i + 1]]) > 0) for i in range(0, n, 97))  # columns sorted again
+
+    def near(rp, ci):
+        rows = np.repeat(np.arange(n), np.diff(rp))
+        return float(np.mean(np.abs(rows - ci) <= 200))
+    assert near(rowPtr, colIdx) < 0.2 and near(rp2, ci2) > 0.8  # 18 of ~20 entries per row are in-community
+    x = np.random.default_rng(0).standard_normal((n, 3)).astype(np.float32)
+    y_new = B @ reorder.permute_rows(x, perm)
+    np.testing.assert_allclose(reorder.unpermute_rows(y_new, perm), A @ x, rtol=1e-5, atol=1e-6)
+    # degree order: hubs first, a permutation, stable
+    dperm = reorder.degree_permutation(rowPtr)
+    k = np.diff(rowPtr)
+    assert np.array_equal(np.sort(dperm), np.arange(n)) and np.all(np.diff(k[dperm]) <= 0)
+    with pytest.raises(ValueError):
+        reorder.permute_csr(rowPtr, colIdx, val, np.zeros(n, np.int64), device="cpu")
+    # a graph without communities keeps (almost) one label: the order is a permutation all the same
+    r, c, n2 = synth.rmat(11, 8 << 11, seed=3)
+    rp, ci, v = synth.to_gcn_csr(r, c, n2)
+    p2 = reorder.community_permutation(rp, ci, device="cpu")
+    assert np.array_equal(np.sort(p2), np.arange(n2))
