@@ -211,9 +211,15 @@ int psp_spmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b, const floa
  * kernels never multiply them in, SDDMM/sddmm_kernel.cu:917-983).  A and B are [*, K] row-major.
  * `scale` may be NULL; when given (an extension of this library used by the attention benchmark) the result
  * is multiplied by scale[p] (csr) -- pass NULL for the reference semantics.
+ * blkWarpNum | PSP_BW_BALANCED (plain layouts; ignored by the row-split ones): the stored entries, not the rows, are
+ * divided between the wavefronts of a fixed grid, so a plain matrix with hub rows runs as evenly as its row-split form
+ * (every entry's result is independent, a row can be cut anywhere).  The reference balances through the row-split
+ * format only (SDDMM/sddmm_kernel.cu:986-1057).
  * colIdx, out and the block values may all be NULL for a matrix without stored entries (an empty device
  * allocation has no address, and only rowPtr -- on the device -- says whether there are any).
  * ------------------------------------------------------------------------------------------- */
+
+#define PSP_BW_BALANCED 0x100
 
 /* ParamSDDMM.csr_sddmm, SDDMM/sddmm.cpp:15-65 -> sddmm_kernel.cu:143-192, 917-983.  out[nnz]. */
 int psp_sddmm_csr_f32(const int *rowPtr, const int *colIdx, const float *A, const float *B,

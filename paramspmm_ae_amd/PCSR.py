@@ -173,6 +173,15 @@ class pcsr_spmm(object):
         self.CF = CF
         self.blkWarpNum = blkWarpNum
         self.result = None
+        # Plain layouts of a graph with hub rows: the SDDMM divides the stored entries, not the rows, between its
+        # wavefronts (every entry's result is independent).  "Hub rows" = a longest row of more than 64 times the
+        # mean; arrays without statistics keep the row-wise walk.
+        self.sddmm_balanced = False
+        if graph is not None and not if_split:
+            fmt = graph.csr_data if vec_size == 1 else graph.bcsr_data
+            longest, mean = getattr(fmt, "max_row_nnz", None), getattr(fmt, "avg_degree", None)
+            if longest is not None and mean:
+                self.sddmm_balanced = float(longest) > 64.0 * float(mean)
 
     # ---- plumbing ---------------------------------------------------------------------------
     def _key(self):
@@ -226,6 +235,8 @@ class pcsr_spmm(object):
         else:
             fn = getattr(SDDMM, _SDDMM[self._key()])
         CF = (A.size(1) + 31) // 32
+        if self.sddmm_balanced and not self.if_split:
+            blkWarpNum |= 0x100  # PSP_BW_BALANCED: divide the entries, not the rows, between the wavefronts
         return fn(A, B, *self._sparse_args(), CF, blkWarpNum)
 
     def AGNN_sddmm(self, A):

@@ -52,7 +52,12 @@ template <int LOGL> __device__ __forceinline__ float psp_group_max(float v)
 // row_max (CSR layouts, may be null): the largest result of every row is also raised into row_max[row] (atomic
 // max, once per lane group and row; the caller has filled the array with the lowest float).  The attention
 // pipeline's softmax-weighted SpMM takes its reference maxima from there instead of sweeping the entries again.
-template <int LOGL, int C, int V, int U, int NR, bool SPLIT, bool SCALE>
+//
+// BAL (plain layouts): the launch is a fixed grid of wavefronts that divide the *stored entries* between them -- each
+// takes consecutive tiles of 2^logW entries, finds the rows that hold them with a 64-ary search in rowPtr and walks
+// them window by window (up to 64 rows at a time, cut at the tile's ends).  Every entry's result is independent, so a
+// row may be cut anywhere, and a hub row of 10^5 entries spreads over a hundred wavefronts instead of pinning one.
+template <int LOGL, int C, int V, int U, int NR, bool SPLIT, bool SCALE, bool BAL = false>
 __global__ void __launch_bounds__(512)
 psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
                  const int *__restrict__ target_row, const float *__restrict__ A, const float *__restrict__ B,
@@ -63,6 +68,7 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
     constexpr int L = 1 << LOGL;
     constexpr int R = PSP_WAVE >> LOGL;
     static_assert(U <= L, "unroll must not exceed the group width");
+    static_assert(!BAL || !SPLIT, "the entry-balanced walk is for the plain layouts (row-split input is balanced already)");
     __shared__ int2 s_seg[PSP_MAX_WAVES][PSP_WAVE];  // (end offset, A row) of the wavefront's filled segments
     // CSR results of narrow groups wait here until the group has 32 of them (a 128-byte line of `out`) and then leave
     // in one burst of stores: a group stores only L floats at a time, and lines written piecemeal are evicted from the
@@ -71,27 +77,33 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
     constexpr int HOLD = (NR <= 2 && LOGL >= 2 && LOGL + NR <= 5) ? ((32 / NR) >> LOGL) : 1;  // chunks held back per group
     __shared__ __align__(8) float s_hold[HOLD > 1 ? PSP_MAX_WAVES : 1][HOLD > 1 ? HOLD * PSP_WAVE * NR : 1];
 
-    const int tile = psp_xcd_tile(stripe);
-    if (tile >= tiles) return;
-
-    const int W = 1 << logW;
     const int lane = threadIdx.x & (PSP_WAVE - 1);
     const int wave = threadIdx.x >> 6;
     const int sub = lane & (L - 1);
     const int grp = lane >> LOGL;
     const int grp_base = lane - sub;
-    const int s0 = (tile * (int)(blockDim.x >> 6) + wave) << logW;
-    if (s0 >= nseg) return;  // wave-uniform
-    const int nvalid = min(W, nseg - s0);
 
-    const int P0 = rowPtr[s0];
-    const int P1 = rowPtr[s0 + nvalid];
+    int off[C];
+    bool live[C];
+#pragma unroll
+    for (int i = 0; i < C; i++) {
+        const int col = ((i << LOGL) + sub) * V;
+        live[i] = col < K;
+        off[i] = live[i] ? col : K - V;
+    }
+
+    // One window: the segments s0 .. s0+nvalid-1 (at most 64), of which only the entries inside [pbeg, pend) count
+    // (the plain walk passes the whole range of the segments).  tabW: power of two >= nvalid.
+    auto run_window = [&](const int s0, const int nvalid, const int pbeg, const int pend, const int tabW) {
+    const int W = tabW;
+    const int P0 = pbeg;
+    const int P1 = min(rowPtr[s0 + nvalid], pend);
     {
         const bool in = lane < nvalid;
-        const int e = in ? rowPtr[s0 + lane + 1] : P1;
+        const int e = in ? min(rowPtr[s0 + lane + 1], pend) : P1;
         const int e_up = __shfl_up(e, 1);  // cross-lane reads stay outside any lane-dependent branch
         const int b_ = (lane == 0) ? P0 : e_up;
-        const bool filled = in && e != b_;
+        const bool filled = in && e > b_;
         const unsigned long long fmask = __ballot(filled);
         const int slot = __popcll(fmask & ((1ull << lane) - 1ull));
         s_seg[wave][lane] = make_int2(P1, -1);
@@ -103,22 +115,13 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     const int2 *w_seg = s_seg[wave];
-    if (P0 == P1) return;
+    if (P0 >= P1) return;
 
     const int q = (P1 - P0 + R - 1) >> (6 - LOGL);
     int a0 = P0 + grp * q;
     if (a0 > P1) a0 = P1;
     const int b0 = min(P1, a0 + q);
     if (a0 >= b0) return;  // the whole group leaves together; nothing below reads other groups' lanes
-
-    int off[C];
-    bool live[C];
-#pragma unroll
-    for (int i = 0; i < C; i++) {
-        const int col = ((i << LOGL) + sub) * V;
-        live[i] = col < K;
-        off[i] = live[i] ? col : K - V;
-    }
 
     // A row(s) of a segment; dead tail vectors are zero so they add nothing to the dot product
     auto load_a = [&](int key, float (&dst)[NR][C][V]) {
@@ -288,6 +291,53 @@ psp_sddmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx,
     }
     if constexpr (HOLD > 1) release();
     if (want_max) emit_row_max(mykey);
+    };  // run_window
+
+    if constexpr (!BAL) {
+        const int tile = psp_xcd_tile(stripe);
+        if (tile >= tiles) return;
+        const int s0 = (tile * (int)(blockDim.x >> 6) + wave) << logW;
+        if (s0 >= nseg) return;  // wave-uniform
+        run_window(s0, min(1 << logW, nseg - s0), rowPtr[s0], 0x7fffffff, 1 << logW);
+    } else {
+        // Tiles of 2^logW stored entries.  Each XCD (workgroups are dealt to them round-robin) owns one contiguous
+        // eighth of the tiles and its wavefronts take them in turn, so at any time an XCD works on a run of
+        // neighbouring tiles -- neighbouring rows, whose B rows share its L2 -- and all XCDs carry the same load.
+        const int nnz = rowPtr[nseg];
+        const int ntiles = (int)(((long long)nnz + (1 << logW) - 1) >> logW);
+        const int wpb = blockDim.x >> 6;
+        const int xcd = blockIdx.x % PSP_XCDS;
+        const int waves_per_xcd = (gridDim.x / PSP_XCDS) * wpb;
+        const int tiles_per_xcd = (ntiles + PSP_XCDS - 1) / PSP_XCDS;
+        const int band_end = min(ntiles, (xcd + 1) * tiles_per_xcd);
+        for (int t = xcd * tiles_per_xcd + (blockIdx.x / PSP_XCDS) * wpb + wave; t < band_end; t += waves_per_xcd) {
+        const int e0 = t << logW;
+        const int e1 = min(nnz, e0 + (1 << logW));
+        // first row whose end lies past e0: 64-ary search, one independent load per lane and round
+        int lo = 0, hi = nseg;  // rowPtr[i + 1] <= e0 for i < lo, > e0 for i >= hi
+        while (lo < hi) {
+            const int step = (hi - lo + 63) >> 6;
+            const int i = lo + lane * step;
+            const bool gt = i >= hi || rowPtr[i + 1] > e0;  // ascending probes: false up to some lane, true from there on
+            const unsigned long long m = __ballot(gt);
+            const int f = m ? __ffsll((long long)m) - 1 : 64;
+            int nlo = f == 0 ? lo : lo + (f - 1) * step + 1;
+            int nhi = f == 64 ? hi : lo + f * step;
+            lo = nlo < hi ? nlo : hi;
+            hi = nhi < hi ? nhi : hi;
+        }
+        int s0 = lo, pbeg = e0;
+        while (pbeg < e1 && s0 < nseg) {  // wave-uniform
+            const int nvalid = min(PSP_WAVE, nseg - s0);
+            run_window(s0, nvalid, pbeg, e1, PSP_WAVE);
+            // the next window's table overwrites this one's: every group has finished reading it here
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            pbeg = min(rowPtr[s0 + nvalid], e1);
+            s0 += nvalid;
+        }
+        }  // tiles of this wavefront
+    }
 }
 
 typedef void (*psp_sddmm_kernel_t)(const int *, const int *, const float *, const int *, const float *,
@@ -299,14 +349,14 @@ typedef void (*psp_sddmm_kernel_t)(const int *, const int *, const float *, cons
     M_(0, 1, 1) M_(1, 1, 2) M_(2, 1, 4) M_(3, 1, 4) M_(4, 1, 4) \
     M_(4, 2, 4) M_(4, 3, 2) M_(4, 4, 2) M_(5, 4, 2) M_(6, 4, 2)
 
-template <int NR, bool SPLIT, bool SCALE>
+template <int NR, bool SPLIT, bool SCALE, bool BAL = false>
 static psp_sddmm_kernel_t psp_sddmm_lookup(int logL, int C, int V)
 {
 #define PSP_CASE(L_, C_, U_)                                                               \
     if (logL == L_ && C == C_) {                                                           \
-        if (V == 4) return psp_sddmm_kernel<L_, C_, 4, U_, NR, SPLIT, SCALE>;            \
-        if (V == 2) return psp_sddmm_kernel<L_, C_, 2, U_, NR, SPLIT, SCALE>;            \
-        return psp_sddmm_kernel<L_, C_, 1, U_, NR, SPLIT, SCALE>;                        \
+        if (V == 4) return psp_sddmm_kernel<L_, C_, 4, U_, NR, SPLIT, SCALE, BAL>;       \
+        if (V == 2) return psp_sddmm_kernel<L_, C_, 2, U_, NR, SPLIT, SCALE, BAL>;       \
+        return psp_sddmm_kernel<L_, C_, 1, U_, NR, SPLIT, SCALE, BAL>;                   \
     }
     PSP_SDDMM_FOR_EACH_LCU(PSP_CASE)
 #undef PSP_CASE

@@ -8,6 +8,8 @@ int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, con
                      int blkWarpNum, hipStream_t stream, float *row_max)
 {
     constexpr bool BCSR = NR > 1;
+    const bool balanced = !SPLIT && (blkWarpNum & PSP_BW_BALANCED) != 0;  // plain layouts only; row-split input is balanced
+    blkWarpNum &= ~PSP_BW_BALANCED;
     PSP_REQUIRE(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8");
     PSP_REQUIRE(nrows >= 0 && K >= 1, "sddmm: bad size (rows %d, K %d)", nrows, K);
     if (nrows == 0) return PSP_OK;
@@ -31,7 +33,20 @@ int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, con
 
     psp_sddmm_kernel_t k = scale ? psp_sddmm_lookup<NR, SPLIT, !BCSR>(logL, C, V)
                                  : psp_sddmm_lookup<NR, SPLIT, false>(logL, C, V);
+    if constexpr (!SPLIT) {
+        if (balanced)
+            k = scale ? psp_sddmm_lookup<NR, false, !BCSR, true>(logL, C, V) : psp_sddmm_lookup<NR, false, false, true>(logL, C, V);
+    }
     if (!k) return psp_fail(PSP_ERR_ARG, "sddmm: no kernel for logL %d coarsen %d vec %d", logL, C, V);
+    if (balanced) {
+        // A fixed grid that fills the GPU once; its wavefronts divide the stored entries between them in tiles of 256
+        // (the entry count is on the device, in rowPtr): each XCD takes one contiguous eighth of the tiles.
+        const int wgs = 256 * 32 / blkWarpNum;
+        dim3 grid(wgs, 1, 1), block(blkWarpNum * PSP_WAVE, 1, 1);
+        hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, BCSR ? val : scale, target_row, A, B, out, nrows, K,
+                           8, wgs, wgs / PSP_XCDS, row_max);
+        return psp_check_launch("sddmm kernel (entry-balanced)");
+    }
 
     // segments per wavefront: as for SpMM (one per lane group for plain input, 16 for row-split input, fewer for
     // small matrices)

@@ -34,10 +34,10 @@ def test_sddmm_parity(oracle, small, fmt, K):
     A = unit_rows(F.n + (F.n & 1), K, K)
     B = unit_rows(F.n, K, K + 1)
     want = sddmm_oracle(oracle, fmt, F, A, B)
-    for bw in (4, 8):
+    for bw in (4, 8, 4 | 0x100, 8 | 0x100):  # 0x100: the entry-balanced walk of the plain layouts (PSP_BW_BALANCED)
         got = sddmm_capi(fmt, F, torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), bw)
         torch.cuda.synchronize()
-        assert_close(got, want, what="%s K=%d bw=%d" % (fmt, K, bw))
+        assert_close(got, want, what="%s K=%d bw=%#x" % (fmt, K, bw))
 
 
 @pytest.mark.parametrize("fmt", FMTS)
@@ -322,3 +322,38 @@ def test_facade_sddmm_with_3x1_blocks(oracle):
         assert_close(got, want, what="facade 3x1 sddmm split=%s" % split)
         ones = op.get_sddmm_result(64, 8)
         assert torch.all(ones[torch.from_numpy(vb != 0).cuda()] == 64)
+
+
+@pytest.mark.parametrize("fmt", ["csr", "bcsr"])
+def test_sddmm_entry_balanced_walk_structures(oracle, fmt):
+    """The entry-balanced walk on the structures that stress it: a hub row spanning many wavefronts' tiles, runs of
+    hundreds of empty rows (windows of 64 rows without an entry), rows of one entry (more than 64 rows per tile),
+    a matrix smaller than one tile, an empty matrix; bit-identical to the row-wise walk (same dot products, same
+    order inside a lane group is not guaranteed, so: to tolerance) and equal to the oracle."""
+    from gpu_util import Formats, sddmm_capi, sddmm_oracle, assert_close
+
+    rng = np.random.default_rng(5)
+    cases = {}
+    n = 9000
+    deg = np.ones(n, np.int64)
+    deg[100] = 8000
+    deg[2000:2900] = 0
+    deg[5000:5200] = rng.integers(40, 90, 200)
+    deg[-300:] = 0
+    rowPtr = np.zeros(n + 1, np.int32)
+    rowPtr[1:] = np.cumsum(deg)
+    cols = np.concatenate([np.sort(rng.choice(n, d, replace=False)) for d in deg]).astype(np.int32)
+    cases["mixed"] = (rowPtr, cols, rng.uniform(0.1, 1, cols.size).astype(np.float32))
+    cases["tiny"] = random_csr(37, 3, 9, values="uniform")
+    cases["empty"] = (np.zeros(11, np.int32), np.zeros(0, np.int32), np.zeros(0, np.float32))
+    for name, (rp, ci, v) in cases.items():
+        F = Formats(oracle, rp, ci, v)
+        for K in (16, 64, 100):
+            print("case", fmt, name, K, flush=True)
+            A = unit_rows(F.n + (F.n & 1), K, K)
+            B = unit_rows(F.n + (F.n & 1), K, K + 1)
+            want = sddmm_oracle(oracle, fmt, F, A, B)
+            for bw in (4 | 0x100, 8 | 0x100):
+                got = sddmm_capi(fmt, F, torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), bw)
+                torch.cuda.synchronize()
+                assert_close(got, want, what="%s %s K=%d balanced" % (fmt, name, K))
