@@ -228,6 +228,8 @@ def main(argv=None):
     p.add_argument("--reorder", choices=["community", "degree"], default=None,
                    help="synthetic graphs: permute rows and columns together at load time (reorder.py); features and labels "
                         "are generated in the new order")
+    p.add_argument("--no_aggregate_first", action="store_true",
+                   help="GCN: always A (H W), also for the first layer when it widens its input (the reference's order)")
     p.add_argument("--no_fuse_relu", action="store_true",
                    help="GCN: apply F.relu between the layers as passes of their own, as the reference's driver does")
     p.add_argument("--config", nargs=4, type=int, default=None, metavar=("IF_SPLIT", "VEC", "CF", "BW"),
@@ -255,8 +257,11 @@ def main(argv=None):
             t0 = time.perf_counter()
             graph = load_graph(args.net, args.path, name, args.synthetic, reorder=args.reorder)
             t1 = time.perf_counter()
-            ops = configure_operators(decider, graph, [hidden, args.num_classes],
-                                      None if args.config is None else tuple(args.config))
+            dims = [hidden, args.num_classes]
+            if (args.net == "GCN" and not args.no_aggregate_first and args.num_features < hidden
+                    and (decider is None or args.num_features in decider.model_dict)):
+                dims.append(args.num_features)  # the first layer runs its sparse product at the features' width
+            ops = configure_operators(decider, graph, dims, None if args.config is None else tuple(args.config))
             print("SpMM-decider config time: {:.3f} (ms)".format((time.perf_counter() - t1) * 1e3))
             model = build_model(args.net, graph, ops, hidden, args.num_features, args.num_classes, args.num_layers)
             if args.no_fuse_relu and hasattr(model, "fuse_relu"):

@@ -129,6 +129,17 @@ static std::vector<Tensor> relu_input_backward(int fmt, Tensor dY, Tensor Z, Ten
     return {dense_xwt_masked(AG, W, Z), weight_gradient_relu(Z, AG)};
 }
 
+// A * D alone, for callers that place the sparse product on the narrower side of the layer: (A H) W costs a sparse
+// product of width in_features where A (H W) costs one of width out_features.  No counterpart among the reference's
+// bindings, whose layer is always A (H W) (SpCONV/SpCONV.h:43-48).
+static Tensor aggregate_op(int fmt, Tensor D, Tensor rowPtr, Tensor colIdx, Tensor values, c10::optional<Tensor> target_row,
+                           int CF, int bw)
+{
+    need_gpu(D, "input");
+    TORCH_CHECK(fmt >= 0 && fmt <= 3 && ((fmt & 1) != 0) == target_row.has_value(), "format code and target_row disagree");
+    return aggregate(fmt, D, rowPtr, colIdx, values, target_row ? &*target_row : nullptr, CF, bw);
+}
+
 static Tensor forward_impl(int fmt, const Tensor &H, const Tensor &W, const Tensor &rowPtr, const Tensor &colIdx,
                            const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
 {
@@ -230,6 +241,7 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     }, "X * W (transW false) or X * W^T for tall-skinny X: (X, W, transW)");
     m.def("nll_loss_mean", &nll_loss_mean, "[loss, stats] of the mean negative log-likelihood (log-probabilities, int64 labels)");
     m.def("nll_loss_mean_backward", &nll_loss_mean_backward, "gradient w.r.t. the log-probabilities: (labels, grad_loss, stats, n, C)");
+    m.def("aggregate", &aggregate_op, "A*D: (fmt, D, rowPtr, colIdx, values, target_row | None, CF, blkWarpNum)");
     m.def("relu_input_forward", &relu_input_forward,
           "A*(relu(Z)*W): (fmt 0..3, Z, W, rowPtr, colIdx, values, target_row or None, CF, blkWarpNum)");
     m.def("relu_input_backward", &relu_input_backward,

@@ -9,6 +9,7 @@ followed by native wave64 configurations packed into the same integer), then the
 """
 import math
 import os
+import gzip
 import pickle
 
 from .PCSR import decider_CF_list, dynamic_CF_prompter
@@ -36,6 +37,8 @@ class SpMMDecider(object):
             if not os.path.exists(pickle_file):
                 raise ValueError("pickle file not found for dim-" + str(dim) + " at path: " + pickle_file + "\n")
             with open(pickle_file, "rb") as f:
+                gz = f.read(2) == b"\x1f\x8b"  # the forests this package ships are gzip-compressed pickles
+            with (gzip.open if gz else open)(pickle_file, "rb") as f:
                 self.tree_dict[dim] = pickle.load(f)
         return self.tree_dict[dim]
 

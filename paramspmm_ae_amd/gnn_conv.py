@@ -24,6 +24,13 @@ def _conv_name(op):
     return _CONV[(bool(op.if_split), op.vec_size != 1)]
 
 
+def _aggregate(op, D):
+    """A D through ``op``'s format and configuration."""
+    fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
+    return SpCONV.aggregate(fmt, D, op.rowPtr, op.colIdx, op.val, op.target_row if op.if_split else None, op.CF,
+                            op.blkWarpNum)
+
+
 class _NllLossMean(torch.autograd.Function):
     @staticmethod
     def forward(ctx, logp, labels):
@@ -63,7 +70,35 @@ class GCNFunction(torch.autograd.Function):
     def backward(ctx, d_output):
         H, weight = ctx.saved_tensors
         op = ctx.ParamSpMM
+        if not ctx.needs_input_grad[0]:
+            # the network's first layer: its input holds features, nothing asks for their gradient
+            return None, SpCONV.weight_gradient(H, _aggregate(op, d_output)), None
         d_input, d_weight = getattr(SpCONV, _conv_name(op) + "_backward")(d_output.contiguous(), H, weight, *_conv_args(op))
+        return d_input, d_weight, None
+
+
+class GCNAggregateFirstFunction(torch.autograd.Function):
+    """The same layer computed as (A H) W: for a layer that widens its input (in_features < out_features) the sparse
+    product then runs at the input's width.  Backward: dW = (A H)^T dY (A H is kept from the forward pass, so the
+    weight gradient needs no sparse product) and dH = A (dY W^T), again at the input's width -- A is symmetric, as in
+    the reference's own backward (gnn_conv.py:56-107).  ``ParamSpMM`` is the operator configured for the *input*
+    width."""
+
+    @staticmethod
+    def forward(ctx, H, weight, ParamSpMM):
+        AH = _aggregate(ParamSpMM, H)
+        ctx.save_for_backward(AH, weight)
+        ctx.ParamSpMM = ParamSpMM
+        return SpCONV.dense_xw(AH, weight, False)
+
+    @staticmethod
+    def backward(ctx, d_output):
+        AH, weight = ctx.saved_tensors
+        d_output = d_output.contiguous()
+        d_weight = SpCONV.weight_gradient(AH, d_output)
+        d_input = None
+        if ctx.needs_input_grad[0]:
+            d_input = _aggregate(ctx.ParamSpMM, SpCONV.dense_xw(d_output, weight, True))
         return d_input, d_weight, None
 
 
@@ -110,9 +145,18 @@ class _Layer(torch.nn.Module):
 
 
 class GCNConv(_Layer):
+    aggregate_first = True  # (A H) W where that is the cheaper order and spmm_dict holds an operator for H's width
+
     def forward(self, H, spmm_dict, relu_input=False):
         """``relu_input``: H holds pre-activation values and the layer computes A (relu(H) W); the activation and its
-        backward are folded into the dense products around the sparse one."""
+        backward are folded into the dense products around the sparse one.
+
+        A layer that widens its input is computed as (A H) W when ``spmm_dict`` also holds an operator for the input's
+        width (the reference's layers look up the output's width only, gnn_conv.py:121-124, and always compute
+        A (H W))."""
+        in_w, out_w = self.weights.shape
+        if self.aggregate_first and not relu_input and in_w < out_w and in_w in spmm_dict:
+            return GCNAggregateFirstFunction.apply(H, self.weights, spmm_dict[in_w])
         fn = GCNReLUInputFunction if relu_input else GCNFunction
         return fn.apply(H, self.weights, self._operator(spmm_dict))
 

@@ -19,6 +19,7 @@ SuiteSparse / OGB collection the reference downloads.
 import argparse
 import json
 import os
+import gzip
 import pickle
 import sys
 import time
@@ -311,7 +312,8 @@ def fit_main(args):
         final = _fit_forest(X, TP, near, n_est, leaves)
         final.n_jobs = 1
         final.psp_cf_list_ = [int(c) for c in cf_lists[d]]  # the CF axis of the class codes (decider.config_PCSR)
-        with open(os.path.join(args.out, "rnd_tree_%d.pkl" % d), "wb") as f:
+        # gzip-compressed (the per-node class histograms are mostly zeros); SpMMDecider.load_pickle reads both forms
+        with gzip.GzipFile(os.path.join(args.out, "rnd_tree_%d.pkl" % d), "wb", compresslevel=6, mtime=0) as f:
             pickle.dump(final, f)
         print("dim %3d: %2d classes  near %.2f  n_estimators %d  leaves %d  acc %.3f  mean norm perf %.4f  within 10%%: %.3f  worst %.3f" % (
             d, TP.shape[1], near, n_est, leaves, report["per_dim"][d]["accuracy"], mean_norm, within10, norm.min()), flush=True)

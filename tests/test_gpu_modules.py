@@ -230,6 +230,42 @@ def test_gcn_layer_with_relu_on_its_input(vec, split, n, width_in, width_out):
     assert bool((Z.grad[Z.detach() <= 0] == 0).all())
 
 
+@pytest.mark.parametrize("vec,split", VARIANTS)
+@pytest.mark.parametrize("n,width_in,width_out,need_dx", [(300, 16, 40, True), (20000, 32, 128, True), (20000, 32, 128, False),
+                                                         (20000, 16, 32, False), (17000, 32, 16, False)])
+def test_gcn_layer_with_the_sparse_product_on_the_narrow_side(vec, split, n, width_in, width_out, need_dx):
+    """A widening layer given an operator for its input's width computes (A H) W; a layer whose input needs no
+    gradient (the network's first) skips the input gradient.  Both against PyTorch autograd of A (H W)."""
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from paramspmm_ae_amd import gnn_conv
+
+    g, rowPtr, colIdx, val = sym_graph(n, 6)
+    S = torch.sparse_csr_tensor(torch.from_numpy(rowPtr).cuda(), torch.from_numpy(colIdx).cuda(), torch.from_numpy(val).cuda(),
+                                size=(n, n))
+    op = pcsr_spmm(g, vec_size=vec, if_split=split, CF=1, blkWarpNum=4)
+    torch.manual_seed(4)
+    layer = gnn_conv.GCNConv(width_in, width_out).cuda()
+    H = torch.randn(n, width_in, device="cuda", requires_grad=need_dx)
+    y = layer(H, {width_out: op, width_in: op})
+    assert type(y.grad_fn).__name__.startswith("GCNAggregateFirstFunction" if width_in < width_out else "GCNFunction")
+    dY = torch.randn_like(y)
+    y.backward(dY)
+    Hr = H.detach().clone().requires_grad_(True)
+    Wr = layer.weights.detach().clone().requires_grad_(True)
+    yr = torch.sparse.mm(S, Hr @ Wr)
+    yr.backward(dY)
+    torch.testing.assert_close(y, yr, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(layer.weights.grad, Wr.grad, rtol=2e-3, atol=2e-3)
+    if need_dx:
+        torch.testing.assert_close(H.grad, Hr.grad, rtol=1e-3, atol=1e-4)
+    else:
+        assert H.grad is None
+    # without an operator for the input's width the layer keeps the reference's order
+    y2 = layer(H, {width_out: op})
+    assert type(y2.grad_fn).__name__.startswith("GCNFunction")
+    torch.testing.assert_close(y2, yr, rtol=1e-4, atol=1e-5)
+
+
 def test_gcn_network_with_folded_relu_equals_the_plain_one():
     """Net_5layers with the activations folded into the layers gives the loss and the gradients of the network with
     F.relu between the layers (GNN.py:43-61)."""
