@@ -197,93 +197,89 @@ int psp_row_scale(float *Y, const float *s, int rows, int N, hipStream_t stream)
 }
 
 // ------------------------------------------------------------------------------------------------
-// selective clear for row-split SpMM.  A workgroup owns 256 consecutive target rows: it finds the segments that
-// target them (target_row is sorted: two binary searches), marks in LDS which rows a segment targets and which of
-// those the SpMM kernel will add to rather than store (a row continuing across two wavefronts, a row with an empty
-// segment), and then clears the rows that need it -- rows nothing targets included -- one wavefront per row with
-// 16-byte stores.  Runs of untargeted rows of any length are thus spread over the whole grid.
+// selective clear for row-split SpMM: the rows the SpMM kernel adds to rather than stores (a row continuing across
+// two wavefronts, a row with an empty segment) and the rows no segment targets.
+//
+// The first `seg_blocks` workgroups walk the segments, one lane per segment (coalesced loads of target_row and
+// rowPtr_split, no search): a wavefront clears the rows its 64 segments flag, and the run of untargeted rows in front
+// of each segment's row (after the last segment too) -- up to PSP_CLEAR_CAP rows of it.  Hub rows of a thousand
+// segments cost nothing extra this way (a workgroup per 256 target rows, which this replaces, spent 85 us scanning
+// the segments of the R-MAT graph's first 256 rows while the rest of the grid had long finished).
+// The remaining workgroups sweep what is left of long runs: one wavefront per PSP_CLEAR_CAP target rows finds the
+// segment its rows start at (a 64-ary search in target_row, one independent load per lane and round) and clears the
+// rows of its block that lie in a run beyond the run's first PSP_CLEAR_CAP rows.  A run that reaches past its cap
+// into a block contains the block's first row, so that one search finds it; a run of 10^5 untargeted rows spreads
+// over hundreds of wavefronts.
 // ------------------------------------------------------------------------------------------------
-#define PSP_CLEAR_ROWS 256
+#define PSP_CLEAR_CAP 256
+
+__device__ __forceinline__ void psp_wave_clear(float *__restrict__ Y, size_t b0, size_t b1, int lane, bool vec4)
+{
+    if (vec4) {
+        const psp_f32x4 z = {0.f, 0.f, 0.f, 0.f};
+        for (size_t j = b0 + 4 * (size_t)lane; j < b1; j += 256) *(psp_f32x4 *)(Y + j) = z;
+    } else {
+        for (size_t j = b0 + lane; j < b1; j += 64) Y[j] = 0.0f;
+    }
+}
 
 __global__ void __launch_bounds__(256)
 psp_split_clear_kernel(const int *__restrict__ rowPtr_split, const int *__restrict__ target_row, float *__restrict__ Y,
-                       int nseg, int N, int nr, int rows_out, int logW)
+                       int nseg, int N, int nr, int rows_out, int logW, int seg_blocks)
 {
-    __shared__ int s_targeted[PSP_CLEAR_ROWS], s_added[PSP_CLEAR_ROWS], s_list[PSP_CLEAR_ROWS];
-    __shared__ int s_range[2], s_count;
     const int ntargets = (rows_out + nr - 1) / nr;
-    const int t0 = blockIdx.x * PSP_CLEAR_ROWS, t1 = min(ntargets, t0 + PSP_CLEAR_ROWS);
-    s_targeted[threadIdx.x] = 0;
-    s_added[threadIdx.x] = 0;
-    if (threadIdx.x == 0) s_count = 0;
-    // first segment whose target is >= t0 (lanes 0..127) / >= t1 (lanes 128..255): a 128-ary search, every round one
-    // independent load per lane instead of a chain of dependent loads in a single lane
-    {
-        __shared__ int s_lo[2], s_hi[2];
-        const int half = threadIdx.x >> 7, t = threadIdx.x & 127;
-        const int key = half == 0 ? t0 : t1;
-        if (t == 0) {
-            s_lo[half] = 0;
-            s_hi[half] = nseg;
-        }
-        __syncthreads();
-        while (true) {  // workgroup-uniform: both halves loop until both ranges are empty
-            const int lo = s_lo[half], hi = s_hi[half];
-            const bool done = s_lo[0] >= s_hi[0] && s_lo[1] >= s_hi[1];
-            __syncthreads();
-            if (done) break;
-            // invariant: target_row[i] < key for i < lo, target_row[i] >= key for i >= hi
-            const int step = (hi - lo + 127) >> 7;  // 0 when the half's range is empty
-            const int i = lo + t * step;
-            // probes are ascending and a probe past the range counts as >= key, so `ge` is false up to some lane and
-            // true from there on
-            const bool ge = step > 0 && (i >= hi || target_row[i] >= key);
-            const unsigned long long m = __ballot(ge);
-            __shared__ unsigned long long s_m[4];
-            if ((threadIdx.x & 63) == 0) s_m[threadIdx.x >> 6] = m;
-            __syncthreads();
-            if (t == 0 && step > 0) {
-                const unsigned long long m0 = s_m[2 * half], m1 = s_m[2 * half + 1];
-                const int first = m0 ? __ffsll((long long)m0) - 1 : (m1 ? 64 + __ffsll((long long)m1) - 1 : 128);
-                // probes before `first` are < key, probe `first` (if any) is >= key
-                int nlo = first == 0 ? lo : lo + (first - 1) * step + 1;
-                int nhi = first == 128 ? hi : lo + first * step;
-                if (nlo > hi) nlo = hi;
-                if (nhi > hi) nhi = hi;
-                s_lo[half] = nlo;
-                s_hi[half] = nhi;
-            }
-            __syncthreads();
-        }
-        if (t == 0) s_range[half] = s_lo[half];
-    }
-    __syncthreads();
-    const int lo = s_range[0], hi = s_range[1];
-    for (int s = lo + threadIdx.x; s < hi; s += 256) {
-        const int t = target_row[s];
-        s_targeted[t - t0] = 1;  // every writer stores the same value
-        const bool boundary = s > 0 && (s & ((1 << logW) - 1)) == 0 && target_row[s - 1] == t;  // continues across two wavefronts
-        const bool empty = rowPtr_split[s] == rowPtr_split[s + 1];
-        if (boundary || empty) s_added[t - t0] = 1;
-    }
-    __syncthreads();
-    if ((int)threadIdx.x < t1 - t0 && (!s_targeted[threadIdx.x] || s_added[threadIdx.x]))
-        s_list[atomicAdd(&s_count, 1)] = t0 + threadIdx.x;
-    __syncthreads();
-    const int count = s_count;
     const int lane = threadIdx.x & 63;
-    const size_t per_target = (size_t)nr * N, total = (size_t)rows_out * N;
-    const bool vec4 = (per_target & 3) == 0 && ((uintptr_t)Y & 15) == 0;
-    for (int i = threadIdx.x >> 6; i < count; i += 4) {
-        const size_t b0 = (size_t)s_list[i] * per_target;
-        const size_t b1 = min(total, b0 + per_target);  // the last target row may be cut by rows_out
-        if (vec4 && ((b1 - b0) & 3) == 0) {
-            const psp_f32x4 z = {0.f, 0.f, 0.f, 0.f};
-            for (size_t j = b0 + 4 * (size_t)lane; j < b1; j += 256) *(psp_f32x4 *)(Y + j) = z;
-        } else {
-            for (size_t j = b0 + lane; j < b1; j += 64) Y[j] = 0.0f;
+    const size_t per_target = (size_t)nr * N, total = (size_t)rows_out * N;  // the last target row may be cut by rows_out
+    const bool vec4 = (per_target & 3) == 0 && (total & 3) == 0 && ((uintptr_t)Y & 15) == 0;
+    if ((int)blockIdx.x < seg_blocks) {
+        // lane s < nseg: segment s; lane s == nseg: a virtual segment that targets the row past the last one, so that
+        // the untargeted rows at the end are the run in front of it
+        const int s = blockIdx.x * 256 + threadIdx.x;
+        const bool in = s < nseg;
+        const int t = in ? target_row[s] : ntargets;
+        const int tp = s == 0 ? -1 : (s <= nseg ? target_row[s - 1] : ntargets);
+        bool added = false;
+        if (in) {
+            const bool boundary = s > 0 && (s & ((1 << logW) - 1)) == 0 && tp == t;  // continues across two wavefronts
+            const bool empty = rowPtr_split[s] == rowPtr_split[s + 1];
+            added = boundary || empty;
         }
+        const int run = s <= nseg ? min(t - tp - 1, PSP_CLEAR_CAP) : 0;  // untargeted rows right in front of row t
+        unsigned long long m = __ballot(added);
+        while (m) {  // wave-uniform
+            const int b = __ffsll((long long)m) - 1;
+            m &= m - 1;
+            const size_t b0 = (size_t)__shfl(t, b) * per_target;
+            psp_wave_clear(Y, b0, min(total, b0 + per_target), lane, vec4);
+        }
+        m = __ballot(run > 0);
+        while (m) {
+            const int b = __ffsll((long long)m) - 1;
+            m &= m - 1;
+            const size_t b0 = (size_t)(__shfl(tp, b) + 1) * per_target;
+            psp_wave_clear(Y, b0, min(total, b0 + (size_t)__shfl(run, b) * per_target), lane, vec4);
+        }
+        return;
     }
+    const int u0 = (((int)blockIdx.x - seg_blocks) * 4 + (int)(threadIdx.x >> 6)) * PSP_CLEAR_CAP;
+    if (u0 >= ntargets) return;  // wave-uniform
+    int lo = 0, hi = nseg;  // target_row[i] < u0 for i < lo, >= u0 for i >= hi
+    while (lo < hi) {
+        const int step = (hi - lo + 63) >> 6;
+        const int i = lo + lane * step;
+        // probes are ascending and a probe past the range counts as >= u0: false up to some lane, true from there on
+        const bool ge = i >= hi || target_row[i] >= u0;
+        const unsigned long long m = __ballot(ge);
+        const int f = m ? __ffsll((long long)m) - 1 : 64;
+        const int nlo = f == 0 ? lo : lo + (f - 1) * step + 1;
+        const int nhi = f == 64 ? hi : lo + f * step;
+        lo = min(nlo, hi);
+        hi = min(nhi, hi);
+    }
+    const int tp = lo > 0 ? target_row[lo - 1] : -1;      // last targeted row in front of the block
+    const int tn = lo < nseg ? target_row[lo] : ntargets;  // first targeted row at or after the block's first row
+    const int r0 = max(u0, tp + 1 + PSP_CLEAR_CAP), r1 = min(min(u0 + PSP_CLEAR_CAP, tn), ntargets);
+    if (r0 < r1) psp_wave_clear(Y, (size_t)r0 * per_target, min(total, (size_t)r1 * per_target), lane, vec4);
 }
 
 int psp_split_clear(const int *rowPtr_split, const int *target_row, float *Y, int nseg, int N, int nr, int rows_out,
@@ -291,8 +287,10 @@ int psp_split_clear(const int *rowPtr_split, const int *target_row, float *Y, in
 {
     const int ntargets = (rows_out + nr - 1) / nr;
     if (ntargets == 0 || N == 0) return PSP_OK;
-    hipLaunchKernelGGL(psp_split_clear_kernel, dim3(psp_ceil_div(ntargets, PSP_CLEAR_ROWS)), dim3(256), 0, stream,
-                       rowPtr_split, target_row, Y, nseg, N, nr, rows_out, logW);
+    const int seg_blocks = nseg / 256 + 1;  // one lane more than there are segments
+    const int sweep_blocks = psp_ceil_div(ntargets, 4 * PSP_CLEAR_CAP);
+    hipLaunchKernelGGL(psp_split_clear_kernel, dim3(seg_blocks + sweep_blocks), dim3(256), 0, stream, rowPtr_split, target_row,
+                       Y, nseg, N, nr, rows_out, logW, seg_blocks);
     return psp_check_launch("split clear kernel");
 }
 

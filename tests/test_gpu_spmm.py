@@ -140,8 +140,9 @@ def selective_clear_always():
     _capi.set_option("split_clear_min", before)
 
 
+@pytest.mark.parametrize("long_runs", [False, True])
 @pytest.mark.parametrize("fmt", ["csr_split", "bcsr_split"])
-def test_split_selective_clear_path(oracle, fmt, selective_clear_always):
+def test_split_selective_clear_path(oracle, fmt, long_runs, selective_clear_always):
     """Large outputs of the row-split formats are not cleared as a whole: only rows shared by two wavefronts, rows
     of empty segments and rows without segments are.  Force that path on a small matrix with long rows, empty
     rows at the start, in the middle and at the end (runs of hundreds of rows nothing targets), and a poisoned Y."""
@@ -152,6 +153,10 @@ def test_split_selective_clear_path(oracle, fmt, selective_clear_always):
     k[:70] = 0
     k[-90:] = 0
     k[1000:1400] = 0
+    if long_runs:  # runs far beyond what the wavefront that finds them clears itself: the sweeping wavefronts take over
+        k[:600] = 0
+        k[1700:4800] = 0
+        k[-1100:] = 0
     keep = np.repeat(k > 0, np.diff(rowPtr))
     rowPtr = np.concatenate([[0], np.cumsum(k)]).astype(np.int32)
     colIdx, val = colIdx[keep], val[keep]
