@@ -547,6 +547,7 @@ def main():
         X, Y = Xs[d], Ys[d]
         a = (p(op.rowPtr), p(op.colIdx), p(op.val))
         nrows = op.rowPtr.numel() - 1
+        bw |= op.bw_flags  # the XCD stripe graph_input chose for this format
         if vec == 1 and not if_split:
             return lambda: L.psp_spmm_csr_f32(*a, p(X), p(Y), nrows, d, rows, cf, bw, stream)
         if vec == 1:
@@ -601,7 +602,9 @@ def main():
         # no-reuse gather volume: every stored entry fetches its row of X (what a matrix without locality moves)
         stored = F["nblk"] if fmt.startswith("bcsr") else nnz
         b_gather = b_alg - 4 * n * d + 4 * stored * d
-        per_dim.append({"dim": d, "format": fmt, "CF": cf, "config": sweep.cf_label(cf), "blkWarpNum": bw, "ms": round(ms, 5),
+        per_dim.append({"dim": d, "format": fmt, "CF": cf, "config": sweep.cf_label(cf), "blkWarpNum": bw,
+                        "xcd_stripe_rows": (ops[(1 if if_split else 0) + (2 if vec == 2 else 0)].bw_flags >> 12) * 256,
+                        "ms": round(ms, 5),
                         "gflops": round(2.0 * nnz * d / (ms * 1e-3) / 1e9, 1), "alg_bytes": b_alg,
                         "alg_GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
                         "gather_bytes": int(b_gather),

@@ -176,6 +176,14 @@ class pcsr_spmm(object):
         # Plain layouts of a graph with hub rows: the SDDMM divides the stored entries, not the rows, between its
         # wavefronts (every entry's result is independent).  "Hub rows" = a longest row of more than 64 times the
         # mean; arrays without statistics keep the row-wise walk.
+        # SpMM: rows dealt to one XCD at a time, from the format's distribution of entries (csr_data.xcd_stripe);
+        # travels in the flag bits of blkWarpNum
+        self.bw_flags = 0
+        if graph is not None:
+            from ._capi import bw_stripe
+
+            fmt = graph.csr_data if vec_size == 1 else graph.bcsr_data
+            self.bw_flags = bw_stripe(fmt.xcd_stripe(if_split))
         self.sddmm_balanced = False
         if graph is not None and not if_split:
             fmt = graph.csr_data if vec_size == 1 else graph.bcsr_data
@@ -202,7 +210,7 @@ class pcsr_spmm(object):
     def _spmm(self, X, val=None, CF=None, blkWarpNum=None):
         fn = getattr(SpMM, self._spmm_name())
         return fn(X, *self._sparse_args(val), self.CF if CF is None else CF,
-                  self.blkWarpNum if blkWarpNum is None else blkWarpNum)
+                  (self.blkWarpNum if blkWarpNum is None else blkWarpNum) | self.bw_flags)
 
     def _dense_input(self, dim, x):
         if x is None and dim is None:
@@ -259,7 +267,7 @@ class pcsr_spmm(object):
         if self.vec_size == 3:
             raise NotImplementedError("the fused GCN operators exist for vec_size 1 and 2 (SpCONV/SpCONV.cpp:498-511)")
         fn = getattr(SpCONV, _SPMM[self._key()] + "_forward")
-        return fn(H, w, *self._sparse_args(), self.CF, self.blkWarpNum)
+        return fn(H, w, *self._sparse_args(), self.CF, self.blkWarpNum | self.bw_flags)
 
     def backward(self, d_output, H, w):
         if d_output is None or H is None:
@@ -267,7 +275,7 @@ class pcsr_spmm(object):
         if self.vec_size == 3:
             raise NotImplementedError("the fused GCN operators exist for vec_size 1 and 2 (SpCONV/SpCONV.cpp:498-511)")
         fn = getattr(SpCONV, _SPMM[self._key()] + "_backward")
-        d_input, d_weight = fn(d_output, H, w, *self._sparse_args(), self.CF, self.blkWarpNum)
+        d_input, d_weight = fn(d_output, H, w, *self._sparse_args(), self.CF, self.blkWarpNum | self.bw_flags)
         return d_input, d_weight
 
     # ---- timing -----------------------------------------------------------------------------
@@ -279,7 +287,7 @@ class pcsr_spmm(object):
         args = self._sparse_args()
         if self.vec_size != 1:
             args.append(self.mtx_edges)  # blocked twins take the true nnz before CF
-        throughput = fn(X, *args, CF, blkWarpNum)
+        throughput = fn(X, *args, CF, blkWarpNum | self.bw_flags)
         if verbose:
             print("dim: {} gflops: {:.0f}".format(X.size(1), throughput))
         return throughput
@@ -316,8 +324,8 @@ class pcsr_spmm(object):
             raise NotImplementedError("time_ms covers the four decider formats; use cf_warpnum_profiling for 3x1 blocks")
         fmt = (1 if self.if_split else 0) + (2 if self.vec_size != 1 else 0)
         return SpMM.spmm_time_ms(fmt, X, self.rowPtr, self.colIdx, self.val, self.target_row,
-                                 self.CF if CF is None else CF, self.blkWarpNum if blkWarpNum is None else blkWarpNum,
-                                 warmup, iters)
+                                 self.CF if CF is None else CF,
+                                 (self.blkWarpNum if blkWarpNum is None else blkWarpNum) | self.bw_flags, warmup, iters)
 
 
 # ---- training-set construction: `python -m paramspmm_ae_amd.PCSR` (PCSR.py:660-871) -----------------------------

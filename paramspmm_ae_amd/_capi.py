@@ -32,6 +32,7 @@ class SpmmPlan(ctypes.Structure):
         ("waves_per_block", _i),
         ("log_segs_per_wave", _i),
         ("even_split", _i),
+        ("xcd_stripe_rows", _i),
     ]
 
     def as_dict(self):
@@ -144,6 +145,15 @@ def unpack_cf(CF):
         return None
     sel = (CF >> 8) & 7
     return (CF & 7) + 1, 1 << ((CF >> 3) & 7), 1 << ((CF >> 6) & 3), (1 << (sel - 1)) if sel else None, bool(CF & (1 << 11))
+
+
+def bw_stripe(rows):
+    """Flag bits for the SpMM operators' blkWarpNum argument (PSP_BW_STRIPE): deal ``rows`` consecutive rows (segments)
+    to one XCD at a time in this launch; 0 / None = the library option."""
+    rows = int(rows or 0)
+    if rows % 256 or not 0 <= rows <= 63 * 256:
+        raise ValueError("bw_stripe: a multiple of 256 up to 16128")
+    return (rows // 256) << 12
 
 
 def set_option(name, value):

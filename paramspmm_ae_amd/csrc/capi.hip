@@ -96,6 +96,8 @@ PSP_EXPORT int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *p
 {
     PSP_REQUIRE(plan != nullptr, "plan is null");
     PSP_REQUIRE(N >= 1, "feature dimension must be positive (got %d)", N);
+    const int stripe_rows = ((blkWarpNum & PSP_BW_STRIPE_MASK) >> PSP_BW_STRIPE_SHIFT) * 256;  // 0: the library option
+    blkWarpNum &= ~PSP_BW_STRIPE_MASK;
     PSP_REQUIRE(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8 (got %d)", blkWarpNum);
     const int V = (N % 4 == 0) ? 4 : (N % 2 == 0) ? 2 : 1;
     const int nvec = N / V;
@@ -133,6 +135,7 @@ PSP_EXPORT int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *p
     plan->waves_per_block = blkWarpNum;
     plan->log_segs_per_wave = logW;
     plan->even_split = (CF & PSP_CF_NATIVE) && (CF & PSP_CF_EVEN_SPLIT) ? 1 : 0;
+    plan->xcd_stripe_rows = stripe_rows;
     return PSP_OK;
 }
 

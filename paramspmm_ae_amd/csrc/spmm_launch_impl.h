@@ -67,7 +67,8 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
                         plan.vec, plan.unroll, softmax ? " (needs N % 4 == 0 and CF <= 4)" : "");
 
     const int align_pct = plan.even_split ? 0 : opt.align_pct;
-    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block), opt.stripe_rows / segs_per_block);
+    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block),
+                                      (plan.xcd_stripe_rows ? plan.xcd_stripe_rows : opt.stripe_rows) / segs_per_block);
     dim3 grid(g.launch, plan.col_tiles, 1), block(plan.waves_per_block * PSP_WAVE, 1, 1);
     hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.stripe, align_pct, row_max, row_sum);
     rc = psp_check_launch("spmm kernel");

@@ -266,6 +266,7 @@ static py::dict spmm_plan(int N, int CF, int blkWarpNum)
     d["waves_per_block"] = p.waves_per_block;
     d["log_segs_per_wave"] = p.log_segs_per_wave;
     d["even_split"] = p.even_split;
+    d["xcd_stripe_rows"] = p.xcd_stripe_rows;
     return d;
 }
 

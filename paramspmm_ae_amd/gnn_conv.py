@@ -17,7 +17,12 @@ def _conv_args(op):
     args = [op.rowPtr, op.colIdx, op.val]
     if op.if_split:
         args.append(op.target_row)
-    return args + [op.CF, op.blkWarpNum]
+    return args + [op.CF, _bw(op)]
+
+
+def _bw(op):
+    """blkWarpNum with the operator's launch flags (the XCD stripe chosen for its format, PCSR.pcsr_spmm.bw_flags)."""
+    return op.blkWarpNum | getattr(op, "bw_flags", 0)
 
 
 def _conv_name(op):
@@ -28,7 +33,7 @@ def _aggregate(op, D):
     """A D through ``op``'s format and configuration."""
     fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
     return SpCONV.aggregate(fmt, D, op.rowPtr, op.colIdx, op.val, op.target_row if op.if_split else None, op.CF,
-                            op.blkWarpNum)
+                            _bw(op))
 
 
 class _NllLossMean(torch.autograd.Function):
@@ -115,7 +120,7 @@ class GCNReLUInputFunction(torch.autograd.Function):
         op = ParamSpMM
         fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
         return SpCONV.relu_input_forward(fmt, Z, weight, op.rowPtr, op.colIdx, op.val,
-                                         op.target_row if op.if_split else None, op.CF, op.blkWarpNum)
+                                         op.target_row if op.if_split else None, op.CF, _bw(op))
 
     @staticmethod
     def backward(ctx, d_output):
@@ -123,7 +128,7 @@ class GCNReLUInputFunction(torch.autograd.Function):
         op = ctx.ParamSpMM
         fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
         d_input, d_weight = SpCONV.relu_input_backward(fmt, d_output.contiguous(), Z, weight, op.rowPtr, op.colIdx, op.val,
-                                                       op.target_row if op.if_split else None, op.CF, op.blkWarpNum)
+                                                       op.target_row if op.if_split else None, op.CF, _bw(op))
         return d_input, d_weight, None
 
 

@@ -20,6 +20,11 @@ import torch
 from . import _capi
 
 
+# candidates of csr_data.xcd_stripe, longest first (multiples of 256), and the XCD share it accepts
+XCD_STRIPES = (8192, 6144, 4096, 3072, 2048, 1536, 1024, 768, 512)
+XCD_IMBALANCE = 1.03
+
+
 def _stat_block(rowPtr, colIdx, num_nodes, num_edges):
     """Statistics of graph_input.py:60-87 with the reference's tensor types (int32 counts, fp32 moments,
     unbiased std)."""
@@ -77,6 +82,7 @@ class csr_data(object):
         self.rowPtr_split = None
         self.target_row = None
         self._dev = {}  # (attribute name, device) -> copy of that attribute on the device
+        self._xcd_stripe = {}  # split? -> result of xcd_stripe()
 
     def on_device(self, name, device):
         """The attribute ``name`` as a tensor on ``device``; uploaded once and kept (the device builders leave
@@ -96,6 +102,39 @@ class csr_data(object):
 
     def _keep_device(self, name, tensor):
         self._dev[(name, tensor.device)] = tensor
+
+    def xcd_stripe(self, split):
+        """Rows (segments when ``split``) the SpMM kernel should deal to one XCD at a time for this format: the
+        longest of XCD_STRIPES under which the eight XCDs get equal shares of the stored entries (largest share at
+        most XCD_IMBALANCE of the mean), else the best balanced one.  Long stripes keep neighbouring rows, and the X
+        rows they gather in common, in one L2; a matrix whose long rows cluster in an index range (an R-MAT graph,
+        a degree-sorted one) needs shorter ones or one XCD runs long after the others have finished.  Passed to the
+        operators as ``blkWarpNum | _capi.bw_stripe(rows)``; no counterpart in the reference (one L2 per GPU)."""
+        key = bool(split)
+        if key in self._xcd_stripe:
+            return self._xcd_stripe[key]
+        ptr = self.rowPtr_split if split else self.rowPtr
+        rows = 0
+        if ptr is not None and ptr.numel() > 1:
+            off = ptr.numpy().astype(np.int64)
+            total = float(off[-1] - off[0])
+            nseg = off.size - 1
+            best = None
+            for stripe in XCD_STRIPES:
+                if total <= 0 or nseg < 16 * stripe:  # fewer than two rounds of stripes: nothing to level
+                    continue
+                edges = off[np.minimum(np.arange(0, nseg + stripe, stripe), nseg)]
+                per_stripe = np.diff(edges)
+                share = np.bincount(np.arange(per_stripe.size) % 8, weights=per_stripe, minlength=8)
+                worst = share.max() * 8.0 / total
+                if worst <= XCD_IMBALANCE:
+                    best = (worst, stripe)
+                    break
+                if best is None or worst < best[0] - 1e-9:
+                    best = (worst, stripe)
+            rows = best[1] if best is not None else 0
+        self._xcd_stripe[key] = rows
+        return rows
 
     # graph_input.py:48-51
     def split_ratio_comp(self, split_granularity):

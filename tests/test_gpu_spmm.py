@@ -347,3 +347,31 @@ def test_spmm_native_configurations(oracle, fmt):
     for bad in (_capi.CF_NATIVE | (7 << 3), _capi.CF_NATIVE | (1 << 13), _capi.pack_cf(4, 8, 2) | (3 << 6),
                 _capi.CF_NATIVE | (2 << 6) | (1 << 3)):
         assert _capi.lib.psp_spmm_csr_f32(p(rp), None, None, p(x), p(x), 4, 16, 4, bad, 4, None) == -1
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_spmm_xcd_stripe_flag(oracle, fmt):
+    """blkWarpNum | PSP_BW_STRIPE(rows) only changes which workgroup takes which rows: plain layouts give the same
+    bits for every stripe, row-split ones agree with the oracle (their atomics add in launch order)."""
+    from gpu_util import Formats, spmm_capi, spmm_oracle, spmm_abs_scale, assert_close
+    from paramspmm_ae_amd import _capi
+
+    rowPtr, colIdx, val = random_csr(40013, 7, 5, empty_frac=0.05, hub=(31, 2500), values="normal")
+    F = Formats(oracle, rowPtr, colIdx, val)
+    for N in (16, 96):
+        X = np.random.default_rng(N).standard_normal((F.n + (F.n & 1), N)).astype(np.float32)
+        want = spmm_oracle(oracle, fmt, F, X)
+        scale = spmm_abs_scale(oracle, F, X, want.shape[0])
+        Xd = torch.from_numpy(X).cuda()
+        base = spmm_capi(fmt, F, Xd, 1, 4)
+        for rows in (256, 768, 1536, 6144, 16128):
+            print("case", fmt, N, rows, flush=True)
+            got = spmm_capi(fmt, F, Xd, 1, 4 | _capi.bw_stripe(rows))
+            torch.cuda.synchronize()
+            assert_close(got, want, what="%s N=%d stripe %d" % (fmt, N, rows), scale=scale)
+            if "split" not in fmt:
+                assert torch.equal(got, base)
+    p = _capi.ptr
+    x = torch.zeros(4, 16, device="cuda")
+    rp = torch.zeros(5, dtype=torch.int32, device="cuda")
+    assert _capi.lib.psp_spmm_csr_f32(p(rp), None, None, p(x), p(x), 4, 16, 4, 1, 4 | (1 << 18), None) == -1

@@ -52,6 +52,17 @@ def test_spmm_plan_mapping():
             p["even_split"]) == (2, 16, 4, 2, 1, 5, 1)
     assert _capi.spmm_plan(16, _capi.pack_cf(4, 8, 2), 4)["coarsen"] == 4
     assert _capi.spmm_plan(8, _capi.pack_cf(4, 8, 2), 4)["coarsen"] == 2
+    # per-launch XCD stripe in the flag bits of blkWarpNum
+    assert _capi.spmm_plan(64, 1, 4)["xcd_stripe_rows"] == 0
+    for rows in (256, 768, 6144, 16128):
+        p = _capi.spmm_plan(64, 2, 8 | _capi.bw_stripe(rows))
+        assert (p["xcd_stripe_rows"], p["waves_per_block"], p["coarsen"]) == (rows, 8, 2)
+    assert _capi.bw_stripe(0) == 0 and _capi.bw_stripe(None) == 0
+    for bad in (100, 16384, -256):
+        with pytest.raises(ValueError):
+            _capi.bw_stripe(bad)
+    with pytest.raises(_capi.ParamSpError):
+        _capi.spmm_plan(64, 1, 4 | (1 << 18))
     # options
     assert _capi.get_option("align_pct") == 50 and _capi.get_option("xcd_stripe_rows") == 8192
     _capi.set_option("align_pct", 25)
@@ -426,3 +437,39 @@ def test_reordering_restores_community_order_and_is_a_similarity_transform():
     rp, ci, v = synth.to_gcn_csr(r, c, n2)
     p2 = reorder.community_permutation(rp, ci, device="cpu")
     assert np.array_equal(np.sort(p2), np.arange(n2))
+
+
+def test_xcd_stripe_levels_a_matrix_whose_long_rows_cluster():
+    """csr_data.xcd_stripe: the longest candidate stripe under which the eight XCDs get equal shares of the entries.
+    Uniform rows keep the longest stripe; rows whose length follows the index bits of an R-MAT graph (every stripe
+    of 2^k rows lands on the same XCD with the same share) make it pick a candidate that is not a power of two, and
+    the share it reports is recomputed here by brute force."""
+    from paramspmm_ae_amd import graph_input as gi
+
+    n = 1 << 18
+
+    def fmt_of(deg):
+        rp = np.zeros(n + 1, np.int64)
+        np.cumsum(deg, out=rp[1:])
+        return gi.csr_data(rp.astype(np.int32), np.zeros(1, np.int32), np.zeros(1, np.float32), n, int(rp[-1]))
+
+    def worst_share(deg, stripe):
+        x = (np.arange(n) // stripe) % 8
+        share = np.bincount(x, weights=deg, minlength=8)
+        return share.max() * 8 / share.sum()
+
+    uniform = np.full(n, 5)
+    assert fmt_of(uniform).xcd_stripe(False) == gi.XCD_STRIPES[0] == 8192
+    # row length = product over the index bits, as in an R-MAT graph
+    idx = np.arange(n)
+    deg = np.ones(n)
+    for b in range(18):
+        deg *= np.where((idx >> b) & 1, 0.6, 1.4)
+    deg = np.maximum(1, np.round(deg * 8)).astype(np.int64)
+    pick = fmt_of(deg).xcd_stripe(False)
+    shares = {s: worst_share(deg, s) for s in gi.XCD_STRIPES}
+    assert shares[8192] > 1.5 and pick & (pick - 1) != 0  # no power-of-two stripe can level this matrix
+    assert shares[pick] <= min(shares.values()) + 1e-9 or shares[pick] <= gi.XCD_IMBALANCE
+    # an empty matrix and one too small for two rounds of stripes leave the choice to the library
+    small = gi.csr_data(np.arange(101, dtype=np.int32), np.zeros(100, np.int32), np.ones(100, np.float32), 100, 100)
+    assert small.xcd_stripe(False) == 0 and small.xcd_stripe(True) == 0
