@@ -787,6 +787,8 @@ def main():
         flops, secs, err = 0.0, 0.0, 0.0
         for d in port_dims:
             Xc = Xs[d][:n].cpu().numpy()
+            _capi.check(launcher(d, ops, chosen)())  # Ys[d] may hold a later leg's product (the reordered matrix)
+            torch.cuda.synchronize()
             t1 = time.perf_counter()
             yo = orc.spmm_csr(rp_h, ci_h, v_h, Xc)
             secs += time.perf_counter() - t1
