@@ -148,6 +148,42 @@ def bench_gather(args):
                       "config": {"workload": "%s gather ceiling" % args.graph, "nodes": n, "nnz": nnz}, "per_dim": table}))
 
 
+def bench_footprint(args):
+    """What the memory system delivers to a gather, as a function of the gathered footprint: 2^24 uniformly random row
+    indices in [0, F), rows of N floats fetched 128 bytes per 8-lane group (psp_probe_gather_f32), F from L2-resident
+    to far beyond the caches.  Gives the two rates an SpMM's gathers run between on this GPU: lines that hit the L2
+    and lines that come from HBM."""
+    import torch
+
+    from paramspmm_ae_amd import _capi
+
+    L, p = _capi.lib, _capi.ptr
+    nnz = 1 << 24
+    dims = [int(d) for d in args.dims.split(",")] if args.dims != DEFAULT_DIMS else [16, 32, 128]
+    stream = torch.cuda.current_stream().cuda_stream
+    gen = torch.Generator(device="cuda").manual_seed(1)
+    table = []
+    for N in dims:
+        lanes = min(8, N // 4)
+        for logF in range(13, 25):
+            F = 1 << logF
+            if F * N * 4 > (2 << 30):
+                break
+            X = torch.ones(F, N, device="cuda")
+            ci = torch.randint(0, F, (nnz,), device="cuda", dtype=torch.int32, generator=gen)
+            ms, unroll, per_wave = gather_probe_ms(ci, nnz, X, lanes)
+            tiles = (N // 4 + lanes - 1) // lanes
+            table.append({"dim": N, "rows": F, "footprint_MiB": round(F * N * 4 / 2 ** 20, 1), "ms": round(ms, 5),
+                          "gathered_GBps": round(4.0 * nnz * N / ms / 1e6, 1),
+                          "requests_per_ns": round(nnz * tiles / ms / 1e6, 2)})
+            del X, ci
+    print(json.dumps({"metric": "gather rate vs footprint (uniform random rows, 128-byte requests)", "unit": "GB/s",
+                      "value": table[-1]["gathered_GBps"], "n_gpus": 1, "steps": 5, "warmup": 1,
+                      "ms_per_step": table[-1]["ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+                      "dtype": "f32", "data": "synthetic",
+                      "config": {"workload": "gather rate vs footprint", "requests": nnz}, "table": table}))
+
+
 def bench_agnn(args):
     """Attention layers on the R-MAT pattern (BASELINE.json configs[3]): per layer e = A_e * <X_i, Y_j> on the
     stored entries (SDDMM, K = 32 and 64, rows L2-normalised), softmax over each row's entries, then SpMM with
@@ -449,10 +485,11 @@ def main():
                     help="spmm workload: permute rows and columns together at load time (paramspmm_ae_amd/reorder.py)")
     ap.add_argument("--no-extras", action="store_true",
                     help="skip what follows the timed region: decider check, gather ceiling, SDDMM and GCN legs")
-    ap.add_argument("--workload", choices=["spmm", "agnn", "gcn", "build", "sddmm", "gather"], default="spmm",
+    ap.add_argument("--workload", choices=["spmm", "agnn", "gcn", "build", "sddmm", "gather", "footprint"], default="spmm",
                     help="spmm: the headline width sweep; agnn: SDDMM -> row softmax -> SpMM attention layers; "
                          "gcn: GCN / GIN training epochs on the SBM graph; build: PCSR construction, host against device; "
-                         "sddmm: SDDMM width sweep over the four formats")
+                         "sddmm: SDDMM width sweep over the four formats; gather: the bare gathers of a pattern beside the kernel; "
+                         "footprint: gather rate of uniformly random rows against the gathered footprint")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU; --gpus %d is not supported (no multi-GPU path exists)" % args.gpus,
@@ -474,6 +511,8 @@ def main():
         return bench_sddmm(args)
     if args.workload == "gather":
         return bench_gather(args)
+    if args.workload == "footprint":
+        return bench_footprint(args)
     from paramspmm_ae_amd import _capi, synth, sweep
     from paramspmm_ae_amd.graph_input import graph_input
 
