@@ -194,7 +194,7 @@ def bench_agnn(args):
     import paramspmm_ae_amd  # noqa: F401
     import ParamSDDMM
     import ParamSpMM
-    from paramspmm_ae_amd import synth
+    from paramspmm_ae_amd import _capi, synth
 
     from paramspmm_ae_amd.decider import SpMMDecider
     from paramspmm_ae_amd.graph_input import graph_input
@@ -209,6 +209,7 @@ def bench_agnn(args):
     dec.gen_model_dict([32])
     if_split, _, CF, bw = dec.config_PCSR(g, 32)  # the edge values live in CSR order, so the CSR layouts are used
     c = g.csr_data
+    bw |= _capi.bw_stripe(c.xcd_stripe(bool(if_split)))  # the XCD stripe chosen for this format
     rp, ci, v = c.rowPtr.cuda(), c.colIdx.cuda(), c.val.cuda()
     rps, tr = c.rowPtr_split.cuda(), c.target_row.cuda()
     gen = torch.Generator(device="cuda").manual_seed(7)
@@ -278,7 +279,7 @@ def bench_sddmm(args):
 
     import paramspmm_ae_amd  # noqa: F401
     import ParamSDDMM
-    from paramspmm_ae_amd import synth
+    from paramspmm_ae_amd import _capi, synth
     from paramspmm_ae_amd.graph_input import graph_input
 
     rowPtr, colIdx, val, n = synth.config_graph(args.graph)
@@ -293,6 +294,7 @@ def bench_sddmm(args):
     nblk = Bf["colIdx"].numel()
     rows = (n + 1) // 2 * 2
     gen = torch.Generator(device="cuda").manual_seed(7)
+    stripe = [_capi.bw_stripe(f.xcd_stripe(sp)) for f, sp in ((c, False), (c, True), (b, False), (b, True))]
 
     def timed(fn):
         for _ in range(args.warmup):
@@ -312,10 +314,14 @@ def bench_sddmm(args):
         Bm = torch.randn(rows, K, device=dev, generator=gen)
         cands = {}
         for bw in (4, 8):
-            cands[("csr", bw)] = lambda bw=bw: ParamSDDMM.csr_sddmm(A, Bm, C["rowPtr"], C["colIdx"], C["val"], 1, bw)
-            cands[("csr_split", bw)] = lambda bw=bw: ParamSDDMM.csr_split_sddmm(A, Bm, C["rowPtr_split"], C["colIdx"], C["val"], C["target_row"], 1, bw)
-            cands[("bcsr", bw)] = lambda bw=bw: ParamSDDMM.bcsr_sddmm(A, Bm, Bf["rowPtr"], Bf["colIdx"], Bf["val"], 1, bw)
-            cands[("bcsr_split", bw)] = lambda bw=bw: ParamSDDMM.bcsr_split_sddmm(A, Bm, Bf["rowPtr_split"], Bf["colIdx"], Bf["val"], Bf["target_row"], 1, bw)
+            # each format with the XCD stripe graph_input chose for it (flag bits of blkWarpNum)
+            cands[("csr", bw)] = lambda bw=bw: ParamSDDMM.csr_sddmm(A, Bm, C["rowPtr"], C["colIdx"], C["val"], 1, bw | stripe[0])
+            cands[("csr_split", bw)] = lambda bw=bw: ParamSDDMM.csr_split_sddmm(A, Bm, C["rowPtr_split"], C["colIdx"], C["val"], C["target_row"], 1, bw | stripe[1])
+            # plain layouts with the entry-balanced walk (PSP_BW_BALANCED), what pcsr_spmm uses on a graph with hub rows
+            cands[("csr_balanced", bw)] = lambda bw=bw: ParamSDDMM.csr_sddmm(A, Bm, C["rowPtr"], C["colIdx"], C["val"], 1, bw | 0x100)
+            cands[("bcsr_balanced", bw)] = lambda bw=bw: ParamSDDMM.bcsr_sddmm(A, Bm, Bf["rowPtr"], Bf["colIdx"], Bf["val"], 1, bw | 0x100)
+            cands[("bcsr", bw)] = lambda bw=bw: ParamSDDMM.bcsr_sddmm(A, Bm, Bf["rowPtr"], Bf["colIdx"], Bf["val"], 1, bw | stripe[2])
+            cands[("bcsr_split", bw)] = lambda bw=bw: ParamSDDMM.bcsr_split_sddmm(A, Bm, Bf["rowPtr_split"], Bf["colIdx"], Bf["val"], Bf["target_row"], 1, bw | stripe[3])
         times = {k: timed(f) for k, f in cands.items()}
         (fmt, bw), ms = min(times.items(), key=lambda kv: kv[1])
         if fmt.startswith("bcsr"):
@@ -723,10 +729,10 @@ def main():
         cs_, bs_ = ops[1], ops[3]
         sd = {}
         for bw in (4, 8):
-            sd[("csr", bw)] = lambda bw=bw: ParamSDDMM.csr_sddmm(A, Bm, c_.rowPtr, c_.colIdx, c_.val, 2, bw)
-            sd[("csr_split", bw)] = lambda bw=bw: ParamSDDMM.csr_split_sddmm(A, Bm, cs_.rowPtr, cs_.colIdx, cs_.val, cs_.target_row, 2, bw)
-            sd[("bcsr", bw)] = lambda bw=bw: ParamSDDMM.bcsr_sddmm(A, Bm, b_.rowPtr, b_.colIdx, b_.val, 2, bw)
-            sd[("bcsr_split", bw)] = lambda bw=bw: ParamSDDMM.bcsr_split_sddmm(A, Bm, bs_.rowPtr, bs_.colIdx, bs_.val, bs_.target_row, 2, bw)
+            sd[("csr", bw)] = lambda bw=bw: ParamSDDMM.csr_sddmm(A, Bm, c_.rowPtr, c_.colIdx, c_.val, 2, bw | c_.bw_flags)
+            sd[("csr_split", bw)] = lambda bw=bw: ParamSDDMM.csr_split_sddmm(A, Bm, cs_.rowPtr, cs_.colIdx, cs_.val, cs_.target_row, 2, bw | cs_.bw_flags)
+            sd[("bcsr", bw)] = lambda bw=bw: ParamSDDMM.bcsr_sddmm(A, Bm, b_.rowPtr, b_.colIdx, b_.val, 2, bw | b_.bw_flags)
+            sd[("bcsr_split", bw)] = lambda bw=bw: ParamSDDMM.bcsr_split_sddmm(A, Bm, bs_.rowPtr, bs_.colIdx, bs_.val, bs_.target_row, 2, bw | bs_.bw_flags)
         sd_ms = {}
         for key, fn in sd.items():
             fn()

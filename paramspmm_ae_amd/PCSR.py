@@ -245,7 +245,7 @@ class pcsr_spmm(object):
         CF = (A.size(1) + 31) // 32
         if self.sddmm_balanced and not self.if_split:
             blkWarpNum |= 0x100  # PSP_BW_BALANCED: divide the entries, not the rows, between the wavefronts
-        return fn(A, B, *self._sparse_args(), CF, blkWarpNum)
+        return fn(A, B, *self._sparse_args(), CF, blkWarpNum | self.bw_flags)
 
     def AGNN_sddmm(self, A):
         """Per stored entry <A[row], A[col]>; for 2x1 blocks the result is [nblk, 2] (PCSR.py:290-320)."""

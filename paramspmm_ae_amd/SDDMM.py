@@ -63,7 +63,7 @@ class pcsr_sddmm(pcsr_spmm):
         (SDDMM.py:119-156).  CF = ceil(dim / 32) as in the reference."""
         assert torch.cuda.is_available()
         A, B = self._ones(dim)
-        self.result = self._operator()(A, B, *self._sparse_args(), (dim + 31) // 32, blkWarpNum).to("cpu")
+        self.result = self._operator()(A, B, *self._sparse_args(), (dim + 31) // 32, blkWarpNum | self.bw_flags).to("cpu")
         return self.result
 
     def profiling(self, blkWarpNum, dim, verbose=True):
@@ -73,7 +73,7 @@ class pcsr_sddmm(pcsr_spmm):
         args = self._sparse_args()
         if self.vec_size != 1:
             args.append(self.mtx_edges)
-        throughput = self._operator("_profile")(A, B, *args, (dim + 31) // 32, blkWarpNum)
+        throughput = self._operator("_profile")(A, B, *args, (dim + 31) // 32, blkWarpNum | self.bw_flags)
         if verbose:
             print("dim: {} gflops: {:.0f}".format(dim, throughput))
         return throughput

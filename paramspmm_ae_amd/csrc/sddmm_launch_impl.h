@@ -10,6 +10,8 @@ int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, con
     constexpr bool BCSR = NR > 1;
     const bool balanced = !SPLIT && (blkWarpNum & PSP_BW_BALANCED) != 0;  // plain layouts only; row-split input is balanced
     blkWarpNum &= ~PSP_BW_BALANCED;
+    const int stripe_flag = ((blkWarpNum & PSP_BW_STRIPE_MASK) >> PSP_BW_STRIPE_SHIFT) * 256;  // 0: the library option
+    blkWarpNum &= ~PSP_BW_STRIPE_MASK;
     PSP_REQUIRE(blkWarpNum == 4 || blkWarpNum == 8, "blkWarpNum must be 4 or 8");
     PSP_REQUIRE(nrows >= 0 && K >= 1, "sddmm: bad size (rows %d, K %d)", nrows, K);
     if (nrows == 0) return PSP_OK;
@@ -55,7 +57,7 @@ int psp_sddmm_launch(const int *rowPtr, const int *colIdx, const float *val, con
     while (logW > 0 && (nrows >> logW) < 4096) logW--;
     if (logW < logR - 1) logW = logR - 1;
     const int segs_per_block = blkWarpNum << logW;
-    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block), psp_stripe_rows() / segs_per_block);
+    const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block), (stripe_flag ? stripe_flag : psp_stripe_rows()) / segs_per_block);
     dim3 grid(g.launch, 1, 1), block(blkWarpNum * PSP_WAVE, 1, 1);
     hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, BCSR ? val : scale, target_row, A, B, out, nrows, K,
                        logW, g.real, g.stripe, row_max);

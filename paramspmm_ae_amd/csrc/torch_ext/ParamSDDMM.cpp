@@ -35,7 +35,7 @@ static void check_sddmm_args(int fmt, const Tensor &A, const Tensor &B, const Te
     // the reference dispatches CF 1..4 only (SDDMM/sddmm.cpp:31-43); wider K is accepted here, CF stays a
     // checked argument so that a caller's mistake still surfaces
     TORCH_CHECK(CF >= 1 && CF <= 8, "CF must be 1..8");
-    TORCH_CHECK((blkWarpNum & ~PSP_BW_BALANCED) == 4 || (blkWarpNum & ~PSP_BW_BALANCED) == 8, "blkWarpNum must be 4 or 8");
+    TORCH_CHECK((blkWarpNum & ~(PSP_BW_BALANCED | PSP_BW_STRIPE_MASK)) == 4 || (blkWarpNum & ~(PSP_BW_BALANCED | PSP_BW_STRIPE_MASK)) == 8, "blkWarpNum must be 4 or 8");
     const long rows = rowPtr.size(0) - 1;
     if (target_row) {
         need_gpu(*target_row, "target_row");
@@ -246,7 +246,7 @@ static void check_vec_sddmm_args(const Tensor &A, const Tensor &B, const Tensor 
     same_device(A, colIdx, "vec_sddmm");
     same_device(A, values, "vec_sddmm");
     TORCH_CHECK(CF >= 1 && CF <= 8, "CF must be 1..8");
-    TORCH_CHECK((blkWarpNum & ~PSP_BW_BALANCED) == 4 || (blkWarpNum & ~PSP_BW_BALANCED) == 8, "blkWarpNum must be 4 or 8");
+    TORCH_CHECK((blkWarpNum & ~(PSP_BW_BALANCED | PSP_BW_STRIPE_MASK)) == 4 || (blkWarpNum & ~(PSP_BW_BALANCED | PSP_BW_STRIPE_MASK)) == 8, "blkWarpNum must be 4 or 8");
     if (target_row) {
         need_gpu(*target_row, "target_row");
         need_i32(*target_row, "target_row");

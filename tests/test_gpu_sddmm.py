@@ -357,3 +357,24 @@ def test_sddmm_entry_balanced_walk_structures(oracle, fmt):
                 got = sddmm_capi(fmt, F, torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda(), bw)
                 torch.cuda.synchronize()
                 assert_close(got, want, what="%s %s K=%d balanced" % (fmt, name, K))
+
+
+@pytest.mark.parametrize("fmt", FMTS)
+def test_sddmm_xcd_stripe_flag(oracle, fmt):
+    """blkWarpNum | PSP_BW_STRIPE(rows) only changes which workgroup takes which rows: every entry's result keeps
+    its bits, with the row-wise and with the entry-balanced walk."""
+    from gpu_util import Formats, sddmm_capi
+    from paramspmm_ae_amd import _capi
+
+    rowPtr, colIdx, val = random_csr(40013, 7, 5, empty_frac=0.05, hub=(31, 2500), values="normal")
+    F = Formats(oracle, rowPtr, colIdx, val)
+    for K in (16, 96):
+        A = torch.from_numpy(unit_rows(F.n + (F.n & 1), K, K)).cuda()
+        B = torch.from_numpy(unit_rows(F.n, K, K + 1)).cuda()
+        base = sddmm_capi(fmt, F, A, B, 4)
+        for rows in (256, 1536, 6144, 16128):
+            for bw in (4, 8 | 0x100):
+                print("case", fmt, K, rows, bw, flush=True)
+                got = sddmm_capi(fmt, F, A, B, bw | _capi.bw_stripe(rows))
+                torch.cuda.synchronize()
+                assert torch.equal(got, base)
