@@ -317,8 +317,10 @@ int psp_gemm_atb_ws_act_f32(const float *A, const float *B, float *C, long long 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: Y[n,K2] = X[n,K1] * W (transW = 0, W is [K1,K2] row-major) or X * W^T (transW != 0, W is [K2,K1]) for
  * tall-skinny X and a small weight matrix: torch::mm(H, W) and torch::mm(AG, W.t()) of the fused GCN layer
- * (SpCONV/SpCONV.h:43-71).  Supported widths: K2 in {16, 32}, K1 in {16, 32, 48, 64} (and 128 with K2 = 16);
- * psp_gemm_xw_supported tells.  Y is overwritten; X and Y 16-byte aligned.  Deterministic (one lane per row).
+ * (SpCONV/SpCONV.h:43-71).  Supported widths: K2 in {16, 32} with K1 in {16, 32, 48, 64} (and 128 with K2 = 16): one
+ * lane per row, FMAs; K2 in {64, 128} with K1 in {16, 32, 64, 128}: fp32 matrix cores (v_mfma_f32_16x16x4_f32), W in
+ * LDS.  psp_gemm_xw_supported tells.  Y is overwritten; X and Y 16-byte aligned.  Deterministic (no atomics, one
+ * fixed summation order per output element).
  * ------------------------------------------------------------------------------------------- */
 int psp_gemm_xw_supported(int K1, int K2);
 int psp_gemm_xw_f32(const float *X, const float *W, float *Y, long long n, int K1, int K2, int transW,

@@ -70,7 +70,15 @@ static psp_xw_kernel_t xw_lookup(int K1, int K2, bool trans, bool relu_x, bool m
     return nullptr;
 }
 
-PSP_EXPORT int psp_gemm_xw_supported(int K1, int K2) { return xw_lookup(K1, K2, false, false, false) != nullptr; }
+// dense_xw_wide.hip: 64 and 128 output columns on the matrix cores
+bool psp_xw_wide_supported(int K1, int K2);
+int psp_xw_wide_launch(const float *X, const float *W, float *Y, long long n, int K1, int K2, int transW, int relu_x,
+                       const float *mask, hipStream_t stream);
+
+PSP_EXPORT int psp_gemm_xw_supported(int K1, int K2)
+{
+    return xw_lookup(K1, K2, false, false, false) != nullptr || psp_xw_wide_supported(K1, K2);
+}
 
 PSP_EXPORT int psp_gemm_xw_act_f32(const float *X, const float *W, float *Y, long long n, int K1, int K2, int transW,
                                    int relu_x, const float *mask, psp_stream_t stream)
@@ -79,11 +87,13 @@ PSP_EXPORT int psp_gemm_xw_act_f32(const float *X, const float *W, float *Y, lon
     PSP_REQUIRE(!(transW && relu_x), "gemm_xw: the activation on X exists for the plain product only");
     PSP_REQUIRE(!(!transW && mask), "gemm_xw: the output mask exists for the transposed product only");
     psp_xw_kernel_t k = xw_lookup(K1, K2, transW != 0, relu_x != 0, mask != nullptr);
-    PSP_REQUIRE(k != nullptr, "gemm_xw: unsupported widths %d x %d (see psp_gemm_xw_supported)", K1, K2);
+    const bool wide = k == nullptr && psp_xw_wide_supported(K1, K2);
+    PSP_REQUIRE(k != nullptr || wide, "gemm_xw: unsupported widths %d x %d (see psp_gemm_xw_supported)", K1, K2);
     if (n == 0) return PSP_OK;
     PSP_REQUIRE(X && W && Y, "gemm_xw: null pointer");
     PSP_REQUIRE((((size_t)X | (size_t)Y | (size_t)mask) & 15) == 0, "gemm_xw: X, Y and mask must be 16-byte aligned");
     PSP_REQUIRE((n + 255) / 256 <= 0x7fffffffLL, "gemm_xw: too many rows");
+    if (wide) return psp_xw_wide_launch(X, W, Y, n, K1, K2, transW, relu_x, mask, (hipStream_t)stream);
     hipLaunchKernelGGL(k, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, (hipStream_t)stream, X, W, Y, n, mask);
     return psp_check_launch("gemm_xw kernel");
 }

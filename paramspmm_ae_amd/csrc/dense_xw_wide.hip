@@ -1,0 +1,168 @@
+// Y[n,K2] = X[n,K1] * W  or  X * W^T  for tall-skinny X and a weight matrix of 64 or 128 output columns: the dense
+// products of the wide GCN / GIN layers (torch::mm(H, W) and torch::mm(AG, W.t()) in SpCONV/SpCONV.h:43-71), with the
+// ReLU between two layers folded in like the narrow kernel of dense_xw.hip does.  At 128 x 128 the product is 32 kflop
+// per row against 1 KB of traffic: matrix-core time and memory time are about equal, so this one runs on the matrix
+// cores (v_mfma_f32_16x16x4_f32, fp32 in, fp32 accumulate).
+//
+// The product is formed transposed, Y^T = W^T X^T, so that a lane ends up with consecutive elements of one output row:
+//   * MFMA operand B (4 x 16) is a piece of X^T: lane (r, q) = (lane % 16, lane / 16) supplies X[row r][k]; it loads
+//     its row 16 bytes at a time, float4 t covering columns 16t + 4q .. 16t + 4q + 3, so the four q-lanes of a row
+//     read 64 contiguous bytes.  Element e of float4 t is used in contraction step (t, e), where the lane's column
+//     16t + 4q + e stands for index k = q of the instruction: which four columns a step contracts is free as long as
+//     operand A follows the same rule;
+//   * operand A (16 x 4) is a piece of W^T read from LDS: lane (r, q) supplies W[16t + 4q + e][16j + r] for column
+//     tile j (T = K2 / 16 tiles).  LDS holds the columns of W permuted, column 16j + r at position r * T + j, so a
+//     lane's T tiles are T consecutive floats: two 16-byte LDS reads per step serve eight MFMAs (sixteen with the two
+//     row blocks a wavefront works on);
+//   * result lane (r, q), tile j, element i is Y[row r][16j + 4q + i]: one 16-byte store per tile, the four q-lanes
+//     of a row writing 64 contiguous bytes.
+// W (at most 64 KB) is staged into LDS once per workgroup, transposed on the way in for the X * W^T form; the grid is
+// sized to the GPU and every wavefront walks blocks of 32 rows with the next block's loads in flight.
+#include "psp_common.h"
+
+typedef float psp_f32x4 __attribute__((ext_vector_type(4)));
+
+#define XWW_ROWS 32  // rows per wavefront and step: two MFMA row blocks share every operand read from LDS
+
+template <int K1, int K2, bool RELU_X, bool MASK>
+// (the bound of 512 lanes leaves the register allocator 256 registers per lane; launched with 256)
+__global__ void __launch_bounds__(512)
+psp_xw_wide_kernel(const float *__restrict__ X, const float *__restrict__ W, float *__restrict__ Y, long long n,
+                   const float *__restrict__ mask, int transW, long long nblocks)
+{
+    constexpr int T = K2 / 16;   // column tiles
+    constexpr int KT = K1 / 16;  // float4 loads per lane and row block
+    constexpr int S = K2 + 4;    // LDS row stride: the four k-rows a step reads fall into different bank halves
+    static_assert(T % 4 == 0 && K1 % 16 == 0, "widths: K2 a multiple of 64, K1 a multiple of 16");  // T % 4: 16-byte LDS reads
+    __shared__ float Ws[K1 * S];
+
+    for (int idx = threadIdx.x; idx < K1 * K2; idx += blockDim.x) {
+        int k, c;
+        if (transW) {  // W is [K2, K1]
+            c = idx / K1;
+            k = idx - c * K1;
+        } else {  // W is [K1, K2]
+            k = idx / K2;
+            c = idx - k * K2;
+        }
+        Ws[k * S + (c & 15) * T + (c >> 4)] = W[idx];
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const int waves = blockDim.x >> 6;
+    const long long stride = (long long)gridDim.x * waves;
+    long long blk = (long long)blockIdx.x * waves + wave;
+    if (blk >= nblocks) return;
+
+    psp_f32x4 xa[2][KT], xb[2][KT];
+    auto load_block = [&](long long b, psp_f32x4 (&x)[2][KT]) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            long long row = b * XWW_ROWS + 16 * h + r;
+            if (row >= n) row = n - 1;  // loaded and computed, never stored
+            const psp_f32x4 *xr = (const psp_f32x4 *)(X + row * K1) + q;
+#pragma unroll
+            for (int t = 0; t < KT; t++) x[h][t] = xr[4 * t];
+        }
+    };
+    auto compute_block = [&](long long b, psp_f32x4 (&x)[2][KT]) {
+        if constexpr (RELU_X) {
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int t = 0; t < KT; t++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) x[h][t][e] = x[h][t][e] < 0.0f ? 0.0f : x[h][t][e];  // NaN stays NaN
+        }
+        psp_f32x4 acc[2][T];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int j = 0; j < T; j++) acc[h][j] = psp_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < KT; t++) {
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const psp_f32x4 *wr = (const psp_f32x4 *)(Ws + (16 * t + 4 * q + e) * S + r * T);
+                psp_f32x4 a4[T / 4];
+#pragma unroll
+                for (int v = 0; v < T / 4; v++) a4[v] = wr[v];
+#pragma unroll
+                for (int j = 0; j < T; j++) {
+#pragma unroll
+                    for (int h = 0; h < 2; h++)
+                        acc[h][j] = __builtin_amdgcn_mfma_f32_16x16x4f32(a4[j / 4][j % 4], x[h][t][e], acc[h][j], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const long long row = b * XWW_ROWS + 16 * h + r;
+            if (row >= n) continue;
+            psp_f32x4 *yr = (psp_f32x4 *)(Y + row * K2) + q;
+            const psp_f32x4 *mr = (const psp_f32x4 *)(mask + row * K2) + q;
+#pragma unroll
+            for (int j = 0; j < T; j++) {
+                psp_f32x4 o = acc[h][j];
+                if constexpr (MASK) {
+                    const psp_f32x4 m = mr[4 * j];
+#pragma unroll
+                    for (int c = 0; c < 4; c++) o[c] = m[c] > 0.0f ? o[c] : 0.0f;
+                }
+                yr[4 * j] = o;
+            }
+        }
+    };
+
+    // two register sets alternate: the next block's rows are requested before the current block is multiplied
+    load_block(blk, xa);
+    while (true) {
+        long long nxt = blk + stride;
+        if (nxt < nblocks) load_block(nxt, xb);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_block(blk, xa);
+        if (nxt >= nblocks) break;
+        blk = nxt;
+        nxt = blk + stride;
+        if (nxt < nblocks) load_block(nxt, xa);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_block(blk, xb);
+        if (nxt >= nblocks) break;
+        blk = nxt;
+    }
+}
+
+typedef void (*psp_xw_wide_kernel_t)(const float *, const float *, float *, long long, const float *, int, long long);
+
+static psp_xw_wide_kernel_t xw_wide_lookup(int K1, int K2, bool relu_x, bool mask)
+{
+#define XWW_CASE(A_, B_)                                                   \
+    if (K1 == A_ && K2 == B_) {                                            \
+        if (mask) return psp_xw_wide_kernel<A_, B_, false, true>;          \
+        return relu_x ? psp_xw_wide_kernel<A_, B_, true, false> : psp_xw_wide_kernel<A_, B_, false, false>; \
+    }
+    XWW_CASE(16, 64) XWW_CASE(32, 64) XWW_CASE(64, 64) XWW_CASE(128, 64)
+    XWW_CASE(16, 128) XWW_CASE(32, 128) XWW_CASE(64, 128) XWW_CASE(128, 128)
+#undef XWW_CASE
+    return nullptr;
+}
+
+bool psp_xw_wide_supported(int K1, int K2) { return xw_wide_lookup(K1, K2, false, false) != nullptr; }
+
+// called by psp_gemm_xw_act_f32 for the widths the one-lane-per-row kernel does not cover; arguments are checked there
+int psp_xw_wide_launch(const float *X, const float *W, float *Y, long long n, int K1, int K2, int transW, int relu_x,
+                       const float *mask, hipStream_t stream)
+{
+    psp_xw_wide_kernel_t k = xw_wide_lookup(K1, K2, relu_x != 0, mask != nullptr);
+    if (!k) return psp_fail(PSP_ERR_ARG, "gemm_xw: unsupported widths %d x %d", K1, K2);
+    const long long nblocks = (n + XWW_ROWS - 1) / XWW_ROWS;
+    // 4 wavefronts per workgroup, two workgroups per CU (two copies of W in LDS side by side); measured against 6 and 8
+    // wavefronts per workgroup and one to four workgroups per CU at 10^6 rows: nothing faster
+    const int waves = 4;
+    const long long want = (nblocks + waves - 1) / waves;
+    const int grid = (int)(want < 512 ? want : 512);
+    hipLaunchKernelGGL(k, dim3(grid), dim3(64 * waves), 0, stream, X, W, Y, n, mask, transW, nblocks);
+    return psp_check_launch("gemm_xw wide kernel");
+}

@@ -202,7 +202,8 @@ def test_gcn_and_gin_layers_match_dense_autograd(vec, split):
 
 
 @pytest.mark.parametrize("vec,split", VARIANTS)
-@pytest.mark.parametrize("n,width_in,width_out", [(300, 24, 40), (20000, 32, 16), (20000, 16, 32), (17000, 128, 16), (16400, 128, 128)])
+@pytest.mark.parametrize("n,width_in,width_out", [(300, 24, 40), (20000, 32, 16), (20000, 16, 32), (17000, 128, 16), (16400, 128, 128),
+                                                  (16411, 64, 64), (16411, 32, 128)])
 def test_gcn_layer_with_relu_on_its_input(vec, split, n, width_in, width_out):
     """A (relu(Z) W) as one function of Z against PyTorch autograd of the same expression (torch.sparse.mm): small
     graphs and unsupported widths take the PyTorch path, 16384 rows and more with widths the library covers run the
@@ -505,10 +506,12 @@ def test_gin_backward_accepts_a_gradient_view():
 
 
 @pytest.mark.parametrize("K1,K2", [(16, 16), (32, 16), (48, 16), (64, 16), (128, 16), (16, 32), (32, 32), (48, 32), (64, 32),
-                                   (24, 16), (128, 128)])
+                                   (24, 16), (96, 96), (16, 64), (32, 64), (64, 64), (128, 64), (16, 128), (32, 128),
+                                   (64, 128), (128, 128)])
 def test_dense_xw_matches_torch(K1, K2):
-    """X*W and X*W^T of the layers through the one-lane-per-row kernel (supported widths) or torch::mm (the last two
-    shapes), against a float64 product; a row count that is not a multiple of the workgroup size."""
+    """X*W and X*W^T of the layers through the one-lane-per-row kernel (16 / 32 output columns), the matrix-core
+    kernel (64 / 128 output columns) or torch::mm (24 x 16, 96 x 96), against a float64 product; a row count that is
+    not a multiple of the workgroup size."""
     import ParamSpCONV
 
     n = 100_003
@@ -639,3 +642,39 @@ def test_weight_gradient_product_small_row_counts(n, K1, K2):
         else:
             _capi.check(_capi.lib.psp_gemm_atb_f32(p(A), p(B), p(C), n, K1, K2, st))
         torch.testing.assert_close(C.double(), want, rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("K1,K2", [(16, 64), (64, 64), (128, 64), (32, 128), (128, 128)])
+@pytest.mark.parametrize("n", [1, 33, 70_001])
+def test_wide_dense_products_with_the_activation_folded_in(K1, K2, n):
+    """psp_gemm_xw_act_f32 on the matrix-core kernel through the C ABI: max(X, 0) W and (X W^T) masked by Z > 0 against
+    float64, at row counts around the 32-row blocks; masked elements are exact zeros, NaN inputs stay in their rows."""
+    from paramspmm_ae_amd import _capi
+
+    L, p = _capi.lib, _capi.ptr
+    assert L.psp_gemm_xw_supported(K1, K2) == 1
+    g = torch.Generator(device="cuda").manual_seed(n + K1 + 7 * K2)
+    X = torch.randn(n, K1, device="cuda", generator=g)
+    W = torch.randn(K1, K2, device="cuda", generator=g)
+    Z = torch.randn(n, K2, device="cuda", generator=g)
+    st = torch.cuda.current_stream().cuda_stream
+    Y = torch.full((n, K2), float("nan"), device="cuda")
+    _capi.check(L.psp_gemm_xw_act_f32(p(X), p(W), p(Y), n, K1, K2, 0, 1, None, st))
+    want = torch.relu(X).double() @ W.double()
+    scale = torch.relu(X).double() @ W.abs().double()
+    assert torch.all((Y.double() - want).abs() <= 1e-5 * scale + 1e-6)
+    Wt = W.t().contiguous()
+    Y2 = torch.full((n, K2), float("nan"), device="cuda")
+    _capi.check(L.psp_gemm_xw_act_f32(p(X), p(Wt), p(Y2), n, K1, K2, 1, 0, p(Z), st))
+    want2 = (X.double() @ W.double()) * (Z > 0)
+    assert torch.all((Y2.double() - want2).abs() <= 1e-5 * (X.abs().double() @ W.abs().double()) + 1e-6)
+    assert bool((Y2[Z <= 0] == 0).all())
+    if n > 40:
+        Xn = X.clone()
+        Xn[17, 3] = float("nan")
+        _capi.check(L.psp_gemm_xw_act_f32(p(Xn), p(W), p(Y), n, K1, K2, 0, 0, None, st))
+        bad = torch.isnan(Y).any(dim=1)
+        assert bool(bad[17]) and int(bad.sum()) == 1
+    # the two fused forms are exclusive, as for the narrow kernel
+    assert L.psp_gemm_xw_act_f32(p(X), p(W), p(Y), n, K1, K2, 1, 1, None, st) == -1
+    assert L.psp_gemm_xw_act_f32(p(X), p(W), p(Y), n, K1, K2, 0, 0, p(Z), st) == -1
