@@ -65,13 +65,13 @@ typedef struct psp_spmm_plan {
 int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan);
 
 /* SpMM and SDDMM entry points (row-wise walks), blkWarpNum | PSP_BW_STRIPE(rows): this launch deals `rows` consecutive rows (segments, block-rows)
- * to one XCD at a time instead of the library option "xcd_stripe_rows".  rows = a multiple of 256 up to 16128 (the field
- * holds rows / 256 in bits 12..17; 0 = the option).  The reference has no counterpart (one L2 on its GPUs): a caller
+ * to one XCD at a time instead of the library option "xcd_stripe_rows".  rows = a multiple of 256 up to 65280 (the field
+ * holds rows / 256 in bits 12..19; 0 = the option).  The reference has no counterpart (one L2 on its GPUs): a caller
  * that knows the matrix picks the longest stripe that still gives the eight XCDs equal shares of the stored entries
  * (graph_input does: csr_data.xcd_stripe), long stripes keeping neighbouring rows -- and the X rows they share -- in
  * one L2, short ones levelling a matrix whose long rows cluster in an index range. */
 #define PSP_BW_STRIPE_SHIFT 12
-#define PSP_BW_STRIPE_MASK (0x3f << PSP_BW_STRIPE_SHIFT)
+#define PSP_BW_STRIPE_MASK (0xff << PSP_BW_STRIPE_SHIFT)
 #define PSP_BW_STRIPE(rows) ((((rows) / 256) << PSP_BW_STRIPE_SHIFT) & PSP_BW_STRIPE_MASK)
 
 /* Library-wide tuning options (no counterpart in the reference, whose launch shapes are compile-time constants):

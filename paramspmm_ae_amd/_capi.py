@@ -151,8 +151,8 @@ def bw_stripe(rows):
     """Flag bits for the SpMM operators' blkWarpNum argument (PSP_BW_STRIPE): deal ``rows`` consecutive rows (segments)
     to one XCD at a time in this launch; 0 / None = the library option."""
     rows = int(rows or 0)
-    if rows % 256 or not 0 <= rows <= 63 * 256:
-        raise ValueError("bw_stripe: a multiple of 256 up to 16128")
+    if rows % 256 or not 0 <= rows <= 255 * 256:
+        raise ValueError("bw_stripe: a multiple of 256 up to 65280")
     return (rows // 256) << 12
 
 

@@ -21,7 +21,7 @@ from . import _capi
 
 
 # candidates of csr_data.xcd_stripe, longest first (multiples of 256), and the XCD share it accepts
-XCD_STRIPES = (8192, 6144, 4096, 3072, 2048, 1536, 1024, 768, 512)
+XCD_STRIPES = (32768, 16384, 8192, 6144, 4096, 3072, 2048, 1536, 1024, 768, 512)
 XCD_IMBALANCE = 1.03
 
 

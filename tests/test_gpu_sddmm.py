@@ -372,7 +372,7 @@ def test_sddmm_xcd_stripe_flag(oracle, fmt):
         A = torch.from_numpy(unit_rows(F.n + (F.n & 1), K, K)).cuda()
         B = torch.from_numpy(unit_rows(F.n, K, K + 1)).cuda()
         base = sddmm_capi(fmt, F, A, B, 4)
-        for rows in (256, 1536, 6144, 16128):
+        for rows in (256, 1536, 6144, 65280):
             for bw in (4, 8 | 0x100):
                 print("case", fmt, K, rows, bw, flush=True)
                 got = sddmm_capi(fmt, F, A, B, bw | _capi.bw_stripe(rows))

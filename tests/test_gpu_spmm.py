@@ -364,7 +364,7 @@ def test_spmm_xcd_stripe_flag(oracle, fmt):
         scale = spmm_abs_scale(oracle, F, X, want.shape[0])
         Xd = torch.from_numpy(X).cuda()
         base = spmm_capi(fmt, F, Xd, 1, 4)
-        for rows in (256, 768, 1536, 6144, 16128):
+        for rows in (256, 768, 1536, 6144, 65280):
             print("case", fmt, N, rows, flush=True)
             got = spmm_capi(fmt, F, Xd, 1, 4 | _capi.bw_stripe(rows))
             torch.cuda.synchronize()
@@ -374,4 +374,4 @@ def test_spmm_xcd_stripe_flag(oracle, fmt):
     p = _capi.ptr
     x = torch.zeros(4, 16, device="cuda")
     rp = torch.zeros(5, dtype=torch.int32, device="cuda")
-    assert _capi.lib.psp_spmm_csr_f32(p(rp), None, None, p(x), p(x), 4, 16, 4, 1, 4 | (1 << 18), None) == -1
+    assert _capi.lib.psp_spmm_csr_f32(p(rp), None, None, p(x), p(x), 4, 16, 4, 1, 4 | (1 << 20), None) == -1

@@ -54,15 +54,15 @@ def test_spmm_plan_mapping():
     assert _capi.spmm_plan(8, _capi.pack_cf(4, 8, 2), 4)["coarsen"] == 2
     # per-launch XCD stripe in the flag bits of blkWarpNum
     assert _capi.spmm_plan(64, 1, 4)["xcd_stripe_rows"] == 0
-    for rows in (256, 768, 6144, 16128):
+    for rows in (256, 768, 6144, 65280):
         p = _capi.spmm_plan(64, 2, 8 | _capi.bw_stripe(rows))
         assert (p["xcd_stripe_rows"], p["waves_per_block"], p["coarsen"]) == (rows, 8, 2)
     assert _capi.bw_stripe(0) == 0 and _capi.bw_stripe(None) == 0
-    for bad in (100, 16384, -256):
+    for bad in (100, 65536, -256):
         with pytest.raises(ValueError):
             _capi.bw_stripe(bad)
     with pytest.raises(_capi.ParamSpError):
-        _capi.spmm_plan(64, 1, 4 | (1 << 18))
+        _capi.spmm_plan(64, 1, 4 | (1 << 20))
     # options
     assert _capi.get_option("align_pct") == 50 and _capi.get_option("xcd_stripe_rows") == 8192
     _capi.set_option("align_pct", 25)
@@ -459,7 +459,7 @@ def test_xcd_stripe_levels_a_matrix_whose_long_rows_cluster():
         return share.max() * 8 / share.sum()
 
     uniform = np.full(n, 5)
-    assert fmt_of(uniform).xcd_stripe(False) == gi.XCD_STRIPES[0] == 8192
+    assert fmt_of(uniform).xcd_stripe(False) == 16384  # the longest candidate that leaves two rounds of stripes on 2^18 rows
     # row length = product over the index bits, as in an R-MAT graph
     idx = np.arange(n)
     deg = np.ones(n)
