@@ -217,6 +217,17 @@ int psp_spmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b, const floa
                            const float *X, float *Y, int Sb, int N, int rows_out, int vec_size, int CF,
                            int blkWarpNum, psp_stream_t stream);
 
+/* The four SpMM formats with the ReLU between two layers folded in (no counterpart among the reference's kernels:
+ * its driver applies F.relu as a pass of its own, GNN.py:43-61, 63-78).  fmt: 0 csr, 1 csr_split, 2 bcsr, 3 bcsr_split,
+ * arrays and sizes as for the plain entry point of that format (target_row NULL for the plain ones).
+ *   relu_x != 0: Y = A * max(X, 0) -- the product reads the previous layer's output through the ReLU, applied to the
+ *   rows as they are gathered (no activated copy of X is written);
+ *   mask != NULL ([rows_out, N], 16-byte aligned like Y): Y = (A * X) where mask > 0, else 0 -- the gradient with respect
+ *   to the pre-activation values a layer was given; a pass over Y that follows the product on the same stream. */
+int psp_spmm_act_f32(int fmt, const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
+                     const float *X, float *Y, int nseg, int N, int rows_out, int CF, int blkWarpNum, int relu_x,
+                     const float *mask, psp_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: SDDMM  out[p] = <A[row(p),:], B[col(p),:]>, fp32, NOT scaled by the stored values (the reference
  * kernels never multiply them in, SDDMM/sddmm_kernel.cu:917-983).  A and B are [*, K] row-major.

@@ -60,11 +60,19 @@ class GIN(torch.nn.Module):
             GINConv(widths[i], widths[i + 1]) for i in range(5)
         )
 
+        self.fuse_relu = True  # False: F.relu between the layers as separate passes, as the reference's driver does
+
     def forward(self):
-        x = self.x
-        for conv in (self.conv1, self.conv2, self.conv3, self.conv4):
-            x = F.relu(conv(x, self.spmm_dict))
-        return F.log_softmax(self.conv5(x, self.spmm_dict), dim=1)
+        if not self.fuse_relu:
+            x = self.x
+            for conv in (self.conv1, self.conv2, self.conv3, self.conv4):
+                x = F.relu(conv(x, self.spmm_dict))
+            return F.log_softmax(self.conv5(x, self.spmm_dict), dim=1)
+        # the same network with every ReLU applied inside the sparse product of the layer that reads it
+        z = self.conv1(self.x, self.spmm_dict)
+        for conv in (self.conv2, self.conv3, self.conv4, self.conv5):
+            z = conv(z, self.spmm_dict, relu_input=True)
+        return F.log_softmax(z, dim=1)
 
 
 class AGNN(torch.nn.Module):
@@ -231,7 +239,7 @@ def main(argv=None):
     p.add_argument("--no_aggregate_first", action="store_true",
                    help="GCN: always A (H W), also for the first layer when it widens its input (the reference's order)")
     p.add_argument("--no_fuse_relu", action="store_true",
-                   help="GCN: apply F.relu between the layers as passes of their own, as the reference's driver does")
+                   help="GCN / GIN: apply F.relu between the layers as passes of their own, as the reference's driver does")
     p.add_argument("--config", nargs=4, type=int, default=None, metavar=("IF_SPLIT", "VEC", "CF", "BW"),
                    help="skip the decider and use this configuration for every layer width")
     args = p.parse_args(argv)
@@ -261,6 +269,8 @@ def main(argv=None):
             if (args.net == "GCN" and not args.no_aggregate_first and args.num_features < hidden
                     and (decider is None or args.num_features in decider.model_dict)):
                 dims.append(args.num_features)  # the first layer runs its sparse product at the features' width
+            if args.net == "GIN" and args.num_features not in dims and (decider is None or args.num_features in decider.model_dict):
+                dims.append(args.num_features)  # GIN aggregates its input: the first layer's product has the features' width
             ops = configure_operators(decider, graph, dims, None if args.config is None else tuple(args.config))
             print("SpMM-decider config time: {:.3f} (ms)".format((time.perf_counter() - t1) * 1e3))
             model = build_model(args.net, graph, ops, hidden, args.num_features, args.num_classes, args.num_layers)

@@ -58,6 +58,7 @@ SIGNATURES = {
     "psp_check_index_dev": [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp],
     "psp_vbsr_count": [_vp, _vp, _i, _i, _i],
     "psp_vbsr_build": [_vp, _vp, _vp, _i, _i, _i, _vp, _vp, _vp],
+    "psp_spmm_act_f32": [_i, _vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp],
     "psp_spmm_vec_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "psp_spmm_vec_split_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "psp_genmask": [_vp, _vp, _vp, _i, _i, _vp, _vp],

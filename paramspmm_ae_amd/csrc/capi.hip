@@ -824,6 +824,46 @@ PSP_EXPORT int psp_spmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b,
                                     (hipStream_t)stream, nullptr, nullptr);
 }
 
+// Y[i] = Y[i] where mask[i] > 0, else 0 (float4 pieces; n a multiple of 4 is not required)
+__global__ void __launch_bounds__(256) psp_mask_kernel(float *__restrict__ Y, const float *__restrict__ mask, size_t n)
+{
+    const size_t n4 = n / 4;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (size_t)gridDim.x * blockDim.x) {
+        psp_f32x4 y = ((const psp_f32x4 *)Y)[i];
+        const psp_f32x4 m = __builtin_nontemporal_load((const psp_f32x4 *)mask + i);
+#pragma unroll
+        for (int e = 0; e < 4; e++) y[e] = m[e] > 0.0f ? y[e] : 0.0f;
+        ((psp_f32x4 *)Y)[i] = y;
+    }
+    const size_t t = n4 * 4 + (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t < n) Y[t] = mask[t] > 0.0f ? Y[t] : 0.0f;
+}
+
+PSP_EXPORT int psp_spmm_act_f32(int fmt, const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
+                                const float *X, float *Y, int nseg, int N, int rows_out, int CF, int blkWarpNum,
+                                int relu_x, const float *mask, psp_stream_t stream)
+{
+    PSP_REQUIRE(fmt >= 0 && fmt <= 3, "spmm_act: format code %d (0 csr, 1 csr_split, 2 bcsr, 3 bcsr_split)", fmt);
+    PSP_REQUIRE(((fmt & 1) != 0) == (target_row != nullptr) || nseg == 0, "spmm_act: target_row and the format code disagree");
+    PSP_REQUIRE((((size_t)mask | (size_t)Y) & 15) == 0, "spmm_act: Y and mask must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const int rx = relu_x != 0;
+    int rc;
+    switch (fmt) {
+    case 0: rc = psp_spmm_launch<1, false>(rowPtr, colIdx, val, nullptr, X, Y, nseg, N, rows_out, CF, blkWarpNum, st, nullptr, nullptr, rx); break;
+    case 1: rc = psp_spmm_launch<1, true>(rowPtr, colIdx, val, target_row, X, Y, nseg, N, rows_out, CF, blkWarpNum, st, nullptr, nullptr, rx); break;
+    case 2: rc = psp_spmm_launch<2, false>(rowPtr, colIdx, val, nullptr, X, Y, nseg, N, rows_out, CF, blkWarpNum, st, nullptr, nullptr, rx); break;
+    default: rc = psp_spmm_launch<2, true>(rowPtr, colIdx, val, target_row, X, Y, nseg, N, rows_out, CF, blkWarpNum, st, nullptr, nullptr, rx); break;
+    }
+    if (rc != PSP_OK || mask == nullptr) return rc;
+    // The mask is a pass of its own over Y (see spmm_kernel.h: applied where the kernel closes a row it was slower).
+    const size_t n = (size_t)rows_out * (size_t)N;
+    if (n == 0) return PSP_OK;
+    const size_t want = (n / 4 + 255) / 256 + 1;
+    hipLaunchKernelGGL(psp_mask_kernel, dim3((unsigned)std::min<size_t>(want, 256 * 32)), dim3(256), 0, st, Y, mask, n);
+    return psp_check_launch("mask pass");
+}
+
 PSP_EXPORT int psp_sddmm_csr_f32(const int *rowPtr, const int *colIdx, const float *A, const float *B,
                                  const float *scale, float *out, int M, int K, int blkWarpNum, psp_stream_t stream)
 {

@@ -1,4 +1,4 @@
 // SpMM kernels of the bcsr format (instantiations only; the template lives in spmm_kernel.h).
 #include "spmm_launch_impl.h"
 template int psp_spmm_launch<2, false>(const int *, const int *, const float *, const int *, const float *, float *,
-                                     int, int, int, int, int, hipStream_t, const float *, float *);
+                                     int, int, int, int, int, hipStream_t, const float *, float *, int);

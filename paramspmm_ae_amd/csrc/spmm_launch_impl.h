@@ -6,7 +6,7 @@
 template <int NR, bool SPLIT>
 int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, const int *target_row,
                     const float *X, float *Y, int nrows, int N, int rows_out, int CF, int blkWarpNum,
-                    hipStream_t stream, const float *row_max, float *row_sum)
+                    hipStream_t stream, const float *row_max, float *row_sum, int relu_x)
 {
     psp_spmm_plan plan;
     int rc = psp_spmm_plan_for(N, CF, blkWarpNum, &plan);
@@ -54,6 +54,7 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     if (rc != PSP_OK) return rc;
     if (nrows == 0) return PSP_OK;
     const bool softmax = row_max != nullptr;
+    PSP_REQUIRE(!(softmax && relu_x), "spmm: the softmax-weighted product takes no activation argument");
     if (softmax && SPLIT) {
         PSP_REQUIRE(row_sum, "spmm softmax: row_sum workspace is null");
         rc = psp_zero_f32(row_sum, (size_t)rows_out, stream);
@@ -61,7 +62,7 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     }
 
     const int segs_per_block = plan.waves_per_block << logW;
-    psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll, softmax);
+    psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll, softmax, relu_x != 0);
     if (!k)
         return psp_fail(PSP_ERR_ARG, "spmm%s: no kernel for coarsen %d vec %d unroll %d%s", softmax ? " softmax" : "", plan.coarsen,
                         plan.vec, plan.unroll, softmax ? " (needs N % 4 == 0 and CF <= 4)" : "");
@@ -70,7 +71,7 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block),
                                       (plan.xcd_stripe_rows ? plan.xcd_stripe_rows : opt.stripe_rows) / segs_per_block);
     dim3 grid(g.launch, plan.col_tiles, 1), block(plan.waves_per_block * PSP_WAVE, 1, 1);
-    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.stripe, align_pct, row_max, row_sum);
+    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.stripe, align_pct, row_max, row_sum, relu_x);
     rc = psp_check_launch("spmm kernel");
     if (rc != PSP_OK || !(softmax && SPLIT)) return rc;
     return psp_row_scale(Y, row_sum, rows_out, N, stream);  // rows that several wavefronts added to

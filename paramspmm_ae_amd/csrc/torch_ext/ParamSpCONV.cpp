@@ -140,6 +140,42 @@ static Tensor aggregate_op(int fmt, Tensor D, Tensor rowPtr, Tensor colIdx, Tens
     return aggregate(fmt, D, rowPtr, colIdx, values, target_row ? &*target_row : nullptr, CF, bw);
 }
 
+// A * max(D, 0) and / or (A * D) kept where mask > 0: the ReLU between two layers folded into the sparse product
+// (psp_spmm_act_f32).  Used by the layers that aggregate first (GIN: (A X) W): the activation is applied as the rows of
+// D are gathered, its backward as the rows of the gradient are written.  No counterpart among the reference's
+// bindings: its driver runs F.relu as a pass of its own (GNN.py:63-78).  float64 and mask shapes the kernel does not
+// take fall back to PyTorch's passes around the plain product.
+static Tensor aggregate_act_op(int fmt, Tensor D, Tensor rowPtr, Tensor colIdx, Tensor values, c10::optional<Tensor> target_row,
+                               int CF, int bw, bool relu_input, c10::optional<Tensor> mask)
+{
+    need_gpu(D, "input");
+    TORCH_CHECK(fmt >= 0 && fmt <= 3 && ((fmt & 1) != 0) == target_row.has_value(), "format code and target_row disagree");
+    check_cf(CF);
+    const Tensor *tr = target_row ? &*target_row : nullptr;
+    if (mask) {
+        need_gpu(*mask, "mask");
+        TORCH_CHECK(mask->dim() == 2 && mask->size(0) == D.size(0) && mask->size(1) == D.size(1), "mask must have the shape of the result");
+    }
+    const bool fused = D.scalar_type() == torch::kFloat32 && (!mask || mask->scalar_type() == torch::kFloat32) &&
+                       D.size(1) > 0 && D.size(0) > 0 && (fmt < 2 || D.size(0) % 2 == 0 || !mask);
+    if (!fused) {
+        Tensor Y = aggregate(fmt, relu_input ? torch::relu(D) : D, rowPtr, colIdx, values, tr, CF, bw);
+        return mask ? at::threshold_backward(Y, *mask, 0) : Y;
+    }
+    Tensor Dc = D.contiguous();
+    check_spmm_args(fmt, Dc, rowPtr, colIdx, values, tr);
+    DeviceGuard guard(Dc.device());
+    const long rows_out = fmt >= 2 ? (Dc.size(0) + 1) / 2 * 2 : Dc.size(0);
+    Tensor Mc;
+    if (mask) Mc = mask->contiguous();
+    Tensor Y = torch::empty({rows_out, Dc.size(1)}, Dc.options());
+    ok(psp_spmm_act_f32(fmt, ip(rowPtr), ip(colIdx), fp(values), tr ? ip(*tr) : nullptr, fp(Dc), fpw(Y),
+                        (int)rowPtr.size(0) - 1, (int)Dc.size(1), (int)rows_out, CF, bw, relu_input ? 1 : 0,
+                        mask ? fp(Mc) : nullptr, stream_of(Dc)));
+    if (Y.size(0) != Dc.size(0)) Y = Y.narrow(0, 0, Dc.size(0));
+    return Y;
+}
+
 static Tensor forward_impl(int fmt, const Tensor &H, const Tensor &W, const Tensor &rowPtr, const Tensor &colIdx,
                            const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
 {
@@ -242,6 +278,8 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("nll_loss_mean", &nll_loss_mean, "[loss, stats] of the mean negative log-likelihood (log-probabilities, int64 labels)");
     m.def("nll_loss_mean_backward", &nll_loss_mean_backward, "gradient w.r.t. the log-probabilities: (labels, grad_loss, stats, n, C)");
     m.def("aggregate", &aggregate_op, "A*D: (fmt, D, rowPtr, colIdx, values, target_row | None, CF, blkWarpNum)");
+    m.def("aggregate_act", &aggregate_act_op,
+          "A*max(D,0) (relu_input) and / or (A*D) where mask > 0: (fmt, D, rowPtr, colIdx, values, target_row | None, CF, blkWarpNum, relu_input, mask | None)");
     m.def("relu_input_forward", &relu_input_forward,
           "A*(relu(Z)*W): (fmt 0..3, Z, W, rowPtr, colIdx, values, target_row or None, CF, blkWarpNum)");
     m.def("relu_input_backward", &relu_input_backward,

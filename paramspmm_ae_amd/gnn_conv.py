@@ -233,6 +233,51 @@ class GINFunction(torch.autograd.Function):
         return d_input, d_weights, None
 
 
+class GINReLUInputFunction(torch.autograd.Function):
+    """(A relu(Z)) W as one function of the pre-activation values Z, for a layer that widens its input: the activation
+    is applied as the sparse product gathers the rows of Z (ParamSpCONV.aggregate_act), the gradient is masked in a pass
+    that follows the backward product.  The reference's driver applies F.relu between the layers (GNN.py:63-78)."""
+
+    @staticmethod
+    def forward(ctx, Z, weight, ParamSpMM):
+        op = ParamSpMM
+        fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
+        X_agg = SpCONV.aggregate_act(fmt, Z, op.rowPtr, op.colIdx, op.val, op.target_row if op.if_split else None, op.CF,
+                                     _bw(op), True, None)
+        ctx.save_for_backward(X_agg, weight, Z)
+        ctx.ParamSpMM = op
+        return SpCONV.dense_xw(X_agg, weight, False)
+
+    @staticmethod
+    def backward(ctx, d_output):
+        X_agg, weights, Z = ctx.saved_tensors
+        op = ctx.ParamSpMM
+        fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
+        d_output = d_output.contiguous()
+        d_weights = SpCONV.weight_gradient(X_agg, d_output)
+        d_input = SpCONV.aggregate_act(fmt, SpCONV.dense_xw(d_output, weights, True), op.rowPtr, op.colIdx, op.val,
+                                       op.target_row if op.if_split else None, op.CF, _bw(op), False, Z)
+        return d_input, d_weights, None
+
+
 class GINConv(_Layer):
-    def forward(self, X, spmm_dict):
-        return GINFunction.apply(X, self.weights, self._operator(spmm_dict))
+    operator_of_input_width = True
+
+    def forward(self, X, spmm_dict, relu_input=False):
+        """``relu_input``: X holds pre-activation values and the layer computes (A relu(X)) W without an activation
+        pass.  A layer that does not widen its input is evaluated as A (relu(X) W) -- the same product, the sparse
+        part at the narrower width -- with the activation and its backward folded into the dense products, like the
+        GCN layer; a widening layer applies the activation inside the sparse product."""
+        in_w, out_w = self.weights.shape
+        if relu_input and in_w >= out_w:
+            op = self._operator(spmm_dict)
+            if op.vec_size in (1, 2):
+                return GCNReLUInputFunction.apply(X, self.weights, op)
+        # the sparse product runs at the input's width: take the operator configured for that width when there is
+        # one (the reference's layers look up the output's width only, gnn_conv.py:223-226)
+        op = spmm_dict[in_w] if self.operator_of_input_width and in_w in spmm_dict else self._operator(spmm_dict)
+        if relu_input and op.vec_size in (1, 2):
+            return GINReLUInputFunction.apply(X, self.weights, op)
+        if relu_input:
+            X = torch.relu(X)
+        return GINFunction.apply(X, self.weights, op)

@@ -678,3 +678,76 @@ def test_wide_dense_products_with_the_activation_folded_in(K1, K2, n):
     # the two fused forms are exclusive, as for the narrow kernel
     assert L.psp_gemm_xw_act_f32(p(X), p(W), p(Y), n, K1, K2, 1, 1, None, st) == -1
     assert L.psp_gemm_xw_act_f32(p(X), p(W), p(Y), n, K1, K2, 0, 0, p(Z), st) == -1
+
+
+@pytest.mark.parametrize("vec,split", VARIANTS)
+@pytest.mark.parametrize("n,width_in,width_out", [(301, 24, 40), (20001, 32, 16), (20000, 16, 128), (17001, 128, 16)])
+def test_gin_layer_with_relu_on_its_input(vec, split, n, width_in, width_out):
+    """(A relu(Z)) W as one function of Z against PyTorch autograd of the same expression: the activation applied as the
+    sparse product gathers its rows, the mask as the backward product writes its rows (odd row counts, widths with a
+    partial column tile, all four formats); the operator of the input's width is the one that runs."""
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from paramspmm_ae_amd.gnn_conv import GINConv
+
+    g, rowPtr, colIdx, val = sym_graph(n, 5)
+    S = torch.sparse_csr_tensor(torch.from_numpy(rowPtr).cuda(), torch.from_numpy(colIdx).cuda(), torch.from_numpy(val).cuda(),
+                                size=(n, n))
+    op = pcsr_spmm(g, vec_size=vec, if_split=split, CF=1, blkWarpNum=4)
+    torch.manual_seed(3)
+    layer = GINConv(width_in, width_out).cuda()
+    Z = torch.randn(n, width_in, device="cuda", requires_grad=True)
+    y = layer(Z, {width_in: op, width_out: op}, relu_input=True)
+    assert type(y.grad_fn).__name__.startswith("GINReLUInputFunction" if width_in < width_out else "GCNReLUInputFunction")
+    dY = torch.randn_like(y)
+    y.backward(dY)
+    Zr = Z.detach().clone().requires_grad_(True)
+    Wr = layer.weights.detach().clone().requires_grad_(True)
+    yr = torch.sparse.mm(S, torch.relu(Zr)) @ Wr
+    yr.backward(dY)
+    torch.testing.assert_close(y, yr, rtol=1e-4, atol=1e-5)
+    torch.testing.assert_close(Z.grad, Zr.grad, rtol=1e-3, atol=1e-4)
+    torch.testing.assert_close(layer.weights.grad, Wr.grad, rtol=2e-3, atol=2e-3)
+    assert bool((Z.grad[Z.detach() <= 0] == 0).all())
+
+
+@pytest.mark.parametrize("fmt", [0, 1, 2, 3])
+def test_spmm_with_activation_arguments_through_the_c_abi(oracle, fmt):
+    """psp_spmm_act_f32: A max(X, 0) equals the plain product of the clamped input bit for bit, the masked product
+    equals the plain one where the mask is positive and is an exact zero elsewhere (a hub row, native
+    configurations, a width that is not a multiple of four)."""
+    from conftest import random_csr
+    from gpu_util import Formats, spmm_capi
+    from paramspmm_ae_amd import _capi
+
+    L, p = _capi.lib, _capi.ptr
+    names = ["csr", "csr_split", "bcsr", "bcsr_split"]
+    rowPtr, colIdx, val = random_csr(6001, 9, 21, empty_frac=0.1, hub=(11, 3000), values="normal")
+    F = Formats(oracle, rowPtr, colIdx, val)
+    d = F.d
+    arrays = [(d["rowPtr"], d["colIdx"], d["val"], None, F.n), (d["rps"], d["colIdx"], d["val"], d["tr"], F.tr.size),
+              (d["rpb"], d["cib"], d["vb"], None, F.rpb.size - 1), (d["rpbs"], d["cib"], d["vb"], d["trb"], F.trb.size)][fmt]
+    st = torch.cuda.current_stream().cuda_stream
+    rows = F.n + (F.n & 1)
+    for N, cf in ((16, 1), (100, 2), (7, 1), (128, _capi.pack_cf(1, 16, 4)), (256, _capi.pack_cf(4, 8, 2, even_split=True))):
+        g = torch.Generator(device="cuda").manual_seed(N)
+        X = torch.randn(rows, N, device="cuda", generator=g)
+        M = torch.randn(rows, N, device="cuda", generator=g)
+        if N == 100:
+            M = M.contiguous()
+        plain = spmm_capi(names[fmt], F, X, cf, 8)
+        clamped = spmm_capi(names[fmt], F, torch.relu(X), cf, 8)
+        Y = torch.full((rows, N), float("nan"), device="cuda")
+        rp, ci, v, tr, nseg = arrays
+        _capi.check(L.psp_spmm_act_f32(fmt, p(rp), p(ci), p(v), p(tr), p(X), p(Y), nseg, N, rows, cf, 8, 1, None, st))
+        if fmt in (0, 2):
+            assert torch.equal(Y, clamped)
+        else:
+            torch.testing.assert_close(Y, clamped, rtol=1e-5, atol=1e-5)
+        _capi.check(L.psp_spmm_act_f32(fmt, p(rp), p(ci), p(v), p(tr), p(X), p(Y), nseg, N, rows, cf, 8, 0, p(M), st))
+        want = torch.where(M > 0, plain, torch.zeros_like(plain))
+        if fmt in (0, 2):
+            assert torch.equal(Y, want)
+        else:
+            torch.testing.assert_close(Y, want, rtol=1e-5, atol=1e-5)
+        assert bool((Y[M <= 0] == 0).all())
+    assert L.psp_spmm_act_f32(4, p(rp), p(ci), p(v), p(tr), p(X), p(Y), nseg, N, rows, 1, 8, 1, None, st) == -1
