@@ -188,7 +188,7 @@ class AGNNFunction(torch.autograd.Function):
         X, weights, edge_attentions = ctx.saved_tensors
         d_output = d_output.contiguous()
         d_input_prime = op.AGNN_spmm(edge_attentions, d_output)
-        d_input = SpCONV.dense_xw(d_input_prime, weights, True)
+        d_input = SpCONV.dense_xw(d_input_prime, weights, True) if ctx.needs_input_grad[0] else None
         d_weights = SpCONV.weight_gradient(X, d_input_prime)  # X^T * d_input_prime
         d_attention = op.AGNN_sddmm(d_output)
         if d_attention.dim() != 1:
@@ -229,7 +229,8 @@ class GINFunction(torch.autograd.Function):
         X_agg, weights = ctx.saved_tensors
         d_output = d_output.contiguous()  # an upstream gradient may be a view (expand, transpose, slice)
         d_weights = SpCONV.weight_gradient(X_agg, d_output)  # X_agg^T * d_output
-        d_input = ctx.ParamSpMM.GIN_spmm(SpCONV.dense_xw(d_output, weights, True))
+        # the network's first layer reads the features, which need no gradient: no dense and no sparse product for it
+        d_input = ctx.ParamSpMM.GIN_spmm(SpCONV.dense_xw(d_output, weights, True)) if ctx.needs_input_grad[0] else None
         return d_input, d_weights, None
 
 
