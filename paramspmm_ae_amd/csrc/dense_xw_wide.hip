@@ -11,9 +11,10 @@
 //     16t + 4q + e stands for index k = q of the instruction: which four columns a step contracts is free as long as
 //     operand A follows the same rule;
 //   * operand A (16 x 4) is a piece of W^T read from LDS: lane (r, q) supplies W[16t + 4q + e][16j + r] for column
-//     tile j (T = K2 / 16 tiles).  LDS holds the columns of W permuted, column 16j + r at position r * T + j, so a
-//     lane's T tiles are T consecutive floats: two 16-byte LDS reads per step serve eight MFMAs (sixteen with the two
-//     row blocks a wavefront works on);
+//     tile j (T = K2 / 16 tiles).  LDS holds the columns of W permuted -- column 16j + r at position
+//     ((j / 4) * 16 + r) * 4 + j % 4 -- so a lane fetches four tiles with one 16-byte read and the sixteen r-lanes of
+//     such a read cover 256 contiguous bytes (no bank conflicts): two reads per step serve eight MFMAs (sixteen with
+//     the two row blocks a wavefront works on);
 //   * result lane (r, q), tile j, element i is Y[row r][16j + 4q + i]: one 16-byte store per tile, the four q-lanes
 //     of a row writing 64 contiguous bytes.
 // W (at most 64 KB) is staged into LDS once per workgroup, transposed on the way in for the X * W^T form; the grid is
@@ -45,7 +46,7 @@ psp_xw_wide_kernel(const float *__restrict__ X, const float *__restrict__ W, flo
             k = idx / K2;
             c = idx - k * K2;
         }
-        Ws[k * S + (c & 15) * T + (c >> 4)] = W[idx];
+        Ws[k * S + (((c >> 6) * 16 + (c & 15)) << 2) + ((c >> 4) & 3)] = W[idx];
     }
     __syncthreads();
 
@@ -85,10 +86,10 @@ psp_xw_wide_kernel(const float *__restrict__ X, const float *__restrict__ W, flo
         for (int t = 0; t < KT; t++) {
 #pragma unroll
             for (int e = 0; e < 4; e++) {
-                const psp_f32x4 *wr = (const psp_f32x4 *)(Ws + (16 * t + 4 * q + e) * S + r * T);
+                const psp_f32x4 *wr = (const psp_f32x4 *)(Ws + (16 * t + 4 * q + e) * S) + r;
                 psp_f32x4 a4[T / 4];
 #pragma unroll
-                for (int v = 0; v < T / 4; v++) a4[v] = wr[v];
+                for (int v = 0; v < T / 4; v++) a4[v] = wr[16 * v];
 #pragma unroll
                 for (int j = 0; j < T; j++) {
 #pragma unroll
