@@ -850,12 +850,16 @@ def main():
         torch.cuda.empty_cache()
         from paramspmm_ae_amd import GNN
 
+        epochs = {}
         with contextlib.redirect_stdout(sys.stderr):
-            res = GNN.main(["--net", "GCN", "--synthetic", "C5", "--hidden_list", "16", "--num_classes", "16",
-                            "--num_features", "32", "--num_epoches", "20"])
-        out["gcn_epoch_ms"] = {"value": round(float(list(res.values())[0]), 3), "unit": "ms per epoch", "epochs": 20,
-                               "config": "GCN, 5 layers, hidden 16, 16 classes, 32 features, fwd+bwd+Adam, SBM 1M nodes "
-                                         "(community order), decider-picked operators"}
+            for net in ("GCN", "GIN"):
+                res = GNN.main(["--net", net, "--synthetic", "C5", "--hidden_list", "16", "32", "128", "--num_classes", "16",
+                                "--num_features", "32", "--num_epoches", "20"])
+                epochs[net] = {str(h): round(float(ms), 3) for (_, h), ms in res.items()}
+        out["gcn_epoch_ms"] = {"value": epochs["GCN"]["16"], "unit": "ms per epoch", "epochs": 20,
+                               "by_hidden": epochs["GCN"], "gin_by_hidden": epochs["GIN"],
+                               "config": "5 layers, hidden 16 / 32 / 128 (value: GCN, hidden 16), 16 classes, 32 features, "
+                                         "fwd+bwd+Adam, SBM 1M nodes (community order), decider-picked operators"}
 
     print(json.dumps(out))
 

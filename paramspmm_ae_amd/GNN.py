@@ -87,13 +87,23 @@ class AGNN(torch.nn.Module):
         self.hidden_layers = nn.ModuleList(AGNNConv(hidden, hidden) for _ in range(num_layers - 2))
         self.conv2 = AGNNConv(hidden, num_classes)
         self.relu = nn.ReLU()
+        self.fuse_relu = True  # False: ReLU between the layers as separate passes, as the reference's driver does
 
     def forward(self):
-        x = self.relu(self.conv1(self.x, self.spmm_dict, self.colIdx))
-        x = F.dropout(x, training=self.training)
+        if not self.fuse_relu:
+            x = self.relu(self.conv1(self.x, self.spmm_dict, self.colIdx))
+            x = F.dropout(x, training=self.training)
+            for conv in self.hidden_layers:
+                x = self.relu(conv(x, self.spmm_dict, self.colIdx))
+            return F.log_softmax(self.conv2(x, self.spmm_dict, self.colIdx), dim=1)
+        # The same network with every ReLU applied by the layer that reads it.  Dropout scales by a non-negative
+        # mask, so it commutes with the activation: dropping the pre-activation values and activating afterwards
+        # gives what the reference's order gives, with the same random mask.
+        z = self.conv1(self.x, self.spmm_dict, self.colIdx)
+        z = F.dropout(z, training=self.training)
         for conv in self.hidden_layers:
-            x = self.relu(conv(x, self.spmm_dict, self.colIdx))
-        return F.log_softmax(self.conv2(x, self.spmm_dict, self.colIdx), dim=1)
+            z = conv(z, self.spmm_dict, self.colIdx, relu_input=True)
+        return F.log_softmax(self.conv2(z, self.spmm_dict, self.colIdx, relu_input=True), dim=1)
 
 
 def capture_training_step(model, labels, optimizer, warmup=3):
@@ -239,7 +249,7 @@ def main(argv=None):
     p.add_argument("--no_aggregate_first", action="store_true",
                    help="GCN: always A (H W), also for the first layer when it widens its input (the reference's order)")
     p.add_argument("--no_fuse_relu", action="store_true",
-                   help="GCN / GIN: apply F.relu between the layers as passes of their own, as the reference's driver does")
+                   help="apply the ReLU between the layers as passes of their own, as the reference's driver does")
     p.add_argument("--config", nargs=4, type=int, default=None, metavar=("IF_SPLIT", "VEC", "CF", "BW"),
                    help="skip the decider and use this configuration for every layer width")
     args = p.parse_args(argv)

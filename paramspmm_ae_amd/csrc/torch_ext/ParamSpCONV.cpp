@@ -275,6 +275,24 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
         need_gpu(W, "W");
         return dense_xw(X, W, transW);
     }, "X * W (transW false) or X * W^T for tall-skinny X: (X, W, transW)");
+    // the dense products of a layer that reads its input through a ReLU, for layers that place them around their
+    // own sparse operators (the attention layer): max(Z, 0) * W, (G * W^T) where Z > 0, max(Z, 0)^T * G
+    m.def("dense_relu_xw", [](Tensor Z, Tensor W) {
+        need_gpu(Z, "Z");
+        need_gpu(W, "W");
+        return dense_relu_xw(Z, W);
+    }, "max(Z, 0) * W: (Z, W)");
+    m.def("dense_xwt_masked", [](Tensor G, Tensor W, Tensor Z) {
+        need_gpu(G, "G");
+        need_gpu(W, "W");
+        need_gpu(Z, "Z");
+        return dense_xwt_masked(G, W, Z);
+    }, "(G * W^T) where Z > 0, else 0: (G, W, Z)");
+    m.def("weight_gradient_relu", [](Tensor Z, Tensor G) {
+        need_gpu(Z, "Z");
+        need_gpu(G, "G");
+        return weight_gradient_relu(Z, G);
+    }, "max(Z, 0)^T * G: (Z, G)");
     m.def("nll_loss_mean", &nll_loss_mean, "[loss, stats] of the mean negative log-likelihood (log-probabilities, int64 labels)");
     m.def("nll_loss_mean_backward", &nll_loss_mean_backward, "gradient w.r.t. the log-probabilities: (labels, grad_loss, stats, n, C)");
     m.def("aggregate", &aggregate_op, "A*D: (fmt, D, rowPtr, colIdx, values, target_row | None, CF, blkWarpNum)");

@@ -171,8 +171,10 @@ class AGNNFunction(torch.autograd.Function):
     (gnn_conv.py:128-180).  No softmax, as in the reference."""
 
     @staticmethod
-    def forward(ctx, X, weights, attention_w, ParamSpMM, colIdx):
-        X_prime = SpCONV.dense_xw(X, weights, False)
+    def forward(ctx, X, weights, attention_w, ParamSpMM, colIdx, relu_input=False):
+        # relu_input: X holds pre-activation values; the activation and its backward ride on the dense products
+        ctx.relu_input = bool(relu_input)
+        X_prime = SpCONV.dense_relu_xw(X, weights) if relu_input else SpCONV.dense_xw(X, weights, False)
         edge_feature = ParamSpMM.AGNN_sddmm(X_prime)
         # csr: [nnz] ; 2x1 blocks: [nblk, 2] -- a single head scales both the same way
         edge_attentions = (edge_feature * attention_w.reshape(())).contiguous()
@@ -188,8 +190,14 @@ class AGNNFunction(torch.autograd.Function):
         X, weights, edge_attentions = ctx.saved_tensors
         d_output = d_output.contiguous()
         d_input_prime = op.AGNN_spmm(edge_attentions, d_output)
-        d_input = SpCONV.dense_xw(d_input_prime, weights, True) if ctx.needs_input_grad[0] else None
-        d_weights = SpCONV.weight_gradient(X, d_input_prime)  # X^T * d_input_prime
+        if not ctx.needs_input_grad[0]:
+            d_input = None
+        elif ctx.relu_input:
+            d_input = SpCONV.dense_xwt_masked(d_input_prime, weights, X)
+        else:
+            d_input = SpCONV.dense_xw(d_input_prime, weights, True)
+        # X^T * d_input_prime (relu(X)^T when the layer reads X through the activation)
+        d_weights = SpCONV.weight_gradient_relu(X, d_input_prime) if ctx.relu_input else SpCONV.weight_gradient(X, d_input_prime)
         d_attention = op.AGNN_sddmm(d_output)
         if d_attention.dim() != 1:
             d_attention = d_attention.view(-1)[op.mask]  # block layout -> CSR slots
@@ -202,7 +210,7 @@ class AGNNFunction(torch.autograd.Function):
             col_f = ctx.colIdx.reshape(-1).to(d_attention.dtype)
             op._colIdx_as_float = col_f
         d_attention_w = torch.dot(d_attention, col_f).reshape(1, 1).expand(1, n_heads)
-        return d_input, d_weights, d_attention_w, None, None
+        return d_input, d_weights, d_attention_w, None, None, None
 
 
 class AGNNConv(_Layer):
@@ -210,8 +218,8 @@ class AGNNConv(_Layer):
         super().__init__(input_dim, output_dim)
         self.attention_w = torch.nn.Parameter(torch.randn(1, n_heads))
 
-    def forward(self, X, spmm_dict, colIdx):
-        return AGNNFunction.apply(X, self.weights, self.attention_w, self._operator(spmm_dict), colIdx)
+    def forward(self, X, spmm_dict, colIdx, relu_input=False):
+        return AGNNFunction.apply(X, self.weights, self.attention_w, self._operator(spmm_dict), colIdx, relu_input)
 
 
 class GINFunction(torch.autograd.Function):

@@ -751,3 +751,40 @@ def test_spmm_with_activation_arguments_through_the_c_abi(oracle, fmt):
             torch.testing.assert_close(Y, want, rtol=1e-5, atol=1e-5)
         assert bool((Y[M <= 0] == 0).all())
     assert L.psp_spmm_act_f32(4, p(rp), p(ci), p(v), p(tr), p(X), p(Y), nseg, N, rows, 1, 8, 1, None, st) == -1
+
+
+@pytest.mark.parametrize("net,hidden", [("GIN", 16), ("GIN", 64), ("AGNN", 16), ("AGNN", 64)])
+def test_gin_and_agnn_networks_with_folded_relu_equal_the_plain_ones(net, hidden):
+    """The GIN and the attention network with their activations folded into the layers give the loss and the gradients
+    of the networks with a ReLU pass between the layers (GNN.py:63-101); the attention network's dropout draws the
+    same mask in both (same seed) and commutes with the activation."""
+    from paramspmm_ae_amd import GNN
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from paramspmm_ae_amd.gnn_conv import nll_loss_mean
+
+    n = 20000
+    g, rowPtr, colIdx, val = sym_graph(n, 9)
+    op = pcsr_spmm(g, vec_size=1, if_split=False, CF=1, blkWarpNum=4)
+    ops = {16: op, 32: op, hidden: op}
+    torch.manual_seed(0)
+    x = torch.randn(n, 32, device="cuda")
+    labels = torch.randint(0, 16, (n,), device="cuda")
+    if net == "GIN":
+        model = GNN.GIN(16, 32, x, ops, hidden).cuda()
+    else:
+        model = GNN.AGNN(16, 32, x, ops, hidden, g.csr_data.colIdx.cuda().unsqueeze(-1)).cuda()
+        with torch.no_grad():  # keep the attention scores of five stacked layers in range
+            for p in model.parameters():
+                p.mul_(0.3)
+    model.train()
+    grads = {}
+    for fused in (True, False):
+        model.fuse_relu = fused
+        model.zero_grad(set_to_none=True)
+        torch.manual_seed(123)  # the dropout mask
+        loss = nll_loss_mean(model(), labels)
+        loss.backward()
+        grads[fused] = (loss.item(), [p.grad.clone() for p in model.parameters()])
+    assert abs(grads[True][0] - grads[False][0]) <= 1e-4 * abs(grads[False][0])
+    for a, b in zip(grads[True][1], grads[False][1]):
+        torch.testing.assert_close(a, b, rtol=2e-3, atol=1e-4 * float(b.abs().max()) + 1e-6)
