@@ -659,7 +659,7 @@ def main():
     by_symbol = {}
     for r in per_dim:
         plan = _capi.spmm_plan(r["dim"], r["CF"], r["blkWarpNum"])
-        sym = "psp_spmm_kernel<%d, %d, %d, %d, %s, false>" % (plan["coarsen"], plan["vec"], plan["unroll"],
+        sym = "psp_spmm_kernel<%d, %d, %d, %d, %s, false, false>" % (plan["coarsen"], plan["vec"], plan["unroll"],
                                                        2 if r["format"].startswith("bcsr") else 1,
                                                        "true" if "split" in r["format"] else "false")
         r["kernel"] = sym
@@ -759,31 +759,33 @@ def main():
         del A, Bm
 
     if not args.no_extras and args.reorder is None and pick == "decider":
-        # ---- the same sweep after the community reordering pass (rows and columns permuted together at load time,
+        # ---- the same sweep after a reordering pass (rows and columns permuted together at load time,
         # paramspmm_ae_amd/reorder.py; the reference's inputs arrive Rabbit-ordered, README.md:14-16) ---------------
-        t1 = time.time()
-        graph_r = graph_input(mtx_name=args.graph, path="")
-        graph_r.verbose = False
-        graph_r.load_from_csr(rowPtr, colIdx, val, reorder="community")
-        load_r = time.time() - t1
-        ops_r = sweep.operators_of(graph_r)
-        chosen_r = {d: tuple(int(v) for v in decider.config_PCSR(graph_r, d)) for d in dims}
-        wall_r, events_r = timed_steps(ops_r, chosen_r)
-        F_r = {"n": n, "nnz": nnz, "S": graph_r.csr_data.target_row.numel(), "Mb": graph_r.bcsr_data.num_nodes,
-               "nblk": graph_r.bcsr_data.colIdx.numel(), "Sb": graph_r.bcsr_data.target_row.numel()}
-        fracs = []
-        for d in dims:
-            ms = float(np.mean([a.elapsed_time(b) for a, b in events_r[d]]))
-            if_split, vec, cf, bw = chosen_r[d]
-            fmt = fmt_names[(1 if if_split else 0) + (2 if vec == 2 else 0)]
-            fracs.append(algorithmic_bytes(fmt, F_r, n, d) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
-        out["reordered"] = {"order": "community (label propagation, vertices sorted by label)",
-                            "value": round(flops_step * args.steps / wall_r / 1e9, 1), "unit": "GFLOP/s",
-                            "ms_per_step": round(wall_r * 1e3 / args.steps, 4), "speedup": round(wall / wall_r, 3),
-                            "mean_frac_over_widths": round(float(np.mean(fracs)), 4),
-                            "load_s_with_reordering": round(load_r, 2), "load_s_without": round(load_s, 2)}
-        del ops_r, graph_r
-        torch.cuda.empty_cache()
+        out["reordered"] = {}
+        for order, text in (("community", "label propagation, vertices sorted by label"),
+                            ("degree", "vertices sorted by descending degree")):
+            t1 = time.time()
+            graph_r = graph_input(mtx_name=args.graph, path="")
+            graph_r.verbose = False
+            graph_r.load_from_csr(rowPtr, colIdx, val, reorder=order)
+            load_r = time.time() - t1
+            ops_r = sweep.operators_of(graph_r)
+            chosen_r = {d: tuple(int(v) for v in decider.config_PCSR(graph_r, d)) for d in dims}
+            wall_r, events_r = timed_steps(ops_r, chosen_r)
+            F_r = {"n": n, "nnz": nnz, "S": graph_r.csr_data.target_row.numel(), "Mb": graph_r.bcsr_data.num_nodes,
+                   "nblk": graph_r.bcsr_data.colIdx.numel(), "Sb": graph_r.bcsr_data.target_row.numel()}
+            fracs = []
+            for d in dims:
+                ms = float(np.mean([a.elapsed_time(b) for a, b in events_r[d]]))
+                if_split, vec, cf, bw = chosen_r[d]
+                fmt = fmt_names[(1 if if_split else 0) + (2 if vec == 2 else 0)]
+                fracs.append(algorithmic_bytes(fmt, F_r, n, d) / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS)
+            out["reordered"][order] = {"order": text, "value": round(flops_step * args.steps / wall_r / 1e9, 1), "unit": "GFLOP/s",
+                                       "ms_per_step": round(wall_r * 1e3 / args.steps, 4), "speedup": round(wall / wall_r, 3),
+                                       "mean_frac_over_widths": round(float(np.mean(fracs)), 4),
+                                       "load_s_with_reordering": round(load_r, 2), "load_s_without": round(load_s, 2)}
+            del ops_r, graph_r
+            torch.cuda.empty_cache()
 
     if not args.no_vendor:
         # vendor library beside it: rocSPARSE CSR SpMM (default algorithm), the counterpart of the cuSPARSE baseline
