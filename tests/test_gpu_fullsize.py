@@ -202,3 +202,81 @@ def test_gcn_operators_at_full_size():
                             "--num_features", "32", "--num_epoches", "2", "--verbose", "False"])
             assert len(res) == 1 and all(np.isfinite(v) and v > 0 for v in res.values())
         torch.cuda.empty_cache()
+
+
+@pytest.mark.parametrize("K", [32, 64])
+def test_attention_layer_on_the_headline_pattern_at_full_size(K):
+    """The attention layer of the R-MAT 2^20 workload (out_e = A_e <X_i, Y_j> with row-normalised X, Y; softmax over
+    each row; SpMM with H [n, 32]) at full size, fused (SDDMM with row maxima -> softmax-weighted SpMM) and as three
+    steps, row-split and plain:
+      * the softmax weights of a row sum to one, so H = ones must come back as ones in every row (to 1e-5 plus the
+        drift of a chain of that many fp32 additions);
+      * a float64 restatement on a row sample (first and last 4096 rows and the 64 longest rows, up to ~60 k entries);
+      * the four paths agree."""
+    import paramspmm_ae_amd  # noqa: F401  (puts lib/ on sys.path)
+    import ParamSDDMM
+    import ParamSpMM
+    from paramspmm_ae_amd import _capi, synth
+    from paramspmm_ae_amd.graph_input import graph_input
+
+    rowPtr, colIdx, val, n = synth.config_graph("C2")
+    g = graph_input("C2", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val)
+    c = g.csr_data
+    rp, ci, v = c.on_device("rowPtr", "cuda"), c.on_device("colIdx", "cuda"), c.on_device("val", "cuda")
+    rps, tr = c.on_device("rowPtr_split", "cuda"), c.on_device("target_row", "cuda")
+    gen = torch.Generator(device="cuda").manual_seed(K)
+    X = torch.nn.functional.normalize(torch.randn(n, K, device="cuda", generator=gen), dim=1).contiguous()
+    Y = torch.nn.functional.normalize(torch.randn(n, K, device="cuda", generator=gen), dim=1).contiguous()
+    H = torch.randn(n, 32, device="cuda", generator=gen)
+    ones = torch.ones(n, 32, device="cuda")
+    bw_s = 4 | _capi.bw_stripe(c.xcd_stripe(True))
+    bw_p = 4 | _capi.bw_stripe(c.xcd_stripe(False))
+
+    def fused_split(D):
+        e, m = ParamSDDMM.csr_split_sddmm_scaled_rowmax(X, Y, rps, ci, v, tr, n, bw_s)
+        return ParamSpMM.csr_split_spmm_softmax(D, rps, ci, e, m, tr, 1, bw_s)
+
+    def fused_plain(D):
+        e, m = ParamSDDMM.csr_sddmm_scaled_rowmax(X, Y, rp, ci, v, bw_p | 0x100)
+        return ParamSpMM.csr_spmm_softmax(D, rp, ci, e, m, 1, bw_p)
+
+    def three_steps_split(D):
+        e = ParamSDDMM.csr_split_sddmm_scaled(X, Y, rps, ci, v, tr, bw_s)
+        return ParamSpMM.csr_split_spmm(D, rps, ci, ParamSDDMM.segment_softmax(rp, e), tr, 1, bw_s)
+
+    def three_steps_plain(D):
+        e = ParamSDDMM.csr_sddmm_scaled(X, Y, rp, ci, v, bw_p | 0x100)
+        return ParamSpMM.csr_spmm(D, rp, ci, ParamSDDMM.segment_softmax(rp, e), 1, bw_p)
+
+    paths = {"fused split": fused_split, "fused plain": fused_plain, "three steps split": three_steps_split,
+             "three steps plain": three_steps_plain}
+    # every row of this graph has its self loop, so every row has weights.  A row of k entries is summed in chains of
+    # about k/8 fp32 additions (the reference: one chain of k); with k nearly equal weights every addition rounds the
+    # same way, so the sum can drift by a fraction of an ulp per addition (measured: 3.2e-5 on the 41 k-entry row)
+    k_row = torch.from_numpy(np.diff(rowPtr).astype(np.float32)).cuda()
+    bound = (1e-5 + 4e-9 * k_row)[:, None]
+    for name, fn in paths.items():
+        print("case", K, name, "ones", flush=True)
+        back = fn(ones)
+        assert bool(((back - 1.0).abs() <= bound).all()), (name, float((back - 1.0).abs().max()))
+    rows = sample_rows(rowPtr)
+    Xh, Yh, Hh = X.cpu().double().numpy(), Y.cpu().double().numpy(), H.cpu().double().numpy()
+    want = np.zeros((rows.size, 32))
+    for t, i in enumerate(rows):
+        cols = colIdx[rowPtr[i]:rowPtr[i + 1]]
+        e = val[rowPtr[i]:rowPtr[i + 1]].astype(np.float64) * (Yh[cols] @ Xh[i])
+        w = np.exp(e - e.max())
+        want[t] = (w / w.sum()) @ Hh[cols]
+    idx = torch.from_numpy(rows).cuda()
+    results = {}
+    for name, fn in paths.items():
+        print("case", K, name, "sample", flush=True)
+        out = fn(H)
+        results[name] = out
+        got = out[idx].cpu().double().numpy()
+        assert np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 2e-6), (name, float(np.abs(got - want).max()))
+    ref = results["three steps plain"]
+    for name, out in results.items():
+        assert bool(((out - ref).abs() <= 2e-6 + 4.0 * bound * ref.abs()).all()), (name, float((out - ref).abs().max()))
