@@ -43,19 +43,27 @@ def dynamic_CF_prompter(dim, CF_set=None, warp_size=32, verbose=False):
 def native_CF_prompter(dim):
     """Configurations of the wave64 kernel that the reference's <CF, blkWarpNum> cannot express, as packed values
     for the ``CF`` argument (``_capi.pack_cf``; the operators pass CF through as an opaque int, PCSR.py:224-237):
-    lane groups of 16 and 32 lanes (4 and 2 sparse rows per wavefront, fewer column tiles) and the even division
-    of a wavefront's entries between its lane groups.  The list depends only on the 32-wide band of ``dim``, like
-    the forest that serves a width (decider.py:52-55), so both stay in step."""
+    lane groups of 16 and 32 lanes (4 and 2 sparse rows per wavefront, fewer column tiles), the even division of a
+    wavefront's entries between its lane groups, and light configurations -- one or two entries in flight per lane,
+    four-lane groups -- whose wavefronts need few registers, so that more of them are resident: on matrices with
+    short, regular rows whose gathers hit the caches (stencils, community-ordered graphs) residency beats loads in
+    flight per wavefront (measured 8-20 % at widths up to 128).  The list depends only on the 32-wide band of
+    ``dim``, like the forest that serves a width (decider.py:52-55), so both stay in step."""
     from ._capi import pack_cf
 
     band = math.ceil(dim / 32)
     if band <= 1:
-        return [pack_cf(1, 8 if dim > 16 else 4, 4, even_split=True)]
+        if dim <= 16:
+            return [pack_cf(1, 4, 4, even_split=True), pack_cf(1, 4, 2, even_split=True), pack_cf(1, 4, 1)]
+        return [pack_cf(1, 8, 4, even_split=True), pack_cf(2, 4, 2, even_split=True), pack_cf(2, 4, 1)]
     cf_max = dynamic_CF_prompter(band * 32)[-1]
     extra = [pack_cf(1, 16, 4), pack_cf(1, 8, 4, even_split=True),
              pack_cf(cf_max, 8, 2 if cf_max <= 4 else 1, even_split=True)]
     if band >= 4:
         extra.append(pack_cf(1, 32, 4))
+    if cf_max <= 4:
+        extra.append(pack_cf(cf_max, 8, 1, even_split=True))
+    extra.append(pack_cf(4, 4, 1, even_split=True))
     return extra
 
 

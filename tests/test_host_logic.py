@@ -279,11 +279,13 @@ def test_decider_round_trip_with_a_forest_trained_in_test(tmp_path):
     # a forest without a recorded CF axis was trained on the reference's table
     assert d.config_PCSR(G(lo), 64) == d.decode_tree(1, 64, CF_list=[1, 2]) == (1, 1, 1, 4)
     assert d.config_PCSR(G(hi), 64) == d.decode_tree(6, 64, CF_list=[1, 2]) == (0, 2, 2, 4)
-    # one that records the widened axis decodes over it: class 38 = blkWarpNum 8, fifth CF of the list, vec2
+    # one that records the widened axis decodes over it: blkWarpNum 8, fifth CF of the list, vec2 (and class 9:
+    # blkWarpNum 4, third CF, vec1_split)
     from paramspmm_ae_amd.PCSR import decider_CF_list
 
     wide = decider_CF_list(64)
-    clf2 = RandomForestClassifier(n_estimators=5, random_state=0).fit(X, np.where(X[:, 0] > 0.5, 38, 9))
+    code_hi = 4 * len(wide) + 4 * 4 + 2
+    clf2 = RandomForestClassifier(n_estimators=5, random_state=0).fit(X, np.where(X[:, 0] > 0.5, code_hi, 9))
     clf2.psp_cf_list_ = wide
     with open(tmp_path / "rnd_tree_64.pkl", "wb") as f:
         pickle.dump(clf2, f)
