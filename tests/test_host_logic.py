@@ -475,3 +475,25 @@ def test_xcd_stripe_levels_a_matrix_whose_long_rows_cluster():
     # an empty matrix and one too small for two rounds of stripes leave the choice to the library
     small = gi.csr_data(np.arange(101, dtype=np.int32), np.zeros(100, np.int32), np.ones(100, np.float32), 100, 100)
     assert small.xcd_stripe(False) == 0 and small.xcd_stripe(True) == 0
+
+
+def test_every_configuration_of_the_deciders_list_has_a_plan():
+    """The CF axis of the decider's class space (the reference's list followed by the native configurations) at every
+    width a forest serves: each entry maps onto the wave64 kernel, covers the width with its column tiles, and the
+    native ones keep what they ask for; widths of one band share one list."""
+    from paramspmm_ae_amd import _capi
+    from paramspmm_ae_amd.PCSR import decider_CF_list, dynamic_CF_prompter, native_CF_prompter
+
+    for dim in range(16, 257, 16):
+        cfs = decider_CF_list(dim)
+        assert cfs[: len(dynamic_CF_prompter(dim))] == dynamic_CF_prompter(dim) and len(set(cfs)) == len(cfs)
+        assert native_CF_prompter(dim) == native_CF_prompter((dim + 31) // 32 * 32)
+        for cf in cfs:
+            for bw in (4, 8):
+                p = _capi.spmm_plan(dim, cf, bw)
+                assert p["lanes_per_row"] * p["coarsen"] * p["vec"] * p["col_tiles"] >= dim
+                assert p["rows_per_wave"] * p["lanes_per_row"] == 64 and 1 <= p["unroll"] <= p["lanes_per_row"]
+                u = _capi.unpack_cf(cf)
+                if u is not None:
+                    c, lanes, unroll, segs, even = u
+                    assert (p["coarsen"], p["lanes_per_row"], p["unroll"], p["even_split"]) == (min(c, dim // 4), lanes, unroll, int(even))
