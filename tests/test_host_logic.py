@@ -480,14 +480,14 @@ def test_xcd_stripe_levels_a_matrix_whose_long_rows_cluster():
 def test_every_configuration_of_the_deciders_list_has_a_plan():
     """The CF axis of the decider's class space (the reference's list followed by the native configurations) at every
     width a forest serves: each entry maps onto the wave64 kernel, covers the width with its column tiles, and the
-    native ones keep what they ask for; widths of one band share one list."""
+    native ones keep what they ask for; the widths one forest serves share one list."""
     from paramspmm_ae_amd import _capi
     from paramspmm_ae_amd.PCSR import decider_CF_list, dynamic_CF_prompter, native_CF_prompter
 
     for dim in range(16, 257, 16):
         cfs = decider_CF_list(dim)
         assert cfs[: len(dynamic_CF_prompter(dim))] == dynamic_CF_prompter(dim) and len(set(cfs)) == len(cfs)
-        assert native_CF_prompter(dim) == native_CF_prompter((dim + 31) // 32 * 32)
+        assert native_CF_prompter(dim) == native_CF_prompter(dim - 15)  # the widths one forest serves share a list
         for cf in cfs:
             for bw in (4, 8):
                 p = _capi.spmm_plan(dim, cf, bw)
