@@ -64,8 +64,9 @@ typedef struct psp_spmm_plan {
 } psp_spmm_plan;
 int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan);
 
-/* SpMM and SDDMM entry points (row-wise walks), blkWarpNum | PSP_BW_STRIPE(rows): this launch deals `rows` consecutive rows (segments, block-rows)
- * to one XCD at a time instead of the library option "xcd_stripe_rows".  rows = a multiple of 256 up to 65280 (the field
+/* SpMM and SDDMM entry points (row-wise walks), blkWarpNum | PSP_BW_STRIPE(rows): this launch deals `rows`
+ * consecutive rows (segments, block-rows) to one XCD at a time instead of the library option "xcd_stripe_rows".
+ * rows = a multiple of 256 up to 65280 (the field
  * holds rows / 256 in bits 12..19; 0 = the option).  The reference has no counterpart (one L2 on its GPUs): a caller
  * that knows the matrix picks the longest stripe that still gives the eight XCDs equal shares of the stored entries
  * (graph_input does: csr_data.xcd_stripe), long stripes keeping neighbouring rows -- and the X rows they share -- in
