@@ -326,14 +326,17 @@ class pcsr_spmm(object):
     def gespmm_ref(self, dim=None, x=None, is_profiling=False, verbose=True):
         return self._vendor("gespmm_compute", "gespmm_profile", "gespmm", dim, x, is_profiling, verbose)
 
-    def time_ms(self, X, CF=None, blkWarpNum=None, warmup=5, iters=20):
-        """Mean milliseconds per SpMM launch (an addition of this build; used by the sweep harness)."""
+    def time_ms(self, X, CF=None, blkWarpNum=None, warmup=5, iters=20, flush_bytes=0):
+        """Mean milliseconds per SpMM launch (an addition of this build; used by the sweep harness).  ``flush_bytes``:
+        fill that much scratch memory before every timed launch, so that the operands come from HBM as inside a
+        training step instead of from the caches the previous, identical launch left warm."""
         if self.vec_size == 3:
             raise NotImplementedError("time_ms covers the four decider formats; use cf_warpnum_profiling for 3x1 blocks")
         fmt = (1 if self.if_split else 0) + (2 if self.vec_size != 1 else 0)
         return SpMM.spmm_time_ms(fmt, X, self.rowPtr, self.colIdx, self.val, self.target_row,
                                  self.CF if CF is None else CF,
-                                 (self.blkWarpNum if blkWarpNum is None else blkWarpNum) | self.bw_flags, warmup, iters)
+                                 (self.blkWarpNum if blkWarpNum is None else blkWarpNum) | self.bw_flags, warmup, iters,
+                                 int(flush_bytes))
 
 
 # ---- training-set construction: `python -m paramspmm_ae_amd.PCSR` (PCSR.py:660-871) -----------------------------

@@ -97,8 +97,12 @@ static int bcsr_split_spmm_profile(Tensor input, Tensor rowPtr_bcsr_split, Tenso
 }
 
 // ---- explicit timing helper of this build: median-free mean over a caller-chosen iteration count -----
+// flush_bytes > 0: every timed launch is preceded by a fill of that many bytes of scratch memory and timed on its
+// own (the sum of the launches' own durations is reported), so that the operands come from HBM as they do inside a
+// training step; 0 repeats the launch back to back, as the reference's *_profile loop does.
 static double spmm_time_ms(int fmt, Tensor input, Tensor rowPtr, Tensor colIdx, Tensor values,
-                           c10::optional<Tensor> target_row, int CF, int blkWarpNum, int warmup, int iters)
+                           c10::optional<Tensor> target_row, int CF, int blkWarpNum, int warmup, int iters,
+                           int64_t flush_bytes)
 {
     TORCH_CHECK(fmt >= 0 && fmt <= 3, "fmt must be 0 (csr), 1 (csr_split), 2 (bcsr) or 3 (bcsr_split)");
     TORCH_CHECK((fmt & 1) == (target_row.has_value() ? 1 : 0), "target_row must be given exactly for split formats");
@@ -109,8 +113,27 @@ static double spmm_time_ms(int fmt, Tensor input, Tensor rowPtr, Tensor colIdx, 
     const long rows_out = fmt >= 2 ? (input.size(0) + 1) / 2 * 2 : input.size(0);
     auto Y = torch::empty({rows_out, input.size(1)}, input.options());
     hipStream_t s = (hipStream_t)stream_of(input);
-    return (double)time_launches(s, warmup, iters,
-                                 [&] { spmm_into(fmt, Y, input, rowPtr, colIdx, values, tr, CF, blkWarpNum); });
+    auto launch = [&] { spmm_into(fmt, Y, input, rowPtr, colIdx, values, tr, CF, blkWarpNum); };
+    if (flush_bytes <= 0) return (double)time_launches(s, warmup, iters, launch);
+    auto scratch = torch::empty({flush_bytes / 4}, input.options().dtype(torch::kFloat32));
+    hipEvent_t e0, e1;
+    TORCH_CHECK(hipEventCreate(&e0) == hipSuccess && hipEventCreate(&e1) == hipSuccess, "hipEventCreate failed");
+    for (int i = 0; i < warmup; i++) launch();
+    double total = 0.0;
+    bool good = true;
+    for (int i = 0; i < iters && good; i++) {
+        scratch.fill_((float)i);
+        good = good && hipEventRecord(e0, s) == hipSuccess;
+        launch();
+        good = good && hipEventRecord(e1, s) == hipSuccess && hipEventSynchronize(e1) == hipSuccess;
+        float ms = 0.f;
+        good = good && hipEventElapsedTime(&ms, e0, e1) == hipSuccess;
+        total += ms;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    TORCH_CHECK(good, "timing the launches failed: ", hipGetErrorString(hipGetLastError()));
+    return total / (double)iters;
 }
 
 // ---- generic vec_size x 1 blocks (SpMM/SpMM.cpp:339-480, 757-889) --------------------------------------------------
@@ -300,7 +323,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("csr_spmm_softmax", &csr_spmm_softmax, "softmax_rows(e) * X: (X, rowPtr, colIdx, e, row_max, CF, blkWarpNum)");
     m.def("csr_split_spmm_softmax", &csr_split_spmm_softmax,
           "the same on the row-split format: (X, rowPtr_split, colIdx, e, row_max, target_row, CF, blkWarpNum)");
-    m.def("spmm_time_ms", &spmm_time_ms, "mean ms per launch: (fmt, X, rowPtr, colIdx, val, target_row|None, CF, bw, warmup, iters)");
+    m.def("spmm_time_ms", &spmm_time_ms, "mean ms per launch: (fmt, X, rowPtr, colIdx, val, target_row|None, CF, bw, warmup, iters, flush_bytes=0)",
+          py::arg("fmt"), py::arg("X"), py::arg("rowPtr"), py::arg("colIdx"), py::arg("val"), py::arg("target_row"), py::arg("CF"),
+          py::arg("blkWarpNum"), py::arg("warmup"), py::arg("iters"), py::arg("flush_bytes") = 0);
     m.def("vendor_spmm_time_ms", &vendor_spmm_time_ms, "mean ms per rocSPARSE SpMM: (format, X, idx_a, idx_b, val, warmup, iters)");
     m.def("spmm_plan", &spmm_plan, "how (N, CF, blkWarpNum) maps onto the wave64 kernel");
 }

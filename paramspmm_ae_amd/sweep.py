@@ -41,11 +41,11 @@ def operators_of(graph, vec_size=2):
     return [pcsr_spmm(graph, vec_size=v if v == 1 else vec_size, if_split=s) for _, v, s in REPRESENTATIONS]
 
 
-def sweep_dim(ops, dim, nnz, n_rows, warmup=3, iters=10, X=None, verify=None, cfs=None):
+def sweep_dim(ops, dim, nnz, n_rows, warmup=3, iters=10, X=None, verify=None, cfs=None, flush_bytes=0):
     """Times all columns for one width.  Returns (ms[cols], gflops[cols]).
 
     ``verify``: optional callable(result_tensor, column_name) run once per column on A*X before timing
-    (the reference verifies every swept configuration, PCSR.py:759-770).
+    (the reference verifies every swept configuration, PCSR.py:759-770).  ``flush_bytes``: see pcsr_spmm.time_ms.
     """
     pad = max(op.vec_size for op in ops)
     pad = 2 if pad == 1 else pad
@@ -64,7 +64,7 @@ def sweep_dim(ops, dim, nnz, n_rows, warmup=3, iters=10, X=None, verify=None, cf
                 if op.vec_size == 3:  # the generic-block operators have no event-timed twin: use their *_profile
                     ms[col] = 2.0 * nnz * dim / 1e6 / max(op.cf_warpnum_profiling(cf, bw, x=X, verbose=False), 1)
                 else:
-                    ms[col] = op.time_ms(X, CF=cf, blkWarpNum=bw, warmup=warmup, iters=iters)
+                    ms[col] = op.time_ms(X, CF=cf, blkWarpNum=bw, warmup=warmup, iters=iters, flush_bytes=flush_bytes)
                 col += 1
     gflops = 2.0 * nnz * dim / 1e6 / ms
     return ms, gflops

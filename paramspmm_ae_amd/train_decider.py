@@ -151,7 +151,9 @@ def sweep_main(args):
     os.makedirs(args.out, exist_ok=True)
     tag = "" if nparts == 1 else "_part%d" % part
     info_rows, names = [], []
-    tp = {d: [] for d in DIMS}
+    dims = [int(d) for d in args.dims.split(",")] if args.dims else DIMS
+    flush_bytes = int(args.flush_mb) << 20
+    tp = {d: [] for d in dims}
     t_start = time.time()
     for idx, (name, build) in enumerate(items):
         t0 = time.time()
@@ -173,8 +175,8 @@ def sweep_main(args):
             err = (op._spmm(X)[:n] - ref).abs().max().item()
             assert err <= 1e-4 * scale, (name, err, scale)
         del X, ref
-        for d in DIMS:
-            ms, gf = sw.sweep_dim(ops, d, nnz, n, warmup=args.warmup, iters=args.iters)
+        for d in dims:
+            ms, gf = sw.sweep_dim(ops, d, nnz, n, warmup=args.warmup, iters=args.iters, flush_bytes=flush_bytes)
             tp[d].append(gf)
         info_rows.append([name] + g._feature_values())
         names.append(name)
@@ -186,7 +188,7 @@ def sweep_main(args):
         info = pd.DataFrame(info_rows, columns=["mtx_name"] + FEATURES)
         info.to_csv(os.path.join(args.out, "mtx_info%s.csv" % tag), index=False)
         if (idx + 1) % 10 == 0 or idx + 1 == len(items):
-            for d in DIMS:
+            for d in dims:
                 pd.DataFrame(np.array(tp[d]), columns=sw.column_names(d)).to_csv(
                     os.path.join(args.out, "dim%d%s.csv" % (d, tag)), index=False)
 
@@ -194,24 +196,25 @@ def sweep_main(args):
 # ------------------------------------------------------------------------------------------------------------
 # fit (CPU)
 # ------------------------------------------------------------------------------------------------------------
-def load_training_data(data_dir):
+def load_training_data(data_dir, dims=None):
     import glob
 
     import pandas as pd
 
     info_files = sorted(glob.glob(os.path.join(data_dir, "mtx_info*.csv")))
     assert info_files, "no mtx_info*.csv under " + data_dir
-    infos, tps = [], {d: [] for d in DIMS}
+    dims = DIMS if dims is None else dims
+    infos, tps = [], {d: [] for d in dims}
     for f in info_files:
         tag = os.path.basename(f)[len("mtx_info"):-len(".csv")]
         info = pd.read_csv(f)
-        per_dim = {d: pd.read_csv(os.path.join(data_dir, "dim%d%s.csv" % (d, tag))) for d in DIMS}
+        per_dim = {d: pd.read_csv(os.path.join(data_dir, "dim%d%s.csv" % (d, tag))) for d in dims}
         rows = min([len(info)] + [len(v) for v in per_dim.values()])
         infos.append(info.iloc[:rows])
-        for d in DIMS:
+        for d in dims:
             tps[d].append(per_dim[d].iloc[:rows])
     info = pd.concat(infos, ignore_index=True)
-    return info, {d: pd.concat(tps[d], ignore_index=True) for d in DIMS}
+    return info, {d: pd.concat(tps[d], ignore_index=True) for d in dims}
 
 
 def _fit_forest(X, TP, near, n_est, leaves):
@@ -247,7 +250,8 @@ def fit_main(args):
     import pandas as pd
     from sklearn.model_selection import GroupKFold
 
-    info, tps = load_training_data(args.data)
+    dims = [int(d) for d in args.dims.split(",")] if args.dims else DIMS
+    info, tps = load_training_data(args.data, dims)
     X = info[FEATURES].to_numpy(dtype=np.float64)
     os.makedirs(args.out, exist_ok=True)
     groups = np.array([family(n) for n in info["mtx_name"]])
@@ -259,8 +263,12 @@ def fit_main(args):
     from . import sweep as sw
     from .PCSR import decider_CF_list, dynamic_CF_prompter
 
+    report_path = os.path.join(args.out, "decider_report.json")
+    if args.dims and os.path.exists(report_path):  # a partial refit keeps the other widths' entries
+        with open(report_path) as f:
+            report["per_dim"] = {int(k): v for k, v in json.load(f)["per_dim"].items()}
     cf_lists = {}
-    for d in DIMS:
+    for d in dims:
         # the table's CF axis: the widened list, or the reference's own when the data come from its sweep
         if list(tps[d].columns) == sw.column_names(d):
             cf_lists[d] = decider_CF_list(d)
@@ -320,7 +328,8 @@ def fit_main(args):
     allw = [v["share_within_10pct_of_best"] for v in report["per_dim"].values()]
     report["share_within_10pct_mean"] = float(np.mean(allw))
     report["share_within_10pct_min"] = float(np.min(allw))
-    with open(os.path.join(args.out, "decider_report.json"), "w") as f:
+    report["per_dim"] = {str(k): report["per_dim"][k] for k in sorted(report["per_dim"], key=int)}
+    with open(report_path, "w") as f:
         json.dump(report, f, indent=1)
     print("matrices %d; within 10%% of best: mean %.3f, min over widths %.3f" % (len(info), np.mean(allw), np.min(allw)))
 
@@ -334,10 +343,15 @@ def main(argv=None):
     s.add_argument("--limit", type=int, default=0)
     s.add_argument("--warmup", type=int, default=2)
     s.add_argument("--iters", type=int, default=6)
+    s.add_argument("--dims", default="", help="comma-separated widths (default: all of 16..256)")
+    s.add_argument("--flush_mb", type=int, default=0,
+                   help="fill this many MiB of scratch memory before every timed launch (operands from HBM, as inside a "
+                        "training step) instead of repeating the launch back to back")
     f = sub.add_parser("fit")
     here = os.path.dirname(os.path.abspath(__file__))
     f.add_argument("--data", default=os.path.join(here, "models", "train_data"))
     f.add_argument("--out", default=os.path.join(here, "models"))
+    f.add_argument("--dims", default="", help="refit these widths only (comma-separated); the report keeps the others")
     ls = sub.add_parser("list")
     args = ap.parse_args(argv)
     if args.cmd == "sweep":
