@@ -606,25 +606,31 @@ def main():
         width.  Returns (wall seconds, {width: [(start event, stop event)]})."""
         launch = {d: launcher(d, ops_, chosen_) for d in dims}
 
-        def step(events=None):
+        def step(events=None, k=0):
             for d in dims:
                 if events is not None:
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0, e1 = events[d][k]
                     e0.record()
                 rc = launch[d]()
                 if events is not None:
                     e1.record()
-                    events[d].append((e0, e1))
                 if rc != 0:
                     _capi.check(rc)
 
         for _ in range(args.warmup):
             step()
+        # the events exist before the clock starts (an event is created by its first record): on a small graph the
+        # timed region would otherwise measure the host creating them
+        events_ = {d: [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+                       for _ in range(args.steps)] for d in dims}
+        for pairs in events_.values():
+            for e0, e1 in pairs:
+                e0.record()
+                e1.record()
         torch.cuda.synchronize()
-        events_ = {d: [] for d in dims}
         t0_ = time.perf_counter()
-        for _ in range(args.steps):
-            step(events_)
+        for k in range(args.steps):
+            step(events_, k)
         torch.cuda.synchronize()
         return time.perf_counter() - t0_, events_
 
