@@ -497,3 +497,62 @@ def test_every_configuration_of_the_deciders_list_has_a_plan():
                 if u is not None:
                     c, lanes, unroll, segs, even = u
                     assert (p["coarsen"], p["lanes_per_row"], p["unroll"], p["even_split"]) == (min(c, dim // 4), lanes, unroll, int(even))
+
+
+def test_decider_fit_on_a_small_table_and_partial_refit_keeps_the_other_widths(tmp_path):
+    """train_decider fit: label files in the reference's schema (PCSR.py:815-818), one forest per width that
+    SpMMDecider loads and decodes to a configuration of that width's list, and a refit of one width (--dims) that
+    leaves the other widths' report entries in place."""
+    import json
+
+    import pandas as pd
+
+    from paramspmm_ae_amd import _capi, sweep, train_decider
+    from paramspmm_ae_amd.decider import SpMMDecider
+    from paramspmm_ae_amd.PCSR import decider_CF_list
+
+    rng = np.random.default_rng(5)
+    data, out = tmp_path / "data", tmp_path / "models"
+    data.mkdir()
+    names = ["%s_n%d_d%d_s%d" % (fam, 1000 * (i + 1), 3 + i, s) for fam in ("cl", "sbm", "band") for i in range(5) for s in range(3)]
+    feats = pd.DataFrame(rng.random((len(names), len(train_decider.FEATURES))), columns=train_decider.FEATURES)
+    pd.concat([pd.DataFrame({"mtx_name": names}), feats], axis=1).to_csv(data / "mtx_info_part0.csv", index=False)
+    for d in (16, 32):
+        cols = sweep.column_names(d)
+        tp = 100.0 + rng.random((len(names), len(cols)))
+        # the first feature decides between two columns, so there is something to learn
+        tp[np.arange(len(names)), np.where(feats.iloc[:, 0] > 0.5, 1, len(cols) - 2)] += 50.0
+        pd.DataFrame(tp, columns=cols).to_csv(data / ("dim%d_part0.csv" % d), index=False)
+
+    train_decider.main(["fit", "--data", str(data), "--out", str(out), "--dims", "16"])
+    report = json.load(open(out / "decider_report.json"))
+    assert list(report["per_dim"]) == ["16"] and report["matrices"] == len(names)
+    train_decider.main(["fit", "--data", str(data), "--out", str(out), "--dims", "32"])
+    report = json.load(open(out / "decider_report.json"))
+    assert list(report["per_dim"]) == ["16", "32"]
+    assert report["per_dim"]["16"]["classes"] == len(sweep.column_names(16))
+
+    labels = pd.read_csv(data / "dim32_OP_SpMM.csv")
+    assert list(labels.columns) == ["mtx_name"] + train_decider.FEATURES + ["OP_SpMM"]
+    want = np.where(feats.iloc[:, 0] > 0.5, 1, len(sweep.column_names(32)) - 2)
+    assert (labels["OP_SpMM"].to_numpy() == want).all()
+
+    dec = SpMMDecider(str(out) + os.sep)
+    dec.gen_model_dict([16, 32])
+
+    class G:  # what config_PCSR reads of a graph_input
+        def __init__(self, row):
+            self.row = row
+
+        def get_info(self):
+            return np.asarray(self.row, dtype=np.float64).reshape(1, -1)
+
+    for d in (16, 32):
+        hits = 0
+        for i in range(len(names)):
+            if_split, vec, cf, bw = dec.config_PCSR(G(feats.iloc[i].to_numpy()), d)
+            assert cf in decider_CF_list(d) and bw in (4, 8) and vec in (1, 2)
+            _capi.spmm_plan(d, cf, bw)  # every decoded configuration has a plan
+            col = [c for c in range(len(sweep.column_names(d))) if sweep.decode_column(d, c) == (if_split, vec, cf, bw)][0]
+            hits += col == (1 if feats.iloc[i, 0] > 0.5 else len(sweep.column_names(d)) - 2)
+        assert hits >= 0.9 * len(names)  # refitted on every matrix: the rule is learnt
