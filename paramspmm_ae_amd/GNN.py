@@ -218,13 +218,25 @@ def build_model(net, graph, operators, hidden, num_features, num_classes, num_la
     return GIN(num_classes, num_features, graph.x, operators, hidden).to(device)
 
 
-def configure_operators(decider, graph, dims, override=None):
+def configure_operators(decider, graph, dims, override=None, try_candidates=0):
     """One pcsr_spmm per layer width, configured by the decider (GNN.py:200-209) or by ``override`` =
-    (if_split, vec_size, CF, blkWarpNum)."""
+    (if_split, vec_size, CF, blkWarpNum).  ``try_candidates`` = k > 1 (an addition of this build): the k configurations
+    the forest rates highest are timed on this matrix (a few launches each, after a cache fill, as inside an epoch) and
+    the fastest is kept."""
     ops = {}
     for dim in dims:
-        if_split, vec_size, CF, blkWarpNum = override if override is not None else decider.config_PCSR(graph, dim)
-        ops[dim] = pcsr_spmm(graph=graph, vec_size=vec_size, if_split=if_split, CF=CF, blkWarpNum=blkWarpNum)
+        if override is not None or try_candidates <= 1:
+            if_split, vec_size, CF, blkWarpNum = override if override is not None else decider.config_PCSR(graph, dim)
+            ops[dim] = pcsr_spmm(graph=graph, vec_size=vec_size, if_split=if_split, CF=CF, blkWarpNum=blkWarpNum)
+            continue
+        X = torch.randn((graph.mtx_nodes + 1) // 2 * 2, dim, device="cuda")  # an even row count serves the 2x1 block formats too
+        best = None
+        for if_split, vec_size, CF, blkWarpNum in decider.candidates_PCSR(graph, dim, try_candidates):
+            op = pcsr_spmm(graph=graph, vec_size=vec_size, if_split=if_split, CF=CF, blkWarpNum=blkWarpNum)
+            ms = op.time_ms(X, warmup=2, iters=5, flush_bytes=256 << 20)
+            if best is None or ms < best[0]:
+                best = (ms, op)
+        ops[dim] = best[1]
     return ops
 
 
@@ -250,6 +262,8 @@ def main(argv=None):
                    help="GCN: always A (H W), also for the first layer when it widens its input (the reference's order)")
     p.add_argument("--no_fuse_relu", action="store_true",
                    help="apply the ReLU between the layers as passes of their own, as the reference's driver does")
+    p.add_argument("--try_candidates", type=int, default=0, metavar="K",
+                   help="time the K configurations the decider rates highest on the matrix and keep the fastest")
     p.add_argument("--config", nargs=4, type=int, default=None, metavar=("IF_SPLIT", "VEC", "CF", "BW"),
                    help="skip the decider and use this configuration for every layer width")
     args = p.parse_args(argv)
@@ -281,7 +295,8 @@ def main(argv=None):
                 dims.append(args.num_features)  # the first layer runs its sparse product at the features' width
             if args.net == "GIN" and args.num_features not in dims and (decider is None or args.num_features in decider.model_dict):
                 dims.append(args.num_features)  # GIN aggregates its input: the first layer's product has the features' width
-            ops = configure_operators(decider, graph, dims, None if args.config is None else tuple(args.config))
+            ops = configure_operators(decider, graph, dims, None if args.config is None else tuple(args.config),
+                                      try_candidates=args.try_candidates)
             print("SpMM-decider config time: {:.3f} (ms)".format((time.perf_counter() - t1) * 1e3))
             model = build_model(args.net, graph, ops, hidden, args.num_features, args.num_classes, args.num_layers)
             if args.no_fuse_relu and hasattr(model, "fuse_relu"):

@@ -72,6 +72,21 @@ class SpMMDecider(object):
         cf_list = getattr(model, "psp_cf_list_", None)
         return self.decode_tree(code, rounded, CF_list=dynamic_CF_prompter(rounded) if cf_list is None else list(cf_list))
 
+    def candidates_PCSR(self, graph, dim, k=3):
+        """The ``k`` configurations the forest rates highest for this matrix, best first (an addition of this build: the
+        first one is ``config_PCSR``'s answer; ``GNN.configure_operators(..., try_candidates=k)`` times them on the
+        matrix itself and keeps the fastest, which bounds the cost of a wrong first guess)."""
+        if dim not in self.model_dict:
+            raise ValueError("dim-" + str(dim) + " not found in model_dict")
+        model = self.model_dict[dim]
+        proba = model.predict_proba(graph.get_info())[0]
+        first = model.predict(graph.get_info()).item()
+        order = sorted(range(len(proba)), key=lambda i: (model.classes_[i] != first, -proba[i]))
+        rounded = math.ceil(dim / 16) * 16
+        cf_list = getattr(model, "psp_cf_list_", None)
+        cf_list = dynamic_CF_prompter(rounded) if cf_list is None else list(cf_list)
+        return [self.decode_tree(model.classes_[i], rounded, CF_list=cf_list) for i in order[:max(1, k)] if proba[i] > 0 or model.classes_[i] == first]
+
 
 def evaluate(filelist, path, dim_list, pickle_path=DEFAULT_PICKLE_PATH, verbose=True):
     """The reference's evaluation run (decider.py:97-175): for every matrix and width the decider's configuration is

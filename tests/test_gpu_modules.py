@@ -788,3 +788,29 @@ def test_gin_and_agnn_networks_with_folded_relu_equal_the_plain_ones(net, hidden
     assert abs(grads[True][0] - grads[False][0]) <= 1e-4 * abs(grads[False][0])
     for a, b in zip(grads[True][1], grads[False][1]):
         torch.testing.assert_close(a, b, rtol=2e-3, atol=1e-4 * float(b.abs().max()) + 1e-6)
+
+
+def test_operators_chosen_among_the_deciders_candidates_compute_the_product():
+    """configure_operators(try_candidates=3): the operator kept for every width is one of the forest's three
+    highest-rated configurations (the first being the decider's own answer) and computes A X (checked against
+    torch.sparse.mm in double precision); an odd row count exercises the padded input of the block formats."""
+    from paramspmm_ae_amd import GNN
+    from paramspmm_ae_amd.decider import SpMMDecider
+
+    n = 30001
+    g, rowPtr, colIdx, val = sym_graph(n, 21)
+    dec = SpMMDecider()
+    dims = [16, 48, 128]
+    dec.gen_model_dict(dims)
+    ops = GNN.configure_operators(dec, g, dims, try_candidates=3)
+    rows = torch.from_numpy(np.repeat(np.arange(n), np.diff(rowPtr)))
+    A = torch.sparse_coo_tensor(torch.stack([rows, torch.from_numpy(colIdx.astype(np.int64))]),
+                                torch.from_numpy(val.astype(np.float64)), (n, n)).cuda()
+    for d in dims:
+        op = ops[d]
+        cands = dec.candidates_PCSR(g, d, 3)
+        assert (int(op.if_split), op.vec_size, op.CF, op.blkWarpNum) in [(int(s), v, c, b) for s, v, c, b in cands]
+        X = torch.randn(n, d, device="cuda")
+        got = op._spmm(X)[:n]
+        want = torch.sparse.mm(A, X.double())
+        assert (got.double() - want).abs().max().item() <= 1e-5 * want.abs().max().item() + 1e-6

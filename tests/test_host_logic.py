@@ -556,3 +556,43 @@ def test_decider_fit_on_a_small_table_and_partial_refit_keeps_the_other_widths(t
             col = [c for c in range(len(sweep.column_names(d))) if sweep.decode_column(d, c) == (if_split, vec, cf, bw)][0]
             hits += col == (1 if feats.iloc[i, 0] > 0.5 else len(sweep.column_names(d)) - 2)
         assert hits >= 0.9 * len(names)  # refitted on every matrix: the rule is learnt
+
+
+def test_decider_candidates_start_with_the_pick_and_are_distinct(tmp_path):
+    """candidates_PCSR: the forest's k most probable classes, decoded; the first is config_PCSR's answer."""
+    import pickle
+
+    from sklearn.ensemble import RandomForestClassifier
+
+    from paramspmm_ae_amd.decider import SpMMDecider
+    from paramspmm_ae_amd.PCSR import decider_CF_list
+
+    rng = np.random.default_rng(11)
+    dim = 64
+    n_classes = 4 * len(decider_CF_list(dim)) * 2
+    Xf = rng.random((300, 15))
+    y = (Xf[:, 0] * 3).astype(int) * 5 + (Xf[:, 1] > 0.5)  # six classes out of the table's n_classes
+    assert y.max() < n_classes
+    forest = RandomForestClassifier(n_estimators=20, max_leaf_nodes=8, random_state=0).fit(Xf, y)
+    forest.psp_cf_list_ = [int(c) for c in decider_CF_list(dim)]
+    with open(tmp_path / "rnd_tree_64.pkl", "wb") as f:
+        pickle.dump(forest, f)
+    dec = SpMMDecider(str(tmp_path) + os.sep)
+    dec.gen_model_dict([dim])
+
+    class G:
+        def __init__(self, row):
+            self.row = row
+
+        def get_info(self):
+            return self.row.reshape(1, -1)
+
+    for i in range(20):
+        g = G(Xf[i])
+        cands = dec.candidates_PCSR(g, dim, 3)
+        assert 1 <= len(cands) <= 3 and len(set(cands)) == len(cands)
+        assert cands[0] == dec.config_PCSR(g, dim)
+        assert dec.candidates_PCSR(g, dim, 1) == cands[:1]
+        codes = set(forest.classes_)
+        for c in cands:  # every candidate is a class the forest knows
+            assert any(dec.decode_tree(code, dim) == c for code in codes)
