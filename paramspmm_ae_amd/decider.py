@@ -79,13 +79,17 @@ class SpMMDecider(object):
         if dim not in self.model_dict:
             raise ValueError("dim-" + str(dim) + " not found in model_dict")
         model = self.model_dict[dim]
-        proba = model.predict_proba(graph.get_info())[0]
-        first = model.predict(graph.get_info()).item()
+        info = graph.get_info()
+        proba = model.predict_proba(info)[0]
+        first = model.predict(info).item()
+        # the predicted class leads (ties in probability are broken the way predict() breaks them), then by rating;
+        # classes no tree voted for are not candidates
         order = sorted(range(len(proba)), key=lambda i: (model.classes_[i] != first, -proba[i]))
+        codes = [model.classes_[i] for i in order if proba[i] > 0 or model.classes_[i] == first][:max(1, k)]
         rounded = math.ceil(dim / 16) * 16
         cf_list = getattr(model, "psp_cf_list_", None)
         cf_list = dynamic_CF_prompter(rounded) if cf_list is None else list(cf_list)
-        return [self.decode_tree(model.classes_[i], rounded, CF_list=cf_list) for i in order[:max(1, k)] if proba[i] > 0 or model.classes_[i] == first]
+        return [self.decode_tree(code, rounded, CF_list=cf_list) for code in codes]
 
 
 def evaluate(filelist, path, dim_list, pickle_path=DEFAULT_PICKLE_PATH, verbose=True):
