@@ -1,11 +1,14 @@
 """SpMM-decider: per-dimension random forests that pick ``<if_split, vec_size, CF, blkWarpNum>`` from the 15
 matrix features (same surface as the reference's decider.py:18-93).
 
-The forests are the ones trained on MI355X timings by ``train_decider.py`` and stored as
-``rnd_tree_<dim>.pkl`` (one per multiple of 16 up to 256).  The class code is the column index of the sweep
-table: blkWarpNum-major, then CF in ``decider_CF_list(dim)`` order (the reference's ``dynamic_CF_prompter`` list
-followed by native wave64 configurations packed into the same integer), then the four representations
-(vec1, vec1_split, vec2, vec2_split) -- see ``decode_tree``.
+The forests are trained on MI355X timings by ``train_decider.py`` and stored as ``rnd_tree_<dim>.pkl`` (one per
+multiple of 16 up to 256), in two sets.  ``models/`` holds forests on the reference's own class space (class code =
+column index of the reference's sweep table: blkWarpNum-major, then CF in ``dynamic_CF_prompter(dim)`` order, then
+the four representations vec1, vec1_split, vec2, vec2_split): plain pickles that the reference's unchanged
+decider.py loads and decodes.  ``models/native/`` holds forests on the widened space, whose CF axis is
+``decider_CF_list(dim)`` -- the reference's list followed by native wave64 configurations packed into the same
+integer -- and who carry that axis as ``psp_cf_list_``; they are this class's default.  ``config_PCSR`` decodes
+either kind with the list the forest was trained on.
 """
 import math
 import os
@@ -14,7 +17,8 @@ import pickle
 
 from .PCSR import decider_CF_list, dynamic_CF_prompter
 
-DEFAULT_PICKLE_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "models") + os.sep
+REFERENCE_SPACE_PICKLE_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "models") + os.sep
+DEFAULT_PICKLE_PATH = os.path.join(REFERENCE_SPACE_PICKLE_PATH, "native") + os.sep
 
 
 def model_dim_for(dim):
@@ -37,7 +41,7 @@ class SpMMDecider(object):
             if not os.path.exists(pickle_file):
                 raise ValueError("pickle file not found for dim-" + str(dim) + " at path: " + pickle_file + "\n")
             with open(pickle_file, "rb") as f:
-                gz = f.read(2) == b"\x1f\x8b"  # the forests this package ships are gzip-compressed pickles
+                gz = f.read(2) == b"\x1f\x8b"  # gzip-compressed pickles are accepted as well
             with (gzip.open if gz else open)(pickle_file, "rb") as f:
                 self.tree_dict[dim] = pickle.load(f)
         return self.tree_dict[dim]
@@ -49,9 +53,10 @@ class SpMMDecider(object):
 
     def decode_tree(self, code, dim, vec_size_list=(1, 2), warpNum_list=(4, 8), CF_list=None):
         """class code -> (if_split, vec_size, CF, blkWarpNum) (decider.py:63-80); if_split is the int 0/1.
-        ``CF_list``: the CF axis the forest was trained on; default ``decider_CF_list(dim)`` (the reference's list
-        followed by the native configurations)."""
-        CF_list = decider_CF_list(dim) if CF_list is None else CF_list
+        ``CF_list``: the CF axis the forest was trained on; default ``dynamic_CF_prompter(dim)``, the reference's
+        (decider.py:69).  A forest on the widened space is decoded with ``decider_CF_list(dim)``, which
+        ``config_PCSR`` takes from the forest itself."""
+        CF_list = dynamic_CF_prompter(dim) if CF_list is None else CF_list
         code = int(code)
         if_split = code % 2
         code //= 2

@@ -14,12 +14,19 @@ SuiteSparse / OGB collection the reference downloads.
                 matrices whose pick is within 10 % of the best swept configuration.
 
     python -m paramspmm_ae_amd.train_decider sweep --out ParamSpMM-log/decider [--part 0/3]
-    python -m paramspmm_ae_amd.train_decider fit --data paramspmm_ae_amd/models/train_data --out paramspmm_ae_amd/models
+    python -m paramspmm_ae_amd.train_decider fit --space reference    # -> models/rnd_tree_<N>.pkl
+    python -m paramspmm_ae_amd.train_decider fit --space native       # -> models/native/rnd_tree_<N>.pkl
+
+Two sets of forests come out of the same sweep tables.  ``--space reference`` keeps the columns of the reference's own
+class space -- 4 representations x ``dynamic_CF_prompter(dim)`` x blkWarpNum {4, 8}, class code = the reference's
+column index (PCSR.py:781-788, 815-818) -- and writes plain pickles, so that the reference's unchanged decider.py
+(``pickle.load(open(...))`` at decider.py:38, ``decode_tree`` at 63-80) loads and decodes them.  ``--space native``
+trains on every swept column (the reference's list followed by the wave64 configurations); those forests record
+their CF axis in ``psp_cf_list_`` and are what this package's ``SpMMDecider`` reads by default.
 """
 import argparse
 import json
 import os
-import gzip
 import pickle
 import sys
 import time
@@ -246,54 +253,78 @@ def family(name):
     return name
 
 
+def reference_space_columns(dim, cf_axis):
+    """Positions, inside a sweep table whose CF axis is ``cf_axis``, of the reference's columns for ``dim`` in the
+    reference's own order (blkWarpNum-major, then ``dynamic_CF_prompter(dim)``, then the four representations):
+    entry k of the result is the table column of reference class code k."""
+    from .PCSR import dynamic_CF_prompter
+
+    legacy = dynamic_CF_prompter(dim)
+    assert list(cf_axis[:len(legacy)]) == list(legacy), "the table's CF axis must start with the reference's list"
+    return np.array([(w * len(cf_axis) + c) * 4 + r for w in range(2) for c in range(len(legacy)) for r in range(4)])
+
+
 def fit_main(args):
     import pandas as pd
     from sklearn.model_selection import GroupKFold
 
+    from . import sweep as sw
+    from .PCSR import decider_CF_list, dynamic_CF_prompter
+
     dims = [int(d) for d in args.dims.split(",")] if args.dims else DIMS
+    reference_space = args.space == "reference"
+    here = os.path.dirname(os.path.abspath(__file__))
+    out = args.out or os.path.join(here, "models", "" if reference_space else "native")
     info, tps = load_training_data(args.data, dims)
     X = info[FEATURES].to_numpy(dtype=np.float64)
-    os.makedirs(args.out, exist_ok=True)
+    os.makedirs(out, exist_ok=True)
     groups = np.array([family(n) for n in info["mtx_name"]])
-    report = {"matrices": int(len(info)), "families": int(len(set(groups))),
+    report = {"class_space": "reference: 4 representations x dynamic_CF_prompter(dim) x blkWarpNum {4, 8}, the class "
+              "code of decider.py:63-80" if reference_space else
+              "native: 4 representations x decider_CF_list(dim) (the reference's CF list followed by the wave64 "
+              "configurations) x blkWarpNum {4, 8}; the forests carry the list as psp_cf_list_",
+              "matrices": int(len(info)), "families": int(len(set(groups))),
               "validation": "5-fold cross-validation grouped by matrix family (same generator parameters, different "
               "seed / hub degree / ordering): every matrix is predicted by a forest that has seen neither it nor "
               "its siblings", "per_dim": {}}
     folds = list(GroupKFold(5).split(X, groups=groups))
-    from . import sweep as sw
-    from .PCSR import decider_CF_list, dynamic_CF_prompter
 
-    report_path = os.path.join(args.out, "decider_report.json")
+    report_path = os.path.join(out, "decider_report.json")
     if args.dims and os.path.exists(report_path):  # a partial refit keeps the other widths' entries
         with open(report_path) as f:
             report["per_dim"] = {int(k): v for k, v in json.load(f)["per_dim"].items()}
-    cf_lists = {}
     for d in dims:
         # the table's CF axis: the widened list, or the reference's own when the data come from its sweep
         if list(tps[d].columns) == sw.column_names(d):
-            cf_lists[d] = decider_CF_list(d)
+            table_cfs = decider_CF_list(d)
         else:
             assert list(tps[d].columns) == sw.column_names(d, dynamic_CF_prompter(d)), "unknown column set at dim %d" % d
-            cf_lists[d] = dynamic_CF_prompter(d)
-        TP = tps[d].to_numpy(dtype=np.float64)
+            table_cfs = dynamic_CF_prompter(d)
+        TP_all = tps[d].to_numpy(dtype=np.float64)
+        legacy_pos = reference_space_columns(d, table_cfs)
+        if reference_space:
+            TP, cf_list = TP_all[:, legacy_pos], dynamic_CF_prompter(d)
+        else:
+            TP, cf_list = TP_all, table_cfs
         y = TP.argmax(axis=1)  # class code = column index (PCSR.py:815-818)
         # label csv in the reference's schema
         lab = pd.concat([info, pd.DataFrame({"OP_SpMM": y})], axis=1)
-        lab.to_csv(os.path.join(args.data, "dim%d_OP_SpMM.csv" % d), index=False)
-        best = None
-        for near in (1.0, 0.97, 0.95):
-            for n_est, leaves in ((30, 64), (30, 128), (50, 128)):  # the notebook's forest sizes are 30 / 50 / 80
+        lab.to_csv(os.path.join(args.data, "dim%d_OP_SpMM%s.csv" % (d, "" if reference_space else "_native")), index=False)
+        tried = []
+        for n_est, leaves in ((30, 64), (30, 128), (50, 128)):  # the notebook's forest sizes are 30 / 50 / 80
+            for near in (1.0, 0.97, 0.95):
                 pick = np.zeros(len(X), dtype=np.int64)
                 for tr, te in folds:
                     pick[te] = _fit_forest(X[tr], TP[tr], near, n_est, leaves).predict(X[te]).astype(np.int64)
                 norm = TP[np.arange(len(X)), pick] / TP.max(axis=1)  # normalised performance of the pick
                 score = (float(np.mean(norm >= 1 / 1.10)), float(norm.mean()))
-                if best is None or score > best[0]:
-                    best = (score, near, n_est, leaves, pick, norm)
+                tried.append((score, near, n_est, leaves, pick, norm))
+        # the smallest forest (they are tried in order of size) whose validated share within 10 % of the best
+        # configuration is within half a point of the best one's: a pickle grows with trees x leaves x classes
+        top = max(t[0] for t in tried)
+        best = next(t for t in tried if t[0][0] >= top[0] - 0.005 and t[0][1] >= top[1] - 0.002)
         (within10, mean_norm), near, n_est, leaves, pick, norm = best
-        n_legacy = 4 * len(dynamic_CF_prompter(d))
-        legacy_cols = np.array([c % (4 * len(cf_lists[d])) < n_legacy for c in range(TP.shape[1])])
-        best_all, best_legacy = TP.max(axis=1), TP[:, legacy_cols].max(axis=1)
+        best_all, best_legacy = TP_all.max(axis=1), TP_all[:, legacy_pos].max(axis=1)
         gain = best_all / best_legacy  # what the native configurations add over the reference's <CF, blkWarpNum> space
         by_family = {}
         for fam in ("cl_", "rmat_", "sbm_", "stencil_", "grid_", "band_"):
@@ -305,30 +336,55 @@ def fit_main(args):
                         by_family[tag] = float(gain[sel & m].mean())
             elif sel.any():
                 by_family[fam.rstrip("_")] = float(gain[sel].mean())
-        report["per_dim"][d] = {
-            "cf_axis": [sw.cf_label(c) for c in cf_lists[d]],
+        entry = {
+            "cf_axis": [sw.cf_label(c) for c in cf_list],
             "native_gain_over_reference_space": {"mean": float(gain.mean()), "max": float(gain.max()),
                                                  "share_of_matrices_with_gain_over_5pct": float(np.mean(gain > 1.05)),
                                                  "mean_by_family": by_family},
-            "share_of_picks_that_are_native": float(np.mean(~legacy_cols[pick])),
             "near_best_threshold": near, "n_estimators": n_est, "max_leaf_nodes": leaves, "classes": int(TP.shape[1]),
             "validated_matrices": int(len(X)), "accuracy": float(np.mean(pick == y)),
             "mean_normalised_performance": mean_norm, "share_within_10pct_of_best": within10,
             "worst_normalised_performance": float(norm.min()),
         }
+        if reference_space:
+            # the same picks measured against the best of every swept column, native ones included: what a caller of
+            # the reference's decider.py gives up against this package's own decider
+            norm_all = TP[np.arange(len(X)), pick] / best_all
+            entry["against_best_of_all_swept_columns"] = {
+                "mean_normalised_performance": float(norm_all.mean()),
+                "share_within_10pct_of_best": float(np.mean(norm_all >= 1 / 1.10)),
+            }
+        else:
+            legacy_cols = np.zeros(TP.shape[1], dtype=bool)
+            legacy_cols[legacy_pos] = True
+            entry["share_of_picks_that_are_native"] = float(np.mean(~legacy_cols[pick]))
+        report["per_dim"][d] = entry
         # the shipped model is refitted on every matrix
         final = _fit_forest(X, TP, near, n_est, leaves)
         final.n_jobs = 1
-        final.psp_cf_list_ = [int(c) for c in cf_lists[d]]  # the CF axis of the class codes (decider.config_PCSR)
-        # gzip-compressed (the per-node class histograms are mostly zeros); SpMMDecider.load_pickle reads both forms
-        with gzip.GzipFile(os.path.join(args.out, "rnd_tree_%d.pkl" % d), "wb", compresslevel=6, mtime=0) as f:
-            pickle.dump(final, f)
+        path = os.path.join(out, "rnd_tree_%d.pkl" % d)
+        if not reference_space:
+            final.psp_cf_list_ = [int(c) for c in cf_list]  # the CF axis of the class codes (decider.config_PCSR)
+        if reference_space:
+            # plain pickles: decider.py:38 reads them with pickle.load(open(path, "rb"))
+            with open(path, "wb") as f:
+                pickle.dump(final, f, protocol=4)
+        else:
+            # read by this package's SpMMDecider only, which accepts a gzip stream (the per-node class histograms of
+            # 32-72 classes are mostly zeros: a fifth of the plain size)
+            import gzip
+
+            with gzip.GzipFile(path, "wb", compresslevel=6, mtime=0) as f:
+                pickle.dump(final, f, protocol=4)
         print("dim %3d: %2d classes  near %.2f  n_estimators %d  leaves %d  acc %.3f  mean norm perf %.4f  within 10%%: %.3f  worst %.3f" % (
-            d, TP.shape[1], near, n_est, leaves, report["per_dim"][d]["accuracy"], mean_norm, within10, norm.min()), flush=True)
+            d, TP.shape[1], near, n_est, leaves, entry["accuracy"], mean_norm, within10, norm.min()), flush=True)
     allw = [v["share_within_10pct_of_best"] for v in report["per_dim"].values()]
     report["share_within_10pct_mean"] = float(np.mean(allw))
     report["share_within_10pct_min"] = float(np.min(allw))
     report["per_dim"] = {str(k): report["per_dim"][k] for k in sorted(report["per_dim"], key=int)}
+    import sklearn
+
+    report["scikit_learn"] = sklearn.__version__  # a pickled forest loads under the version that wrote it (or newer)
     with open(report_path, "w") as f:
         json.dump(report, f, indent=1)
     print("matrices %d; within 10%% of best: mean %.3f, min over widths %.3f" % (len(info), np.mean(allw), np.min(allw)))
@@ -350,7 +406,10 @@ def main(argv=None):
     f = sub.add_parser("fit")
     here = os.path.dirname(os.path.abspath(__file__))
     f.add_argument("--data", default=os.path.join(here, "models", "train_data"))
-    f.add_argument("--out", default=os.path.join(here, "models"))
+    f.add_argument("--space", choices=("reference", "native"), default="native",
+                   help="class space of the forests: the reference's own (loadable and decodable by its unchanged "
+                        "decider.py) or every swept column")
+    f.add_argument("--out", default="", help="default: models/ for --space reference, models/native/ for --space native")
     f.add_argument("--dims", default="", help="refit these widths only (comma-separated); the report keeps the others")
     ls = sub.add_parser("list")
     args = ap.parse_args(argv)

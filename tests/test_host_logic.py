@@ -225,6 +225,7 @@ def test_cf_search_space_and_decoding_match_reference_integers(oracle):
         assert len(names) == 8 * len(cfs)
         for code in range(8 * len(cfs)):
             got = d.decode_tree(code, dim, CF_list=cfs)
+            assert got == d.decode_tree(code, dim)  # the default CF axis is the reference's (decider.py:69)
             assert got == oracle.decode_tree(code, dim) == sweep.decode_column(dim, code, cfs)
             rep = ["vec1", "vec1_split", "vec2", "vec2_split"][code % 4]
             assert names[code] == "%s_TP_%d%d" % (rep, got[2], got[3])
@@ -235,7 +236,7 @@ def test_cf_search_space_and_decoding_match_reference_integers(oracle):
         names = sweep.column_names(dim)
         assert len(names) == len(set(names)) == 8 * len(wide)
         for code in range(8 * len(wide)):
-            if_split, vec, cf, bw = d.decode_tree(code, dim)
+            if_split, vec, cf, bw = d.decode_tree(code, dim, CF_list=wide)
             assert (if_split, vec, cf, bw) == sweep.decode_column(dim, code)
             assert (if_split, vec) == ((code % 2), (1, 2)[code // 2 % 2]) and cf == wide[code // 4 % len(wide)]
             assert bw == (4, 8)[code // (4 * len(wide))]
@@ -516,13 +517,13 @@ def test_decider_fit_on_a_small_table_and_partial_refit_keeps_the_other_widths(t
     data.mkdir()
     names = ["%s_n%d_d%d_s%d" % (fam, 1000 * (i + 1), 3 + i, s) for fam in ("cl", "sbm", "band") for i in range(5) for s in range(3)]
     feats = pd.DataFrame(rng.random((len(names), len(train_decider.FEATURES))), columns=train_decider.FEATURES)
-    pd.concat([pd.DataFrame({"mtx_name": names}), feats], axis=1).to_csv(data / "mtx_info_part0.csv", index=False)
+    pd.concat([pd.DataFrame({"mtx_name": names}), feats], axis=1).to_csv(data / "mtx_info.csv", index=False)
     for d in (16, 32):
         cols = sweep.column_names(d)
         tp = 100.0 + rng.random((len(names), len(cols)))
         # the first feature decides between two columns, so there is something to learn
         tp[np.arange(len(names)), np.where(feats.iloc[:, 0] > 0.5, 1, len(cols) - 2)] += 50.0
-        pd.DataFrame(tp, columns=cols).to_csv(data / ("dim%d_part0.csv" % d), index=False)
+        pd.DataFrame(tp, columns=cols).to_csv(data / ("dim%d.csv" % d), index=False)
 
     train_decider.main(["fit", "--data", str(data), "--out", str(out), "--dims", "16"])
     report = json.load(open(out / "decider_report.json"))
@@ -532,10 +533,26 @@ def test_decider_fit_on_a_small_table_and_partial_refit_keeps_the_other_widths(t
     assert list(report["per_dim"]) == ["16", "32"]
     assert report["per_dim"]["16"]["classes"] == len(sweep.column_names(16))
 
-    labels = pd.read_csv(data / "dim32_OP_SpMM.csv")
+    labels = pd.read_csv(data / "dim32_OP_SpMM_native.csv")
     assert list(labels.columns) == ["mtx_name"] + train_decider.FEATURES + ["OP_SpMM"]
     want = np.where(feats.iloc[:, 0] > 0.5, 1, len(sweep.column_names(32)) - 2)
     assert (labels["OP_SpMM"].to_numpy() == want).all()
+
+    # the same table fitted on the reference's class space: the widened table's columns of the reference's CF list,
+    # renumbered in the reference's order (blkWarpNum-major); plain pickles without a recorded CF axis
+    ref_out = tmp_path / "models_ref"
+    train_decider.main(["fit", "--data", str(data), "--out", str(ref_out), "--space", "reference", "--dims", "32"])
+    ref_cols = train_decider.reference_space_columns(32, decider_CF_list(32))
+    assert [sweep.column_names(32)[c] for c in ref_cols] == sweep.column_names(32, [1])
+    labels = pd.read_csv(data / "dim32_OP_SpMM.csv")
+    tp32 = pd.read_csv(data / "dim32.csv").to_numpy()
+    assert (labels["OP_SpMM"].to_numpy() == tp32[:, ref_cols].argmax(axis=1)).all() and labels["OP_SpMM"].max() < 8
+    import pickle
+
+    forest = pickle.load(open(ref_out / "rnd_tree_32.pkl", "rb"))
+    assert not hasattr(forest, "psp_cf_list_") and set(forest.classes_) <= set(range(8))
+    rep = json.load(open(ref_out / "decider_report.json"))["per_dim"]["32"]
+    assert rep["classes"] == 8 and "against_best_of_all_swept_columns" in rep
 
     dec = SpMMDecider(str(out) + os.sep)
     dec.gen_model_dict([16, 32])
@@ -595,4 +612,4 @@ def test_decider_candidates_start_with_the_pick_and_are_distinct(tmp_path):
         assert dec.candidates_PCSR(g, dim, 1) == cands[:1]
         codes = set(forest.classes_)
         for c in cands:  # every candidate is a class the forest knows
-            assert any(dec.decode_tree(code, dim) == c for code in codes)
+            assert any(dec.decode_tree(code, dim, CF_list=decider_CF_list(dim)) == c for code in codes)
