@@ -17,7 +17,10 @@ The JSON line also carries
   decider_vs_best  t(decider's pick) / t(best swept configuration) per width, from a short sweep of every
                    <representation, CF, blkWarpNum> after the timed region (PCSR.py:754-788, rnd_tree.ipynb cell 4);
   sddmm            one SDDMM width (K = 64) on the same pattern with its own roofline;
-  gcn_epoch_ms     20 GCN training epochs (5 layers, hidden 16, 16 classes) on the 1M-node block model (GNN.py:126-151);
+  other_graphs     the other graphs of the benchmark set in the decider's configuration: 5-point stencil 2048^2 at
+                   N = 64 / 128, block model (community order and random order) at N = 128, Chung-Lu 2.45M at N = 128;
+  gcn_epoch_ms     GCN / GIN training epochs (5 layers, hidden 16 / 32 / 128, 16 classes) on the 1M-node block model,
+                   1 warm-up + 200 timed epochs as in GNN.py:126-151;
   cpu_baseline     torch.sparse.mm on the host cores (the product the reference verifies against, verification.py:18-46)
                    on a bounded sample of the widths; cpu_scalar_port is the oracle's one-thread C restatement, which also
                    checks the GPU result at those widths.
@@ -73,6 +76,67 @@ def measured_traffic(graph, rows_of):
             return None
         total += table[key]
     return int(total / len(rows_of))
+
+
+def measured_sddmm_traffic(graph, K, fmt, bw):
+    """HBM bytes of one SDDMM launch from the committed counter summary (profiles/psp_sddmm_kernel_<graph>_trace_and_pmc.md,
+    table "fastest configuration per width": | K | layout | wavefronts | ... | HBM bytes | ...); None without a
+    matching line."""
+    path = os.path.join(ROOT, "profiles", "psp_sddmm_kernel_%s_trace_and_pmc.md" % graph)
+    if not os.path.exists(path):
+        return None
+    header = None
+    for line in open(path):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if cells and cells[0] == "K" and "HBM bytes" in cells:
+            header = cells
+        elif header and len(cells) == len(header) and cells[0].isdigit():
+            row = dict(zip(header, cells))
+            if int(row["K"]) == K and row["layout"] == fmt and int(row["wavefronts"]) == bw:
+                return int(row["HBM bytes"])
+    return None
+
+
+def other_graph_leg(name, dims, decider, reps=10):
+    """One more graph of the benchmark set at a few widths, in the decider's configuration: per width the mean
+    launch duration (HIP events on the launching stream), algorithmic bytes and their fraction of the HBM roofline,
+    and the measured traffic of the committed counter summary for that graph when it has the configuration."""
+    import torch
+    from paramspmm_ae_amd import _capi, sweep, synth
+    from paramspmm_ae_amd.graph_input import graph_input
+
+    t0 = time.time()
+    rowPtr, colIdx, val, n = synth.config_graph(name)
+    graph = graph_input(mtx_name=name, path="")
+    graph.verbose = False
+    graph.load_from_csr(rowPtr, colIdx, val)
+    nnz = graph.mtx_edges
+    ops = sweep.operators_of(graph)
+    fmt_names = ["csr", "csr_split", "bcsr", "bcsr_split"]
+    F = {"n": n, "nnz": nnz, "S": graph.csr_data.target_row.numel(), "Mb": graph.bcsr_data.num_nodes,
+         "nblk": graph.bcsr_data.colIdx.numel(), "Sb": graph.bcsr_data.target_row.numel()}
+    rows = (n + 1) // 2 * 2
+    gen = torch.Generator(device="cuda").manual_seed(99)
+    res = []
+    for d in dims:
+        X = torch.randn(rows, d, device="cuda", generator=gen)
+        if rows != n:
+            X[n:].zero_()
+        if_split, vec, cf, bw = (int(v) for v in decider.config_PCSR(graph, d))
+        op = ops[(1 if if_split else 0) + (2 if vec == 2 else 0)]
+        fmt = fmt_names[(1 if if_split else 0) + (2 if vec == 2 else 0)]
+        ms = op.time_ms(X, CF=cf, blkWarpNum=bw, warmup=3, iters=reps)
+        b_alg = algorithmic_bytes(fmt, F, n, d)
+        row = {"dim": d, "format": fmt, "CF": cf, "config": sweep.cf_label(cf), "blkWarpNum": bw, "ms": round(float(ms), 5),
+               "gflops": round(2.0 * nnz * d / ms / 1e6, 1), "alg_bytes": int(b_alg),
+               "frac": round(b_alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
+        row["traffic"] = measured_traffic(name, [row])
+        res.append(row)
+        del X
+    out = {"nodes": n, "nnz": int(nnz), "setup_s": round(time.time() - t0, 1), "widths": res}
+    del ops, graph
+    torch.cuda.empty_cache()
+    return out
 
 
 def gather_probe_ms(colIdx_dev, nnz, X, lanes, reps=5):
@@ -759,7 +823,8 @@ def main():
         out["sddmm"] = {"K": K, "format": sfmt, "blkWarpNum": sbw, "ms": round(sms, 5), "gflops": round(2.0 * nnz * K / sms / 1e6, 1),
                         "all_ms": {"%s/%d" % k: round(v, 5) for k, v in sd_ms.items()},
                         "roofline": {"bound": "hbm", "achieved": round(salg / sms / 1e6, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                                     "frac": round(salg / sms / 1e6 / HBM_PEAK_GBS, 4), "traffic": None,
+                                     "frac": round(salg / sms / 1e6 / HBM_PEAK_GBS, 4),
+                                     "traffic": measured_sddmm_traffic(args.graph, K, sfmt, sbw),
                                      "kernel": "psp_sddmm_kernel, K = 64, %s, %d wavefronts per workgroup" % (sfmt, sbw),
                                      "alg_bytes_per_launch": int(salg), "ms_per_launch": round(sms, 5)}}
         del A, Bm
@@ -852,19 +917,29 @@ def main():
                                   "max_abs_gpu_minus_oracle": err}
 
     if not args.no_extras and args.graph == "C2":
-        # ---- GCN training epochs on the 1M-node block model (the metric's second half) ------------------------------
         for d in list(Xs):
             del Xs[d], Ys[d]
+        del ops, graph
         torch.cuda.empty_cache()
+        # ---- the other graphs of the benchmark set, decider-picked configurations -----------------------------------
+        if decider is not None:
+            out["other_graphs"] = {
+                "C3s 5-point stencil 2048^2": other_graph_leg("C3s", [64, 128], decider),
+                "C5 block model 1M nodes, community order": other_graph_leg("C5", [128], decider),
+                "C5p block model 1M nodes, random order": other_graph_leg("C5p", [128], decider),
+                "C3 Chung-Lu 2.45M nodes": other_graph_leg("C3", [128], decider, reps=5),
+            }
+        # ---- GCN training epochs on the 1M-node block model (the metric's second half) ------------------------------
         from paramspmm_ae_amd import GNN
 
         epochs = {}
+        n_epochs = 200  # the reference's protocol: 1 warm-up epoch + 200 timed ones (GNN.py:126-151)
         with contextlib.redirect_stdout(sys.stderr):
             for net in ("GCN", "GIN"):
                 res = GNN.main(["--net", net, "--synthetic", "C5", "--hidden_list", "16", "32", "128", "--num_classes", "16",
-                                "--num_features", "32", "--num_epoches", "20"])
+                                "--num_features", "32", "--num_epoches", str(n_epochs)])
                 epochs[net] = {str(h): round(float(ms), 3) for (_, h), ms in res.items()}
-        out["gcn_epoch_ms"] = {"value": epochs["GCN"]["16"], "unit": "ms per epoch", "epochs": 20,
+        out["gcn_epoch_ms"] = {"value": epochs["GCN"]["16"], "unit": "ms per epoch", "epochs": n_epochs,
                                "by_hidden": epochs["GCN"], "gin_by_hidden": epochs["GIN"],
                                "config": "5 layers, hidden 16 / 32 / 128 (value: GCN, hidden 16), 16 classes, 32 features, "
                                          "fwd+bwd+Adam, SBM 1M nodes (community order), decider-picked operators"}

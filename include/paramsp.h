@@ -31,6 +31,15 @@ enum psp_status {
 };
 
 const char *psp_last_error(void);
+
+/* Version of the ABI this header describes; psp_version() returns the one the loaded library was built from.  A
+ * caller compiled against this header must find psp_version() >= PSP_ABI_VERSION before it calls anything else:
+ * buffers that the library fills have grown between versions under unchanged symbol names --
+ *   200: psp_spmm_plan gained log_segs_per_wave, even_split, xcd_stripe_rows (10 ints; 7 before);
+ *        psp_nll_loss_mean_f32 writes 3 + 3*1024 floats of `stats` (2 before);
+ *   300: option "whole_rows".
+ * The extension modules and the ctypes loader of this package check it when they are imported. */
+#define PSP_ABI_VERSION 300
 int psp_version(void);
 
 /* How a (N, CF, blkWarpNum) request of the Python layer maps onto the wave64 kernels.
@@ -79,8 +88,14 @@ int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan);
  *   "xcd_stripe_rows"  rows (segments) dealt to one XCD at a time by the SpMM kernels (default 8192),
  *   "align_pct"        lane groups take whole segments when that costs at most this many percent more steps than
  *                      the even division of a wavefront's entries (default 50),
- *   "split_clear_min"  row-split outputs of at least this many floats are cleared selectively (default 4 Mi).
- * The environment (PSP_XCD_STRIPE_ROWS, PSP_ALIGN_PCT, PSP_SPLIT_CLEAR_MIN) sets the initial values, once.
+ *   "split_clear_min"  row-split outputs of at least this many floats are cleared selectively (default 4 Mi),
+ *   "whole_rows"       1: a lane group is always handed whole rows (segments), however uneven that is.  Every element
+ *                      of a plain CSR / BCSR product is then one FMA chain over the row's stored entries in storage
+ *                      order, which is the summation order of the reference's one-warp-per-row kernels
+ *                      (SpMM/SpMM_kernel.cu:1157-1212, 1362-1440): results repeat the sequential chain bit for bit.
+ *                      Default 0: rows may be cut between lane groups and summed piecewise (faster on skewed rows).
+ * The environment (PSP_XCD_STRIPE_ROWS, PSP_ALIGN_PCT, PSP_SPLIT_CLEAR_MIN, PSP_WHOLE_ROWS) sets the initial values,
+ * once.
  * psp_get_option returns the value, or a negative psp_status for an unknown name.  Not synchronised with running
  * launches: set options before the calls they should affect. */
 int psp_set_option(const char *name, long long value);
@@ -301,7 +316,10 @@ int psp_segment_softmax_ws_f32(const int *rowPtr, const float *in, float *out, i
  * allocates and frees nothing.  M may not exceed PSP_SEGMENT_SOFTMAX_STATIC_MAX_ROWS (PSP_ERR_ARG beyond it: use the
  * _ws_ form).  The stream's device must be the current device.  All calls on one GPU share the array: two calls
  * that overlap on one GPU (different streams, or graphs replayed concurrently) race on it; calls on one stream, or
- * otherwise ordered, do not. */
+ * otherwise ordered, do not.  The first call on a device looks the array's address up (hipGetDevice, a lock,
+ * hipGetSymbolAddress: host work, no allocation); every later call on that device is kernel launches only.  Make one
+ * call per device outside any stream capture before capturing one -- an empty call (M = 0) does the lookup and
+ * launches nothing. */
 #define PSP_SEGMENT_SOFTMAX_STATIC_MAX_ROWS (1 << 21)
 int psp_segment_softmax_static_f32(const int *rowPtr, const float *in, float *out, int M, int nnz,
                                    psp_stream_t stream);

@@ -25,7 +25,7 @@ int psp_fail(int code, const char *fmt, ...)
 }
 
 // Library-wide options: defaults, overridden once by the environment (PSP_XCD_STRIPE_ROWS, PSP_ALIGN_PCT,
-// PSP_SPLIT_CLEAR_MIN) when the library is first used, and afterwards only through psp_set_option.
+// PSP_SPLIT_CLEAR_MIN, PSP_WHOLE_ROWS) when the library is first used, and afterwards only through psp_set_option.
 psp_options &psp_opts(void)
 {
     static psp_options o = [] {
@@ -33,6 +33,7 @@ psp_options &psp_opts(void)
         d.stripe_rows = 8192;
         d.align_pct = 50;
         d.split_clear_min = (long long)4 << 20;
+        d.whole_rows = 0;
         if (const char *e = getenv("PSP_XCD_STRIPE_ROWS")) {
             if (atoi(e) > 0) d.stripe_rows = atoi(e);
         }
@@ -42,6 +43,7 @@ psp_options &psp_opts(void)
         if (const char *e = getenv("PSP_SPLIT_CLEAR_MIN")) {
             if (atoll(e) >= 0) d.split_clear_min = atoll(e);
         }
+        if (const char *e = getenv("PSP_WHOLE_ROWS")) d.whole_rows = atoi(e) != 0;
         return d;
     }();
     return o;
@@ -61,6 +63,9 @@ PSP_EXPORT int psp_set_option(const char *name, long long value)
     } else if (!strcmp(name, "split_clear_min")) {
         PSP_REQUIRE(value >= 0, "set_option: split_clear_min must not be negative");
         o.split_clear_min = value;
+    } else if (!strcmp(name, "whole_rows")) {
+        PSP_REQUIRE(value == 0 || value == 1, "set_option: whole_rows is 0 or 1");
+        o.whole_rows = (int)value;
     } else {
         return psp_fail(PSP_ERR_ARG, "set_option: unknown option '%s'", name);
     }
@@ -74,11 +79,12 @@ PSP_EXPORT long long psp_get_option(const char *name)
     if (!strcmp(name, "xcd_stripe_rows")) return o.stripe_rows;
     if (!strcmp(name, "align_pct")) return o.align_pct;
     if (!strcmp(name, "split_clear_min")) return o.split_clear_min;
+    if (!strcmp(name, "whole_rows")) return o.whole_rows;
     return psp_fail(PSP_ERR_ARG, "get_option: unknown option '%s'", name);
 }
 
 PSP_EXPORT const char *psp_last_error(void) { return g_err; }
-PSP_EXPORT int psp_version(void) { return 200; }
+PSP_EXPORT int psp_version(void) { return 300; }
 
 // ------------------------------------------------------------------------------------------------
 // (N, CF, blkWarpNum) -> wave64 launch plan
@@ -567,11 +573,13 @@ PSP_EXPORT int psp_segment_softmax_static_f32(const int *rowPtr, const float *in
     PSP_REQUIRE(M <= PSP_STATIC_SOFTMAX_MAX_ROWS,
                 "segment_softmax_static: %d rows exceed the built-in scratch of %d rows; use psp_segment_softmax_ws_f32", M,
                 PSP_STATIC_SOFTMAX_MAX_ROWS);
-    if (M == 0 || nnz == 0) return PSP_OK;
-    PSP_REQUIRE(rowPtr && in && out, "segment_softmax_static: null pointer");
+    // The address lookup of the first call on a device is host work that does not belong under stream capture: an
+    // empty call (M = 0) performs it and launches nothing, which is how a caller prepares a device before capturing.
     float *scratch = nullptr;
     const int rc = psp_softmax_scratch_ptr(&scratch);
     if (rc != PSP_OK) return rc;
+    if (M == 0 || nnz == 0) return PSP_OK;
+    PSP_REQUIRE(rowPtr && in && out, "segment_softmax_static: null pointer");
     // Nothing has to start at zero: the first kernel resets the pair of every long row of this call, and pairs of
     // other rows (left by earlier calls) are never read.
     return psp_segment_softmax_ws_f32(rowPtr, in, out, M, nnz, scratch, stream);

@@ -17,8 +17,10 @@
 //     the two row blocks a wavefront works on);
 //   * result lane (r, q), tile j, element i is Y[row r][16j + 4q + i]: one 16-byte store per tile, the four q-lanes
 //     of a row writing 64 contiguous bytes.
-// W (at most 64 KB) is staged into LDS once per workgroup, transposed on the way in for the X * W^T form; the grid is
-// sized to the GPU and every wavefront walks blocks of 32 rows with the next block's loads in flight.
+// W (K1 rows of K2 + 4 floats: 66 KB at 128 x 128) is staged into LDS once per workgroup, transposed on the way in for
+// the X * W^T form.  That is more than the 64 KB a workgroup gets on earlier CDNA parts: the kernel is built for
+// gfx950 only, whose CUs have 160 KB, and two workgroups per CU (the launch shape) need 132 KB of it.  The grid is sized
+// to the GPU and every wavefront walks blocks of 32 rows with the next block's loads in flight.
 #include "psp_common.h"
 
 typedef float psp_f32x4 __attribute__((ext_vector_type(4)));
@@ -35,6 +37,8 @@ psp_xw_wide_kernel(const float *__restrict__ X, const float *__restrict__ W, flo
     constexpr int KT = K1 / 16;  // float4 loads per lane and row block
     constexpr int S = K2 + 4;    // LDS row stride: the four k-rows a step reads fall into different bank halves
     static_assert(T % 4 == 0 && K1 % 16 == 0, "widths: K2 a multiple of 64, K1 a multiple of 16");  // T % 4: 16-byte LDS reads
+    // two workgroups share a CU's 160 KB of LDS
+    static_assert(sizeof(float) * K1 * S <= 80 * 1024, "W does not fit half of a gfx950 CU's LDS");
     __shared__ float Ws[K1 * S];
 
     for (int idx = threadIdx.x; idx < K1 * K2; idx += blockDim.x) {
@@ -150,7 +154,20 @@ static psp_xw_wide_kernel_t xw_wide_lookup(int K1, int K2, bool relu_x, bool mas
     return nullptr;
 }
 
-bool psp_xw_wide_supported(int K1, int K2) { return xw_wide_lookup(K1, K2, false, false) != nullptr; }
+bool psp_xw_wide_supported(int K1, int K2)
+{
+    if (xw_wide_lookup(K1, K2, false, false) == nullptr) return false;
+    // the staged W must fit what the device grants one workgroup (160 KB per CU on gfx950)
+    static int lds_of[64];  // per device, looked up once (0 = not yet; races write the same value)
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    int lds = lds_of[dev];
+    if (lds == 0) {
+        if (hipDeviceGetAttribute(&lds, hipDeviceAttributeMaxSharedMemoryPerBlock, dev) != hipSuccess) return false;
+        lds_of[dev] = lds;
+    }
+    return (size_t)lds >= sizeof(float) * (size_t)K1 * (size_t)(K2 + 4);
+}
 
 // called by psp_gemm_xw_act_f32 for the widths the one-lane-per-row kernel does not cover; arguments are checked there
 int psp_xw_wide_launch(const float *X, const float *W, float *Y, long long n, int K1, int K2, int transW, int relu_x,

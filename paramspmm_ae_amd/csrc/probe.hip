@@ -26,9 +26,14 @@ psp_probe_gather_kernel(const int *__restrict__ colIdx, long long nnz, const flo
     long long a = e0 + (long long)grp * q, b = a + q;
     if (a > e1) a = e1;
     if (b > e1) b = e1;
-    const int col0 = (blockIdx.y << logL) * 4 + sub * 4;  // this lane's first column
+    // A lane whose columns lie past N stays active -- ds_bpermute reads 0 from an inactive lane, which would turn
+    // the entries those lanes fetched into gathers of X row 0 -- and loads the last valid vector instead, as the SpMM
+    // kernel does; what it loads is not added.
+    const int col_own = (blockIdx.y << logL) * 4 + sub * 4;  // this lane's first column
+    const bool live = col_own < N;
+    const int col0 = live ? col_own : N - 4;
     psp_f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    if (col0 < N) {
+    {
         // lane `sub` takes the U consecutive entries base + sub*U .. (one 4U-byte load, whole lines per group), as
         // the SpMM kernel does
         for (long long base = a; base < b; base += L * U) {
@@ -61,7 +66,7 @@ psp_probe_gather_kernel(const int *__restrict__ colIdx, long long nnz, const flo
                 }
 #pragma unroll
                 for (int u = 0; u < U; u++)
-                    if (base + (long long)j * U + u < b) acc += x[u];
+                    if (live && base + (long long)j * U + u < b) acc += x[u];
             }
         }
     }

@@ -57,6 +57,7 @@ struct psp_options {
     int stripe_rows;            // rows (or segments) one XCD stripe should span
     int align_pct;              // whole segments per lane group when that costs at most this many percent more steps
     long long split_clear_min;  // row-split outputs of at least this many floats are cleared selectively
+    int whole_rows;             // SpMM: a lane group always takes whole segments (reference summation order)
 };
 psp_options &psp_opts(void);
 int psp_stripe_rows(void);

@@ -37,6 +37,11 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     if (logW < logR - 1) logW = logR - 1;
     if (logW > 6) logW = 6;
     const psp_options &opt = psp_opts();
+    // whole_rows: every lane group is handed whole segments whatever their lengths, so each element of a plain row
+    // is one FMA chain over the row's entries in storage order -- the summation order of the reference's
+    // one-warp-per-row kernels (SpMM_kernel.cu:1157-1212), bit for bit -- at the price of the balance between the
+    // lane groups.  That needs at least one segment per lane group.
+    if (opt.whole_rows && logW < logR) logW = logR;
 
     // rows the kernel does not store to must read as zero
     if (SPLIT) {
@@ -67,7 +72,7 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
         return psp_fail(PSP_ERR_ARG, "spmm%s: no kernel for coarsen %d vec %d unroll %d%s", softmax ? " softmax" : "", plan.coarsen,
                         plan.vec, plan.unroll, softmax ? " (needs N % 4 == 0 and CF <= 4)" : "");
 
-    const int align_pct = plan.even_split ? 0 : opt.align_pct;
+    const int align_pct = opt.whole_rows ? (1 << 30) : (plan.even_split ? 0 : opt.align_pct);
     const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block),
                                       (plan.xcd_stripe_rows ? plan.xcd_stripe_rows : opt.stripe_rows) / segs_per_block);
     dim3 grid(g.launch, plan.col_tiles, 1), block(plan.waves_per_block * PSP_WAVE, 1, 1);

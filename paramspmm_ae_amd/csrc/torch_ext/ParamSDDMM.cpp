@@ -327,6 +327,7 @@ static int cusparse_sddmm_profile(Tensor A, Tensor B, Tensor rowPtr, Tensor colI
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
+    pspglue::check_abi();
     m.def("csr_sddmm", &csr_sddmm, "CSR SDDMM (HIP, gfx950)");
     m.def("csr_split_sddmm", &csr_split_sddmm, "row-split CSR SDDMM (HIP, gfx950)");
     m.def("bcsr_sddmm", &bcsr_sddmm, "2x1 BCSR SDDMM (HIP, gfx950)");

@@ -262,6 +262,7 @@ PSP_CONV_SPLIT(bcsr_split_spmm, 3)
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
+    pspglue::check_abi();
     m.def("split_csr", &pspglue::split_csr, "row split on the host");
     m.def("split_csr_par", &pspglue::split_csr_par, "row split on the host with a precomputed segment prefix");
     // addition of this build: H^T * G for tall-skinny operands (memory-speed kernel for widths 16..64, else torch::mm)

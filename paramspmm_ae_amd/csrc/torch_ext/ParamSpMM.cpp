@@ -295,6 +295,7 @@ static py::dict spmm_plan(int N, int CF, int blkWarpNum)
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
+    pspglue::check_abi();
     m.def("split_csr", &pspglue::split_csr, "row split on the host (CPU int32 rowPtr, granularity)");
     m.def("split_csr_par", &pspglue::split_csr_par, "row split on the host with a precomputed segment prefix");
     m.def("csr_spmm", &csr_spmm, "CSR SpMM (HIP, gfx950)");

@@ -12,6 +12,14 @@
 
 namespace pspglue {
 
+// The modules are compiled against include/paramsp.h; a libparamsp_hip.so built from an older header fills smaller
+// structs and buffers under the same symbol names.  Called first thing when a module is imported.
+inline void check_abi()
+{
+    TORCH_CHECK(psp_version() >= PSP_ABI_VERSION, "libparamsp_hip.so is version ", psp_version(),
+                ", this module was built against ", PSP_ABI_VERSION, ": rebuild the library");
+}
+
 // PyTorch-ROCm presents HIP devices under the "cuda" device type; these are its guard / stream types for that.
 using DeviceGuard = c10::hip::HIPGuardMasqueradingAsCUDA;
 
