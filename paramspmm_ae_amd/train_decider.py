@@ -319,10 +319,7 @@ def fit_main(args):
                 norm = TP[np.arange(len(X)), pick] / TP.max(axis=1)  # normalised performance of the pick
                 score = (float(np.mean(norm >= 1 / 1.10)), float(norm.mean()))
                 tried.append((score, near, n_est, leaves, pick, norm))
-        # the smallest forest (they are tried in order of size) whose validated share within 10 % of the best
-        # configuration is within half a point of the best one's: a pickle grows with trees x leaves x classes
-        top = max(t[0] for t in tried)
-        best = next(t for t in tried if t[0][0] >= top[0] - 0.005 and t[0][1] >= top[1] - 0.002)
+        best = max(tried, key=lambda t: t[0])  # the first of equals: the smaller forest
         (within10, mean_norm), near, n_est, leaves, pick, norm = best
         best_all, best_legacy = TP_all.max(axis=1), TP_all[:, legacy_pos].max(axis=1)
         gain = best_all / best_legacy  # what the native configurations add over the reference's <CF, blkWarpNum> space
