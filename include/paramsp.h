@@ -37,7 +37,7 @@ const char *psp_last_error(void);
  * buffers that the library fills have grown between versions under unchanged symbol names --
  *   200: psp_spmm_plan gained log_segs_per_wave, even_split, xcd_stripe_rows (10 ints; 7 before);
  *        psp_nll_loss_mean_f32 writes 3 + 3*1024 floats of `stats` (2 before);
- *   300: option "whole_rows".
+ *   300: option "whole_rows"; the windowed-CSR entry points.
  * The extension modules and the ctypes loader of this package check it when they are imported. */
 #define PSP_ABI_VERSION 300
 int psp_version(void);
@@ -296,6 +296,32 @@ int psp_sddmm_vec_f32(const int *rowPtr_b, const int *colIdx_b, const float *val
 int psp_sddmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b, const float *val_b, const int *target_row,
                             const float *A, const float *B, float *out, int Sb, int K, int vec_size,
                             int blkWarpNum, psp_stream_t stream);
+
+/* ---------------------------------------------------------------------------------------------
+ * Windowed CSR: a fifth representation, for matrices whose entries cluster around the diagonal (community-ordered
+ * graphs, meshes, banded matrices).  No counterpart in the reference.  Rows are cut into blocks of PSP_WINDOW_BLOCK;
+ * an entry is local when its column lies in [block start - PSP_WINDOW_HALO, block end + PSP_WINDOW_HALO).  The format
+ * keeps every row's entries, local ones first (each part in its original order), columns absolute:
+ *   rowPtr_w[2M + 2]: 2i = start of row i, 2i + 1 = start of its remote part; 2M and 2M + 1 = nnz;
+ *   colIdx_w[nnz], val_w[nnz]: the permuted entries.
+ * psp_window_build fills them on the host, psp_window_build_dev on the device (same result).
+ * psp_spmm_window_f32: Y[0..M) = A X (square A with nnz = rowPtr_w[2M] stored entries, X with at least M rows),
+ * Y[M..rows_out) = 0.  The X rows of a workgroup's window are staged in LDS and the local entries read them there;
+ * only remote entries gather from global memory.  N must be a multiple of 4.  variant: 0 automatic, 1 / 2 / 3 = column tiles of 16 / 32 / 64 floats
+ * (psp_spmm_window_plan reports tile width, rows per workgroup and LDS bytes, and returns the variant chosen).
+ * relu_x != 0: the rows of X enter as max(x, 0); mask (may be null): an output element is kept only where
+ * mask > 0, else it is an exact zero (mask has Y's shape).  Results lie within the fp32 tolerance of the CSR product
+ * (local entries are summed before remote ones), they are not bit-identical to it.
+ * ------------------------------------------------------------------------------------------- */
+#define PSP_WINDOW_BLOCK 64
+#define PSP_WINDOW_HALO 64
+int psp_window_build(const int *rowPtr, const int *colIdx, const float *val, int M, int *rowPtr_w, int *colIdx_w,
+                     float *val_w);
+int psp_window_build_dev(const int *rowPtr, const int *colIdx, const float *val, int M, int *rowPtr_w, int *colIdx_w,
+                         float *val_w, psp_stream_t stream);
+int psp_spmm_window_plan(int N, int variant, int *tile_cols, int *rows_per_block, int *lds_bytes);
+int psp_spmm_window_f32(const int *rowPtr_w, const int *colIdx_w, const float *val_w, const float *X, float *Y, int M,
+                        int nnz, int N, int rows_out, int variant, int relu_x, const float *mask, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: softmax over the stored entries of every CSR row (out[p] = exp(e[p]-max_r) / sum_r).

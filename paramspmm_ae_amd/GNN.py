@@ -218,16 +218,37 @@ def build_model(net, graph, operators, hidden, num_features, num_classes, num_la
     return GIN(num_classes, num_features, graph.x, operators, hidden).to(device)
 
 
-def configure_operators(decider, graph, dims, override=None, try_candidates=0):
+WINDOW_MIN_LOCAL_SHARE = 0.5  # windowed layout: tried when at least this share of the entries is local
+
+
+def _try_window(graph, dim, op):
+    """The windowed layout against ``op`` on this matrix (an addition of this build): when at least half of the
+    entries have their column within the row's window, both are timed (a few launches each, after a cache fill, as
+    inside an epoch) and the faster one is returned.  The class space of the forests has no such representation, so
+    the choice is made by this measurement instead of by the decider."""
+    if dim % 4 or graph.csr_data.val.dim() != 1:
+        return op
+    cand = pcsr_spmm(graph=graph, vec_size=1, if_split=False, CF=0, window=True)
+    if cand.window_local_share < WINDOW_MIN_LOCAL_SHARE:
+        return op
+    X = torch.randn((graph.mtx_nodes + 1) // 2 * 2, dim, device="cuda")
+    ms_op = op.time_ms(X, warmup=2, iters=5, flush_bytes=256 << 20)
+    ms_w = cand.time_ms(X, warmup=2, iters=5, flush_bytes=256 << 20)
+    return cand if ms_w < ms_op else op
+
+
+def configure_operators(decider, graph, dims, override=None, try_candidates=0, try_window=True):
     """One pcsr_spmm per layer width, configured by the decider (GNN.py:200-209) or by ``override`` =
     (if_split, vec_size, CF, blkWarpNum).  ``try_candidates`` = k > 1 (an addition of this build): the k configurations
     the forest rates highest are timed on this matrix (a few launches each, after a cache fill, as inside an epoch) and
-    the fastest is kept."""
+    the fastest is kept.  ``try_window``: see _try_window (not with ``override``)."""
     ops = {}
     for dim in dims:
         if override is not None or try_candidates <= 1:
             if_split, vec_size, CF, blkWarpNum = override if override is not None else decider.config_PCSR(graph, dim)
             ops[dim] = pcsr_spmm(graph=graph, vec_size=vec_size, if_split=if_split, CF=CF, blkWarpNum=blkWarpNum)
+            if override is None and try_window:
+                ops[dim] = _try_window(graph, dim, ops[dim])
             continue
         X = torch.randn((graph.mtx_nodes + 1) // 2 * 2, dim, device="cuda")  # an even row count serves the 2x1 block formats too
         best = None
@@ -236,7 +257,7 @@ def configure_operators(decider, graph, dims, override=None, try_candidates=0):
             ms = op.time_ms(X, warmup=2, iters=5, flush_bytes=256 << 20)
             if best is None or ms < best[0]:
                 best = (ms, op)
-        ops[dim] = best[1]
+        ops[dim] = _try_window(graph, dim, best[1]) if try_window else best[1]
     return ops
 
 
@@ -264,6 +285,9 @@ def main(argv=None):
                    help="apply the ReLU between the layers as passes of their own, as the reference's driver does")
     p.add_argument("--try_candidates", type=int, default=0, metavar="K",
                    help="time the K configurations the decider rates highest on the matrix and keep the fastest")
+    p.add_argument("--no_window", action="store_true",
+                   help="never replace the decider's operator by the windowed layout (tried when at least half of the "
+                        "entries lie near the diagonal)")
     p.add_argument("--config", nargs=4, type=int, default=None, metavar=("IF_SPLIT", "VEC", "CF", "BW"),
                    help="skip the decider and use this configuration for every layer width")
     args = p.parse_args(argv)
@@ -295,8 +319,10 @@ def main(argv=None):
                 dims.append(args.num_features)  # the first layer runs its sparse product at the features' width
             if args.net == "GIN" and args.num_features not in dims and (decider is None or args.num_features in decider.model_dict):
                 dims.append(args.num_features)  # GIN aggregates its input: the first layer's product has the features' width
+            # (the attention network orders its per-entry vectors by the graph's own colIdx: it keeps the PCSR formats)
             ops = configure_operators(decider, graph, dims, None if args.config is None else tuple(args.config),
-                                      try_candidates=args.try_candidates)
+                                      try_candidates=args.try_candidates,
+                                      try_window=not args.no_window and args.net != "AGNN")
             print("SpMM-decider config time: {:.3f} (ms)".format((time.perf_counter() - t1) * 1e3))
             model = build_model(args.net, graph, ops, hidden, args.num_features, args.num_classes, args.num_layers)
             if args.no_fuse_relu and hasattr(model, "fuse_relu"):

@@ -140,11 +140,17 @@ _SDDMM = {(False, False): "csr_sddmm", (True, False): "csr_split_sddmm", (False,
 
 class pcsr_spmm(object):
     def __init__(self, graph, vec_size, if_split, mtx_nodes=None, mtx_edges=None, rowPtr=None, colIdx=None,
-                 val=None, target_row=None, CF=1, blkWarpNum=4, device="cuda"):
+                 val=None, target_row=None, CF=1, blkWarpNum=4, device="cuda", window=False):
+        """``window`` (an addition of this build): the CSR matrix in the library's windowed layout, whose SpMM reads
+        the X rows near the diagonal from LDS (vec_size 1, not split, a loaded graph; CF then names the kernel
+        variant, 0 = automatic).  The SDDMM of such an operator runs on the same permuted CSR arrays."""
         if vec_size not in (1, 2, 3):
             raise ValueError("this build has vec_size 1 (CSR), 2 (2x1 BCSR) and 3 (3x1 blocks)")
         if_split = bool(if_split)
         self.mask = None
+        self.window = bool(window)
+        if self.window and (graph is None or vec_size != 1 or if_split):
+            raise ValueError("window=True needs a loaded graph, vec_size 1 and if_split False")
         if graph is None:
             if mtx_edges is None or mtx_nodes is None or rowPtr is None or colIdx is None or val is None:
                 raise ValueError("when graph is None, mtx_nodes, mtx_edges, rowPtr, colIdx, val should be given")
@@ -181,6 +187,12 @@ class pcsr_spmm(object):
         self.CF = CF
         self.blkWarpNum = blkWarpNum
         self.result = None
+        self.window_local_share = None
+        if self.window:
+            # rowPtr_w has 2 M + 2 entries (row start, start of the row's remote part); colIdx / val are the row-wise
+            # permuted entries, so rowPtr_w[0::2] with them is again a CSR matrix (what the SDDMM walks)
+            self.rowPtr_w, self.colIdx, self.val, self.window_local_share = graph.csr_data.window_format(device)
+            self.CF = CF if 0 <= CF <= 3 else 0
         # Plain layouts of a graph with hub rows: the SDDMM divides the stored entries, not the rows, between its
         # wavefronts (every entry's result is independent).  "Hub rows" = a longest row of more than 64 times the
         # mean; arrays without statistics keep the row-wise walk.
@@ -200,6 +212,17 @@ class pcsr_spmm(object):
                 self.sddmm_balanced = float(longest) > 64.0 * float(mean)
 
     # ---- plumbing ---------------------------------------------------------------------------
+    @property
+    def fmt_code(self):
+        """Format code of the extension modules' generic entry points: 0 csr, 1 csr_split, 2 bcsr, 3 bcsr_split,
+        4 windowed csr."""
+        return 4 if self.window else (1 if self.if_split else 0) + (2 if self.vec_size != 1 else 0)
+
+    @property
+    def spmm_rowPtr(self):
+        """The row pointer array the SpMM entry points of this operator's format take."""
+        return self.rowPtr_w if self.window else self.rowPtr
+
     def _key(self):
         return (self.if_split, self.vec_size != 1)
 
@@ -216,6 +239,9 @@ class pcsr_spmm(object):
         return args
 
     def _spmm(self, X, val=None, CF=None, blkWarpNum=None):
+        if self.window:
+            return SpMM.window_spmm(X, self.rowPtr_w, self.colIdx, self.val if val is None else val,
+                                    self.CF if CF is None else CF)
         fn = getattr(SpMM, self._spmm_name())
         return fn(X, *self._sparse_args(val), self.CF if CF is None else CF,
                   (self.blkWarpNum if blkWarpNum is None else blkWarpNum) | self.bw_flags)
@@ -274,6 +300,8 @@ class pcsr_spmm(object):
             raise ValueError("H and w should be given")
         if self.vec_size == 3:
             raise NotImplementedError("the fused GCN operators exist for vec_size 1 and 2 (SpCONV/SpCONV.cpp:498-511)")
+        if self.window:
+            return SpCONV.aggregate(4, SpCONV.dense_xw(H, w, False), self.rowPtr_w, self.colIdx, self.val, None, self.CF, 4)
         fn = getattr(SpCONV, _SPMM[self._key()] + "_forward")
         return fn(H, w, *self._sparse_args(), self.CF, self.blkWarpNum | self.bw_flags)
 
@@ -282,6 +310,9 @@ class pcsr_spmm(object):
             raise ValueError("d_output and H should be given")
         if self.vec_size == 3:
             raise NotImplementedError("the fused GCN operators exist for vec_size 1 and 2 (SpCONV/SpCONV.cpp:498-511)")
+        if self.window:
+            AG = SpCONV.aggregate(4, d_output, self.rowPtr_w, self.colIdx, self.val, None, self.CF, 4)
+            return SpCONV.dense_xw(AG, w, True), SpCONV.weight_gradient(H, AG)
         fn = getattr(SpCONV, _SPMM[self._key()] + "_backward")
         d_input, d_weight = fn(d_output, H, w, *self._sparse_args(), self.CF, self.blkWarpNum | self.bw_flags)
         return d_input, d_weight
@@ -291,6 +322,12 @@ class pcsr_spmm(object):
         """GFLOP/s (int) of this variant with an explicit (CF, blkWarpNum) (PCSR.py:433-505)."""
         assert torch.cuda.is_available()
         X = self._dense_input(dim, x)
+        if self.window:  # no *_profile twin: the event-timed mean of the same number of launches
+            ms = SpMM.spmm_time_ms(4, X, self.rowPtr_w, self.colIdx, self.val, None, CF if 0 <= CF <= 3 else 0, 4, 20, 200, 0)
+            throughput = int(2.0 * self.mtx_edges * X.size(1) / 1e6 / ms) if ms > 0 else 0
+            if verbose:
+                print("dim: {} gflops: {:.0f}".format(X.size(1), throughput))
+            return throughput
         fn = getattr(SpMM, self._spmm_name() + "_profile")
         args = self._sparse_args()
         if self.vec_size != 1:
@@ -332,8 +369,7 @@ class pcsr_spmm(object):
         training step instead of from the caches the previous, identical launch left warm."""
         if self.vec_size == 3:
             raise NotImplementedError("time_ms covers the four decider formats; use cf_warpnum_profiling for 3x1 blocks")
-        fmt = (1 if self.if_split else 0) + (2 if self.vec_size != 1 else 0)
-        return SpMM.spmm_time_ms(fmt, X, self.rowPtr, self.colIdx, self.val, self.target_row,
+        return SpMM.spmm_time_ms(self.fmt_code, X, self.spmm_rowPtr, self.colIdx, self.val, self.target_row,
                                  self.CF if CF is None else CF,
                                  (self.blkWarpNum if blkWarpNum is None else blkWarpNum) | self.bw_flags, warmup, iters,
                                  int(flush_bytes))

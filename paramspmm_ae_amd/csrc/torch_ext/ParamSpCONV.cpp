@@ -6,8 +6,12 @@
 using namespace pspglue;
 using torch::Tensor;
 
-static void check_cf(int CF)
+static void check_cf(int CF, int fmt = 0)
 {
+    if (fmt == 4) {  // windowed csr: CF names the kernel variant
+        TORCH_CHECK(CF >= 0 && CF <= 3, "the windowed format takes variant 0..3 in place of CF");
+        return;
+    }
     // SpCONV dispatches CF 1..4 only (SpCONV/SpCONV.cpp:92-124)
     TORCH_CHECK((CF >= 1 && CF <= 8) || (CF & PSP_CF_NATIVE), "CF must be 1..8 (or a native configuration)");
 }
@@ -17,7 +21,7 @@ static void check_cf(int CF)
 static Tensor aggregate(int fmt, const Tensor &D, const Tensor &rowPtr, const Tensor &colIdx, const Tensor &values,
                         const Tensor *target_row, int CF, int blkWarpNum)
 {
-    check_cf(CF);
+    check_cf(CF, fmt);
     Tensor Dc = D.contiguous();
     Tensor Y = spmm_new(fmt, Dc, rowPtr, colIdx, values, target_row, CF, blkWarpNum);
     if (Y.size(0) != Dc.size(0)) Y = Y.narrow(0, 0, Dc.size(0));
@@ -115,7 +119,7 @@ static Tensor relu_input_forward(int fmt, Tensor Z, Tensor W, Tensor rowPtr, Ten
 {
     need_gpu(Z, "input");
     need_gpu(W, "weight");
-    TORCH_CHECK(fmt >= 0 && fmt <= 3 && ((fmt & 1) != 0) == target_row.has_value(), "format code and target_row disagree");
+    TORCH_CHECK(fmt >= 0 && fmt <= 4 && (fmt == 1 || fmt == 3) == target_row.has_value(), "format code and target_row disagree");
     return aggregate(fmt, dense_relu_xw(Z, W), rowPtr, colIdx, values, target_row ? &*target_row : nullptr, CF, bw);
 }
 // [dZ, dW] = [ ((A dY) W^T) where Z > 0,  relu(Z)^T (A dY) ]
@@ -124,7 +128,7 @@ static std::vector<Tensor> relu_input_backward(int fmt, Tensor dY, Tensor Z, Ten
 {
     need_gpu(Z, "input");
     need_gpu(W, "weight");
-    TORCH_CHECK(fmt >= 0 && fmt <= 3 && ((fmt & 1) != 0) == target_row.has_value(), "format code and target_row disagree");
+    TORCH_CHECK(fmt >= 0 && fmt <= 4 && (fmt == 1 || fmt == 3) == target_row.has_value(), "format code and target_row disagree");
     Tensor AG = aggregate(fmt, dY, rowPtr, colIdx, values, target_row ? &*target_row : nullptr, CF, bw);
     return {dense_xwt_masked(AG, W, Z), weight_gradient_relu(Z, AG)};
 }
@@ -136,7 +140,7 @@ static Tensor aggregate_op(int fmt, Tensor D, Tensor rowPtr, Tensor colIdx, Tens
                            int CF, int bw)
 {
     need_gpu(D, "input");
-    TORCH_CHECK(fmt >= 0 && fmt <= 3 && ((fmt & 1) != 0) == target_row.has_value(), "format code and target_row disagree");
+    TORCH_CHECK(fmt >= 0 && fmt <= 4 && (fmt == 1 || fmt == 3) == target_row.has_value(), "format code and target_row disagree");
     return aggregate(fmt, D, rowPtr, colIdx, values, target_row ? &*target_row : nullptr, CF, bw);
 }
 
@@ -149,15 +153,16 @@ static Tensor aggregate_act_op(int fmt, Tensor D, Tensor rowPtr, Tensor colIdx, 
                                int CF, int bw, bool relu_input, c10::optional<Tensor> mask)
 {
     need_gpu(D, "input");
-    TORCH_CHECK(fmt >= 0 && fmt <= 3 && ((fmt & 1) != 0) == target_row.has_value(), "format code and target_row disagree");
-    check_cf(CF);
+    TORCH_CHECK(fmt >= 0 && fmt <= 4 && (fmt == 1 || fmt == 3) == target_row.has_value(), "format code and target_row disagree");
+    check_cf(CF, fmt);
     const Tensor *tr = target_row ? &*target_row : nullptr;
     if (mask) {
         need_gpu(*mask, "mask");
         TORCH_CHECK(mask->dim() == 2 && mask->size(0) == D.size(0) && mask->size(1) == D.size(1), "mask must have the shape of the result");
     }
+    const bool blocked = pspglue::fmt_blocked(fmt);
     const bool fused = D.scalar_type() == torch::kFloat32 && (!mask || mask->scalar_type() == torch::kFloat32) &&
-                       D.size(1) > 0 && D.size(0) > 0 && (fmt < 2 || D.size(0) % 2 == 0 || !mask);
+                       D.size(1) > 0 && D.size(0) > 0 && (!blocked || D.size(0) % 2 == 0 || !mask);
     if (!fused) {
         Tensor Y = aggregate(fmt, relu_input ? torch::relu(D) : D, rowPtr, colIdx, values, tr, CF, bw);
         return mask ? at::threshold_backward(Y, *mask, 0) : Y;
@@ -165,13 +170,18 @@ static Tensor aggregate_act_op(int fmt, Tensor D, Tensor rowPtr, Tensor colIdx, 
     Tensor Dc = D.contiguous();
     check_spmm_args(fmt, Dc, rowPtr, colIdx, values, tr);
     DeviceGuard guard(Dc.device());
-    const long rows_out = fmt >= 2 ? (Dc.size(0) + 1) / 2 * 2 : Dc.size(0);
+    const long rows_out = blocked ? (Dc.size(0) + 1) / 2 * 2 : Dc.size(0);
     Tensor Mc;
     if (mask) Mc = mask->contiguous();
     Tensor Y = torch::empty({rows_out, Dc.size(1)}, Dc.options());
-    ok(psp_spmm_act_f32(fmt, ip(rowPtr), ip(colIdx), fp(values), tr ? ip(*tr) : nullptr, fp(Dc), fpw(Y),
-                        (int)rowPtr.size(0) - 1, (int)Dc.size(1), (int)rows_out, CF, bw, relu_input ? 1 : 0,
-                        mask ? fp(Mc) : nullptr, stream_of(Dc)));
+    if (fmt == 4)  // windowed csr: the activation is applied as the window is staged, the mask where a row is stored
+        ok(psp_spmm_window_f32(ip(rowPtr), ip(colIdx), fp(values), fp(Dc), fpw(Y), pspglue::fmt_rows(fmt, rowPtr),
+                               (int)colIdx.size(0), (int)Dc.size(1), (int)rows_out, CF, relu_input ? 1 : 0,
+                               mask ? fp(Mc) : nullptr, stream_of(Dc)));
+    else
+        ok(psp_spmm_act_f32(fmt, ip(rowPtr), ip(colIdx), fp(values), tr ? ip(*tr) : nullptr, fp(Dc), fpw(Y),
+                            (int)rowPtr.size(0) - 1, (int)Dc.size(1), (int)rows_out, CF, bw, relu_input ? 1 : 0,
+                            mask ? fp(Mc) : nullptr, stream_of(Dc)));
     if (Y.size(0) != Dc.size(0)) Y = Y.narrow(0, 0, Dc.size(0));
     return Y;
 }

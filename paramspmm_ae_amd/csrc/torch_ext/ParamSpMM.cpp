@@ -104,13 +104,13 @@ static double spmm_time_ms(int fmt, Tensor input, Tensor rowPtr, Tensor colIdx, 
                            c10::optional<Tensor> target_row, int CF, int blkWarpNum, int warmup, int iters,
                            int64_t flush_bytes)
 {
-    TORCH_CHECK(fmt >= 0 && fmt <= 3, "fmt must be 0 (csr), 1 (csr_split), 2 (bcsr) or 3 (bcsr_split)");
-    TORCH_CHECK((fmt & 1) == (target_row.has_value() ? 1 : 0), "target_row must be given exactly for split formats");
+    TORCH_CHECK(fmt >= 0 && fmt <= 4, "fmt must be 0 (csr), 1 (csr_split), 2 (bcsr), 3 (bcsr_split) or 4 (windowed csr)");
+    TORCH_CHECK((fmt == 1 || fmt == 3) == target_row.has_value(), "target_row must be given exactly for split formats");
     TORCH_CHECK(warmup >= 0 && iters >= 1, "warmup >= 0 and iters >= 1 required");
     const Tensor *tr = target_row.has_value() ? &target_row.value() : nullptr;
     check_spmm_args(fmt, input, rowPtr, colIdx, values, tr);
     pspglue::DeviceGuard guard(input.device());
-    const long rows_out = fmt >= 2 ? (input.size(0) + 1) / 2 * 2 : input.size(0);
+    const long rows_out = pspglue::fmt_blocked(fmt) ? (input.size(0) + 1) / 2 * 2 : input.size(0);
     auto Y = torch::empty({rows_out, input.size(1)}, input.options());
     hipStream_t s = (hipStream_t)stream_of(input);
     auto launch = [&] { spmm_into(fmt, Y, input, rowPtr, colIdx, values, tr, CF, blkWarpNum); };
@@ -275,6 +275,47 @@ static double vendor_spmm_time_ms(int format, Tensor X, Tensor ia, Tensor ib, Te
     return (double)time_launches((hipStream_t)stream_of(X), warmup, iters, [&] { op.run(); });
 }
 
+// ---- windowed CSR (an addition of this build, include/paramsp.h: psp_window_build / psp_spmm_window_f32) ------------
+// [rowPtr_w (2M + 2), colIdx_w, val_w] of a CSR matrix, on the device the arrays live on (CPU tensors: host builder)
+static std::vector<Tensor> window_build(Tensor rowPtr, Tensor colIdx, Tensor values)
+{
+    need_i32(rowPtr, "rowPtr");
+    need_i32(colIdx, "colIdx");
+    need_f32(values, "values", 1);
+    TORCH_CHECK(rowPtr.size(0) >= 1 && values.size(0) == colIdx.size(0), "window_build: array sizes disagree");
+    TORCH_CHECK(rowPtr.is_contiguous() && colIdx.is_contiguous() && values.is_contiguous(), "window_build: contiguous arrays");
+    pspglue::same_device(rowPtr, colIdx, "window_build");
+    pspglue::same_device(rowPtr, values, "window_build");
+    const int M = (int)rowPtr.size(0) - 1;
+    Tensor rp = torch::empty({2 * (long)M + 2}, rowPtr.options());
+    Tensor ci = torch::empty_like(colIdx), v = torch::empty_like(values);
+    if (rowPtr.device().is_cpu()) {
+        ok(psp_window_build(ip(rowPtr), ip(colIdx), fp(values), M, rp.data_ptr<int>(), colIdx.numel() ? ci.data_ptr<int>() : nullptr,
+                            fpw(v)));
+    } else {
+        DeviceGuard guard(rowPtr.device());
+        ok(psp_window_build_dev(ip(rowPtr), ip(colIdx), fp(values), M, rp.data_ptr<int>(),
+                                colIdx.numel() ? ci.data_ptr<int>() : nullptr, fpw(v), stream_of(rowPtr)));
+    }
+    return {rp, ci, v};
+}
+static Tensor window_spmm(Tensor input, Tensor rowPtr_w, Tensor colIdx_w, Tensor values_w, int variant)
+{
+    return pspglue::spmm_new(4, input, rowPtr_w, colIdx_w, values_w, nullptr, variant, 4);
+}
+static py::dict window_plan(int N, int variant)
+{
+    int tn = 0, rb = 0, lds = 0;
+    const int v = psp_spmm_window_plan(N, variant, &tn, &rb, &lds);
+    ok(v);
+    py::dict d;
+    d["variant"] = v;
+    d["tile_cols"] = tn;
+    d["rows_per_block"] = rb;
+    d["lds_bytes"] = lds;
+    return d;
+}
+
 static py::dict spmm_plan(int N, int CF, int blkWarpNum)
 {
     psp_spmm_plan p;
@@ -296,6 +337,9 @@ static py::dict spmm_plan(int N, int CF, int blkWarpNum)
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
 {
     pspglue::check_abi();
+    m.def("window_build", &window_build, "windowed CSR of a CSR matrix: (rowPtr, colIdx, values) -> [rowPtr_w, colIdx_w, values_w]");
+    m.def("window_spmm", &window_spmm, "windowed CSR SpMM (HIP, gfx950): (X, rowPtr_w, colIdx_w, values_w, variant)");
+    m.def("window_plan", &window_plan, "(N, variant) -> tile width, rows per workgroup, LDS bytes of the windowed kernel");
     m.def("split_csr", &pspglue::split_csr, "row split on the host (CPU int32 rowPtr, granularity)");
     m.def("split_csr_par", &pspglue::split_csr_par, "row split on the host with a precomputed segment prefix");
     m.def("csr_spmm", &csr_spmm, "CSR SpMM (HIP, gfx950)");

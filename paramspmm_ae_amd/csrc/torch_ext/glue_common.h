@@ -121,8 +121,14 @@ inline std::vector<torch::Tensor> split_csr_par(torch::Tensor rowPtr, torch::Ten
 }
 
 // ---- SpMM into a fresh tensor ------------------------------------------------------------------------
-// fmt: 0 csr, 1 csr_split, 2 bcsr, 3 bcsr_split.  Output rows follow the reference: rows(X) for csr formats
-// (zeros_like, SpMM_kernel.cu:136,208), rows(X) rounded up to even for bcsr formats (281-282, 352-353).
+// fmt: 0 csr, 1 csr_split, 2 bcsr, 3 bcsr_split, 4 windowed csr (an addition of this build: rowPtr is the
+// [2M + 2] array of psp_window_build, CF selects the kernel variant).  Output rows follow the reference: rows(X) for
+// csr formats (zeros_like, SpMM_kernel.cu:136,208), rows(X) rounded up to even for bcsr formats (281-282, 352-353).
+inline bool fmt_blocked(int fmt) { return fmt == 2 || fmt == 3; }
+inline int fmt_rows(int fmt, const torch::Tensor &rowPtr)
+{
+    return fmt == 4 ? (int)(rowPtr.size(0) - 2) / 2 : (int)rowPtr.size(0) - 1;
+}
 inline void check_spmm_args(int fmt, const torch::Tensor &X, const torch::Tensor &rowPtr, const torch::Tensor &colIdx,
                             const torch::Tensor &values, const torch::Tensor *target_row)
 {
@@ -133,7 +139,8 @@ inline void check_spmm_args(int fmt, const torch::Tensor &X, const torch::Tensor
     need_fp(X, "input", 2);
     need_i32(rowPtr, "rowPtr");
     need_i32(colIdx, "colIdx");
-    const bool blocked = fmt >= 2;
+    TORCH_CHECK(fmt >= 0 && fmt <= 4, "format code must be 0..4");
+    const bool blocked = fmt_blocked(fmt);
     need_fp(values, "values", blocked ? 2 : 1);
     same_dtype(X, values, "spmm");
     if (blocked) TORCH_CHECK(values.size(1) == 2, "values of a bcsr format must be [nblk, 2]");
@@ -148,8 +155,14 @@ inline void check_spmm_args(int fmt, const torch::Tensor &X, const torch::Tensor
         same_device(X, *target_row, "spmm");
         TORCH_CHECK(target_row->size(0) == rowPtr.size(0) - 1, "target_row must have one entry per row segment");
     }
-    const long rows = rowPtr.size(0) - 1;
-    if (fmt == 0) TORCH_CHECK(rows <= X.size(0), "rowPtr describes more rows than input has");
+    if (fmt == 4) {
+        TORCH_CHECK(rowPtr.size(0) >= 2 && rowPtr.size(0) % 2 == 0, "rowPtr of the windowed format has 2 M + 2 entries");
+        TORCH_CHECK(!target_row, "the windowed format has no target_row");
+        TORCH_CHECK(X.scalar_type() == torch::kFloat32 && X.size(1) % 4 == 0,
+                    "the windowed format takes float32 input whose width is a multiple of 4");
+    }
+    const long rows = fmt_rows(fmt, rowPtr);
+    if (fmt == 0 || fmt == 4) TORCH_CHECK(rows <= X.size(0), "rowPtr describes more rows than input has");
     if (fmt == 2) TORCH_CHECK(2 * rows <= (X.size(0) + 1) / 2 * 2, "rowPtr describes more block-rows than input has");
 }
 
@@ -157,12 +170,17 @@ inline void spmm_into(int fmt, torch::Tensor &Y, const torch::Tensor &X, const t
                       const torch::Tensor &colIdx, const torch::Tensor &values, const torch::Tensor *target_row,
                       int CF, int blkWarpNum)
 {
-    const int nrows = (int)rowPtr.size(0) - 1, N = (int)X.size(1), rows_out = (int)Y.size(0);
+    const int nrows = fmt_rows(fmt, rowPtr), N = (int)X.size(1), rows_out = (int)Y.size(0);
     if (N == 0 || rows_out == 0) return;
     psp_stream_t s = stream_of(X);
+    if (fmt == 4) {
+        ok(psp_spmm_window_f32(ip(rowPtr), ip(colIdx), fp(values), fp(X), fpw(Y), nrows, (int)colIdx.size(0), N, rows_out, CF, 0,
+                               nullptr, s));
+        return;
+    }
     if (is_f64(X)) {
         ok(psp_spmm_f64(ip(rowPtr), ip(colIdx), dp(values), target_row ? ip(*target_row) : nullptr, dp(X), dpw(Y), nrows, N,
-                        rows_out, fmt >= 2 ? 2 : 1, s));
+                        rows_out, fmt_blocked(fmt) ? 2 : 1, s));
         return;
     }
     int rc;
@@ -180,7 +198,7 @@ inline torch::Tensor spmm_new(int fmt, const torch::Tensor &X, const torch::Tens
 {
     check_spmm_args(fmt, X, rowPtr, colIdx, values, target_row);
     pspglue::DeviceGuard guard(X.device());
-    const long rows_out = fmt >= 2 ? (X.size(0) + 1) / 2 * 2 : X.size(0);
+    const long rows_out = fmt_blocked(fmt) ? (X.size(0) + 1) / 2 * 2 : X.size(0);
     // the library defines every element of Y, so no zero-initialised allocation is needed
     auto Y = torch::empty({rows_out, X.size(1)}, X.options());
     spmm_into(fmt, Y, X, rowPtr, colIdx, values, target_row, CF, blkWarpNum);

@@ -29,10 +29,20 @@ def _conv_name(op):
     return _CONV[(bool(op.if_split), op.vec_size != 1)]
 
 
+def _fmt(op):
+    """Format code of the generic entry points (pcsr_spmm.fmt_code: 0 csr, 1 csr_split, 2 bcsr, 3 bcsr_split,
+    4 windowed csr); operators of other origin are described by if_split / vec_size."""
+    code = getattr(op, "fmt_code", None)
+    return (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0) if code is None else code
+
+
+def _row_ptr(op):
+    return getattr(op, "spmm_rowPtr", op.rowPtr)
+
+
 def _aggregate(op, D):
     """A D through ``op``'s format and configuration."""
-    fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
-    return SpCONV.aggregate(fmt, D, op.rowPtr, op.colIdx, op.val, op.target_row if op.if_split else None, op.CF,
+    return SpCONV.aggregate(_fmt(op), D, _row_ptr(op), op.colIdx, op.val, op.target_row if op.if_split else None, op.CF,
                             _bw(op))
 
 
@@ -69,6 +79,8 @@ class GCNFunction(torch.autograd.Function):
     def forward(ctx, H, weight, ParamSpMM):
         ctx.save_for_backward(H, weight)
         ctx.ParamSpMM = ParamSpMM
+        if _fmt(ParamSpMM) == 4:  # the windowed layout has no named operator of its own: dense product, then A
+            return _aggregate(ParamSpMM, SpCONV.dense_xw(H, weight, False))
         return getattr(SpCONV, _conv_name(ParamSpMM) + "_forward")(H, weight, *_conv_args(ParamSpMM))
 
     @staticmethod
@@ -78,6 +90,9 @@ class GCNFunction(torch.autograd.Function):
         if not ctx.needs_input_grad[0]:
             # the network's first layer: its input holds features, nothing asks for their gradient
             return None, SpCONV.weight_gradient(H, _aggregate(op, d_output)), None
+        if _fmt(op) == 4:
+            AG = _aggregate(op, d_output.contiguous())
+            return SpCONV.dense_xw(AG, weight, True), SpCONV.weight_gradient(H, AG), None
         d_input, d_weight = getattr(SpCONV, _conv_name(op) + "_backward")(d_output.contiguous(), H, weight, *_conv_args(op))
         return d_input, d_weight, None
 
@@ -118,16 +133,14 @@ class GCNReLUInputFunction(torch.autograd.Function):
         ctx.save_for_backward(Z, weight)
         ctx.ParamSpMM = ParamSpMM
         op = ParamSpMM
-        fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
-        return SpCONV.relu_input_forward(fmt, Z, weight, op.rowPtr, op.colIdx, op.val,
+        return SpCONV.relu_input_forward(_fmt(op), Z, weight, _row_ptr(op), op.colIdx, op.val,
                                          op.target_row if op.if_split else None, op.CF, _bw(op))
 
     @staticmethod
     def backward(ctx, d_output):
         Z, weight = ctx.saved_tensors
         op = ctx.ParamSpMM
-        fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
-        d_input, d_weight = SpCONV.relu_input_backward(fmt, d_output.contiguous(), Z, weight, op.rowPtr, op.colIdx, op.val,
+        d_input, d_weight = SpCONV.relu_input_backward(_fmt(op), d_output.contiguous(), Z, weight, _row_ptr(op), op.colIdx, op.val,
                                                        op.target_row if op.if_split else None, op.CF, _bw(op))
         return d_input, d_weight, None
 
@@ -250,8 +263,7 @@ class GINReLUInputFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, Z, weight, ParamSpMM):
         op = ParamSpMM
-        fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
-        X_agg = SpCONV.aggregate_act(fmt, Z, op.rowPtr, op.colIdx, op.val, op.target_row if op.if_split else None, op.CF,
+        X_agg = SpCONV.aggregate_act(_fmt(op), Z, _row_ptr(op), op.colIdx, op.val, op.target_row if op.if_split else None, op.CF,
                                      _bw(op), True, None)
         ctx.save_for_backward(X_agg, weight, Z)
         ctx.ParamSpMM = op
@@ -261,10 +273,9 @@ class GINReLUInputFunction(torch.autograd.Function):
     def backward(ctx, d_output):
         X_agg, weights, Z = ctx.saved_tensors
         op = ctx.ParamSpMM
-        fmt = (1 if op.if_split else 0) + (2 if op.vec_size != 1 else 0)
         d_output = d_output.contiguous()
         d_weights = SpCONV.weight_gradient(X_agg, d_output)
-        d_input = SpCONV.aggregate_act(fmt, SpCONV.dense_xw(d_output, weights, True), op.rowPtr, op.colIdx, op.val,
+        d_input = SpCONV.aggregate_act(_fmt(op), SpCONV.dense_xw(d_output, weights, True), _row_ptr(op), op.colIdx, op.val,
                                        op.target_row if op.if_split else None, op.CF, _bw(op), False, Z)
         return d_input, d_weights, None
 

@@ -103,6 +103,29 @@ class csr_data(object):
     def _keep_device(self, name, tensor):
         self._dev[(name, tensor.device)] = tensor
 
+    def window_format(self, device="cuda"):
+        """(rowPtr_w, colIdx_w, val_w, local share) of this CSR matrix in the windowed layout of the library
+        (psp_window_build: every row's entries reordered so that the ones whose column lies within 64 rows of the
+        row's 64-row block come first), built on ``device`` once and kept.  No counterpart in the reference; the
+        CSR arrays must be the plain (vec_size 1) ones."""
+        import ParamSpMM
+
+        device = torch.device(device)
+        if device.type == "cuda" and device.index is None:
+            device = torch.device("cuda", torch.cuda.current_device())
+        key = ("window", device)
+        got = self._dev.get(key)
+        if got is None:
+            if self.val.dim() != 1:
+                raise ValueError("the windowed layout exists for the CSR format (vec_size 1)")
+            rp, ci, v = ParamSpMM.window_build(self.on_device("rowPtr", device), self.on_device("colIdx", device),
+                                               self.on_device("val", device))
+            nnz = max(int(self.colIdx.numel()), 1)
+            local = float((rp[1:-1:2].long() - rp[0:-2:2].long()).sum().item()) / nnz
+            got = (rp, ci, v, local)
+            self._dev[key] = got
+        return got
+
     def xcd_stripe(self, split):
         """Rows (segments when ``split``) the SpMM kernel should deal to one XCD at a time for this format: the
         longest of XCD_STRIPES under which the eight XCDs get equal shares of the stored entries (largest share at

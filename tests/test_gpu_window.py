@@ -1,0 +1,225 @@
+"""Windowed CSR (psp_window_build / psp_spmm_window_f32): the format builders against a numpy restatement, bit for bit
+(index work), and the SpMM against the CPU oracle's CSR product within rel 1e-5 / abs 1e-6 (the kernel adds a row's
+local entries before its remote ones, so it is not bit-identical to the sequential chain), through the C ABI, the
+extension modules and the GNN layers."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from conftest import random_csr
+
+BLOCK, HALO = 64, 64
+
+
+def banded_csr(n, per_row, width, seed, far=0.0, hub=None, empty_frac=0.0):
+    """Rows with ``per_row`` (Poisson) entries within +-width of the diagonal, a share ``far`` of them anywhere."""
+    rng = np.random.default_rng(seed)
+    deg = rng.poisson(per_row, n)
+    if empty_frac:
+        deg[rng.random(n) < empty_frac] = 0
+    if hub is not None:
+        deg[hub[0]] = hub[1]
+    cols = []
+    for i, d in enumerate(deg):
+        near = np.clip(i + rng.integers(-width, width + 1, d), 0, n - 1)
+        anywhere = rng.integers(0, n, d)
+        c = np.unique(np.where(rng.random(d) < far, anywhere, near))
+        cols.append(c)
+    rowPtr = np.zeros(n + 1, np.int32)
+    rowPtr[1:] = np.cumsum([c.size for c in cols])
+    colIdx = (np.concatenate(cols) if rowPtr[-1] else np.zeros(0)).astype(np.int32)
+    val = rng.uniform(0.1, 1.0, colIdx.size).astype(np.float32)
+    return rowPtr, colIdx, val
+
+
+def window_reference(rowPtr, colIdx, val):
+    """numpy restatement of the format: per row the entries whose column lies in [64 (r // 64) - 64, 64 (r // 64) + 128)
+    first, the others after, each part in the original order."""
+    M = rowPtr.size - 1
+    rows = np.repeat(np.arange(M, dtype=np.int64), np.diff(rowPtr))
+    lo = rows // BLOCK * BLOCK - HALO
+    local = (colIdx >= lo) & (colIdx < lo + BLOCK + 2 * HALO)
+    order = np.lexsort((np.arange(colIdx.size), ~local, rows))  # stable: row, then local first, then position
+    rp = np.empty(2 * M + 2, np.int32)
+    rp[0:2 * M:2] = rowPtr[:-1]
+    cs = np.concatenate([[0], np.cumsum(local)])
+    rp[1:2 * M:2] = rowPtr[:-1] + (cs[rowPtr[1:]] - cs[rowPtr[:-1]])  # start of the remote part
+    rp[2 * M] = rp[2 * M + 1] = rowPtr[-1]
+    return rp, colIdx[order], val[order], float(local.mean()) if colIdx.size else 0.0
+
+
+CASES = {
+    "banded": lambda: banded_csr(5000, 14, 40, 1, far=0.1, empty_frac=0.05),
+    "banded_hub": lambda: banded_csr(3001, 9, 30, 2, far=0.15, hub=(70, 900)),
+    "wide_band": lambda: banded_csr(2000, 60, 60, 3, far=0.02),       # rows with more than 32 local entries
+    "random": lambda: random_csr(4099, 11, 4, empty_frac=0.1, hub=(5, 700), values="uniform"),  # nearly all remote
+    "tiny": lambda: banded_csr(37, 3, 5, 5),
+    "one_block": lambda: banded_csr(64, 6, 64, 6),
+}
+
+
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_host_builder_matches_the_numpy_restatement(name):
+    from paramspmm_ae_amd import _capi
+
+    rowPtr, colIdx, val = CASES[name]()
+    M, nnz = rowPtr.size - 1, colIdx.size
+    rp, ci, v = np.full(2 * M + 2, -7, np.int32), np.full(nnz, -7, np.int32), np.full(nnz, np.nan, np.float32)
+    p = _capi.ptr
+    _capi.check(_capi.lib.psp_window_build(p(rowPtr), p(colIdx), p(val), M, p(rp), p(ci), p(v)))
+    want = window_reference(rowPtr, colIdx, val)
+    assert np.array_equal(rp, want[0]) and np.array_equal(ci, want[1]) and np.array_equal(v, want[2])
+    # the permutation stays inside the rows
+    for r in range(0, M, max(1, M // 50)):
+        a, b = rowPtr[r], rowPtr[r + 1]
+        assert sorted(ci[a:b].tolist()) == sorted(colIdx[a:b].tolist())
+
+
+def test_host_builder_rejects_a_broken_row_pointer():
+    from paramspmm_ae_amd import _capi
+
+    p = _capi.ptr
+    rowPtr = np.array([0, 3, 2, 4], np.int32)
+    z = np.zeros(8, np.int32)
+    f = np.zeros(8, np.float32)
+    assert _capi.lib.psp_window_build(p(rowPtr), p(z), p(f), 3, p(np.zeros(8, np.int32)), p(z.copy()), p(f.copy())) == -1
+    a, b, c = ctypes.c_int(), ctypes.c_int(), ctypes.c_int()
+    assert _capi.lib.psp_spmm_window_plan(18, 0, a, b, c) == -1      # width not a multiple of 4
+    assert _capi.lib.psp_spmm_window_plan(64, 4, a, b, c) == -1      # no such variant
+    assert [_capi.lib.psp_spmm_window_plan(n, 0, a, b, c) for n in (4, 16, 20, 32, 36, 256)] == [1, 1, 2, 2, 3, 3]
+
+
+def _spmm_window(F, X, variant=0, relu=False, mask=None, rows_out=None):
+    from paramspmm_ae_amd import _capi
+
+    rp, ci, v, M = F
+    rows_out = X.shape[0] if rows_out is None else rows_out
+    Y = torch.full((rows_out, X.shape[1]), float("nan"), device="cuda")
+    p = _capi.ptr
+    _capi.check(_capi.lib.psp_spmm_window_f32(p(rp), p(ci), p(v), p(X), p(Y), M, int(ci.numel()), X.shape[1], rows_out, variant, int(relu),
+                                              p(mask), torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    return Y
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_device_builder_and_spmm_against_the_oracle(oracle, name):
+    from gpu_util import assert_close, dev
+    from paramspmm_ae_amd import _capi
+
+    rowPtr, colIdx, val = CASES[name]()
+    M, nnz = rowPtr.size - 1, colIdx.size
+    want_fmt = window_reference(rowPtr, colIdx, val)
+    rp = torch.full((2 * M + 2,), -7, dtype=torch.int32, device="cuda")
+    ci = torch.full((max(nnz, 1),), -7, dtype=torch.int32, device="cuda")[:nnz]
+    v = torch.full((max(nnz, 1),), float("nan"), device="cuda")[:nnz]
+    p = _capi.ptr
+    print("case build", name, M, nnz, flush=True)
+    rp_in, ci_in, v_in = dev(rowPtr), dev(colIdx), dev(val)  # named: the arrays must outlive the launch that reads them
+    _capi.check(_capi.lib.psp_window_build_dev(p(rp_in), p(ci_in), p(v_in), M, p(rp), p(ci), p(v),
+                                               torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    assert np.array_equal(rp.cpu().numpy(), want_fmt[0])
+    assert np.array_equal(ci.cpu().numpy(), want_fmt[1]) and np.array_equal(v.cpu().numpy(), want_fmt[2])
+    F = (rp, ci, v, M)
+    for N in (4, 16, 20, 32, 48, 64, 100, 128, 256):
+        X = np.random.default_rng(N).standard_normal((M + 3, N)).astype(np.float32)
+        want = oracle.spmm_csr(rowPtr, colIdx, val, X, rows_out=M + 3)
+        scale = oracle.spmm_csr(rowPtr, colIdx, np.abs(val), np.abs(X), rows_out=M + 3)
+        Xd = torch.from_numpy(X).cuda()
+        for variant in (0, 1, 2, 3):
+            print("case spmm", name, N, variant, flush=True)
+            got = _spmm_window(F, Xd, variant)
+            assert_close(got, want, what="%s N=%d variant %d" % (name, N, variant), scale=scale)
+            assert bool((got[M:] == 0).all())
+    # the folded activation and mask: A max(X, 0) equals the product of the clamped input bit for bit; the masked
+    # product equals the plain one where the mask is positive and is an exact zero elsewhere
+    X = torch.randn(M + 1, 64, device="cuda")
+    mask = torch.randn(M + 1, 64, device="cuda")
+    plain = _spmm_window(F, X)
+    assert torch.equal(_spmm_window(F, X, relu=True), _spmm_window(F, torch.relu(X)))
+    got = _spmm_window(F, X, mask=mask)
+    assert torch.equal(got, torch.where(mask > 0, plain, torch.zeros_like(plain)))
+
+
+@pytest.mark.gpu
+def test_non_finite_inputs_stay_in_their_rows(oracle):
+    rowPtr, colIdx, val = banded_csr(1500, 9, 30, 9, far=0.2, hub=(3, 400))
+    from gpu_util import dev
+    from paramspmm_ae_amd import _capi
+    import ParamSpMM
+
+    rp, ci, v = ParamSpMM.window_build(dev(rowPtr), dev(colIdx), dev(val))
+    M = rowPtr.size - 1
+    for N in (16, 64):
+        X = np.random.default_rng(N).standard_normal((M, N)).astype(np.float32)
+        X[colIdx[5]] = np.inf
+        X[colIdx[colIdx.size // 2]] = np.nan
+        X[0] = np.inf       # the row the padding of the index registers points at
+        X[M - 1] = np.inf
+        want = oracle.spmm_csr(rowPtr, colIdx, val, X)
+        got = _spmm_window((rp, ci, v, M), torch.from_numpy(X).cuda()).cpu().numpy()
+        assert np.array_equal(np.isnan(got), np.isnan(want)), N
+        assert np.array_equal(np.isposinf(got), np.isposinf(want))
+        fin = np.isfinite(want)
+        np.testing.assert_allclose(got[fin], want[fin], rtol=1e-4, atol=1e-5)
+
+
+@pytest.mark.gpu
+def test_window_operator_through_the_modules_and_a_gcn_layer(oracle):
+    """pcsr_spmm(window=True): SpMM, the fused forward / backward, the SDDMM on the permuted arrays, and a GCN layer's
+    gradients against dense autograd."""
+    import ParamSpMM
+    from gpu_util import assert_close
+    from paramspmm_ae_amd import gnn_conv
+    from paramspmm_ae_amd.graph_input import graph_input
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+
+    n = 2500
+    rowPtr, colIdx, val = banded_csr(n, 8, 50, 12, far=0.1)
+    # symmetric pattern with symmetric values (the layers multiply by A where the algebra asks for A^T)
+    import scipy.sparse as sp
+
+    A = sp.csr_matrix((val, colIdx, rowPtr), shape=(n, n))
+    A = ((A + A.T) * 0.5).tocsr()
+    A.sort_indices()
+    rowPtr, colIdx, val = A.indptr.astype(np.int32), A.indices.astype(np.int32), A.data.astype(np.float32)
+    g = graph_input("banded", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val)
+    op = pcsr_spmm(g, vec_size=1, if_split=False, window=True)
+    assert op.fmt_code == 4 and 0.5 < op.window_local_share <= 1.0
+    assert abs(op.window_local_share - window_reference(rowPtr, colIdx, val)[3]) < 1e-6
+    X = np.random.default_rng(0).standard_normal((n, 32)).astype(np.float32)
+    want = oracle.spmm_csr(rowPtr, colIdx, val, X)
+    scale = oracle.spmm_csr(rowPtr, colIdx, np.abs(val), np.abs(X))
+    Xd = torch.from_numpy(X).cuda()
+    assert_close(op.GIN_spmm(Xd), want, what="window GIN_spmm", scale=scale)
+    op.get_spmm_result(x=Xd)
+    assert_close(op.result, want, what="window get_spmm_result", scale=scale)
+    assert op.profiling(dim=16, verbose=False) > 0 and op.time_ms(Xd, warmup=1, iters=2) > 0
+    # SDDMM on the permuted arrays: ones -> K for every stored entry
+    assert bool((op.get_sddmm_result(48, 4) == 48).all())
+    # the plain CSR kernel reads the permuted arrays as a matrix with unsorted rows: same product
+    plain = ParamSpMM.csr_spmm(Xd, op.rowPtr, op.colIdx, op.val, 1, 4)
+    assert_close(plain, want, what="csr kernel on the permuted arrays", scale=scale)
+
+    Ad = torch.from_numpy(A.toarray().astype(np.float64)).cuda()
+    for cls, relu_in in ((gnn_conv.GCNConv, False), (gnn_conv.GCNConv, True), (gnn_conv.GINConv, False), (gnn_conv.GINConv, True)):
+        for in_w, out_w in ((32, 16), (16, 32)):
+            layer = cls(in_w, out_w).cuda()
+            H = torch.randn(n, in_w, device="cuda", requires_grad=True)
+            ops = {in_w: op, out_w: op}
+            y = layer(H, ops, relu_input=True) if relu_in else layer(H, ops)
+            dY = torch.randn_like(y)
+            y.backward(dY)
+            Hr = H.detach().double().requires_grad_(True)
+            Wr = layer.weights.detach().double().requires_grad_(True)
+            yr = Ad @ ((torch.relu(Hr) if relu_in else Hr) @ Wr)
+            yr.backward(dY.double())
+            torch.testing.assert_close(y.double(), yr, rtol=1e-4, atol=1e-4)
+            torch.testing.assert_close(H.grad.double(), Hr.grad, rtol=1e-4, atol=1e-4)
+            torch.testing.assert_close(layer.weights.grad.double(), Wr.grad, rtol=1e-3, atol=1e-3)
