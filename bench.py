@@ -118,6 +118,13 @@ def other_graph_leg(name, dims, decider, reps=10):
     rows = (n + 1) // 2 * 2
     gen = torch.Generator(device="cuda").manual_seed(99)
     res = []
+    import ParamSpMM
+    from paramspmm_ae_amd.GNN import WINDOW_MIN_LOCAL_SHARE
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+
+    win = pcsr_spmm(graph, vec_size=1, if_split=False, CF=0, window=True)
+    if win.window_local_share < WINDOW_MIN_LOCAL_SHARE:
+        win = None
     for d in dims:
         X = torch.randn(rows, d, device="cuda", generator=gen)
         if rows != n:
@@ -131,10 +138,20 @@ def other_graph_leg(name, dims, decider, reps=10):
                "gflops": round(2.0 * nnz * d / ms / 1e6, 1), "alg_bytes": int(b_alg),
                "frac": round(b_alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
         row["traffic"] = measured_traffic(name, [row])
+        if win is not None and d % 4 == 0:
+            # the windowed layout beside it (what GNN.configure_operators would keep if it is faster): its algorithmic
+            # bytes are those of the CSR product plus the second row pointer per row
+            ms_w = win.time_ms(X, warmup=3, iters=reps)
+            b_w = algorithmic_bytes("csr", F, n, d) + 4 * (n + 1)
+            row["windowed"] = {"ms": round(float(ms_w), 5), "gflops": round(2.0 * nnz * d / ms_w / 1e6, 1),
+                               "alg_bytes": int(b_w), "frac": round(b_w / ms_w / 1e6 / HBM_PEAK_GBS, 4),
+                               "variant": int(ParamSpMM.window_plan(d, 0)["variant"])}
         res.append(row)
         del X
     out = {"nodes": n, "nnz": int(nnz), "setup_s": round(time.time() - t0, 1), "widths": res}
-    del ops, graph
+    if win is not None:
+        out["window_local_share"] = round(win.window_local_share, 4)
+    del ops, graph, win
     torch.cuda.empty_cache()
     return out
 
@@ -925,7 +942,7 @@ def main():
         if decider is not None:
             out["other_graphs"] = {
                 "C3s 5-point stencil 2048^2": other_graph_leg("C3s", [64, 128], decider),
-                "C5 block model 1M nodes, community order": other_graph_leg("C5", [128], decider),
+                "C5 block model 1M nodes, community order": other_graph_leg("C5", [16, 128], decider),
                 "C5p block model 1M nodes, random order": other_graph_leg("C5p", [128], decider),
                 "C3 Chung-Lu 2.45M nodes": other_graph_leg("C3", [128], decider, reps=5),
             }

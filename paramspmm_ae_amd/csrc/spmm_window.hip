@@ -444,25 +444,33 @@ PSP_EXPORT int psp_spmm_window_plan(int N, int variant, int *tile_cols, int *row
 
 // Blocks one workgroup walks in a row.  Measured on a community-ordered block model (10^6 rows) with runs of 2 .. 64
 // blocks at every width: the longer the run the better -- a run pays for its first window (192 rows instead of 64)
-// and for the one wait the pipeline cannot hide -- up to the point where the launch has just as many workgroups as
-// the GPU holds at once; beyond it CUs idle.  So: one workgroup per slot, each with an equal share of the blocks.
-// workgroups per CU: 4 of 256 lanes, 2 of 512 (registers).  PSP_WINDOW_RUN overrides the choice.
-static int pspw_run_length(int nblocks, int tiles, int threads)
+// and for the one wait the pipeline cannot hide -- up to the point where the launch has exactly as many workgroups as
+// the GPU holds at once.  One workgroup more than that and the launch takes half as long again (the late workgroup
+// starts when the first one ends, and every workgroup runs for the whole launch); fewer and CUs idle.  So the launch
+// is sized from the occupancy the runtime reports for the kernel: at most that many workgroups (a multiple of the
+// 8 XCDs per column tile, so that the grid holds no empty ones), each with an equal share of the blocks.
+// PSP_WINDOW_RUN overrides the choice.
+static int pspw_run_length(int nblocks, int tiles, int variant, const pspw_variant &k, int lds)
 {
     static const int forced = [] {
         const char *e = getenv("PSP_WINDOW_RUN");
         return e ? atoi(e) : 0;
     }();
     if (forced > 0) return forced;
-    static const int cus = [] {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess) return 256;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return 256;
-        return n;
-    }();
-    const long long slots = (long long)cus * (threads <= 256 ? 4 : 2);
-    const long long run = ((long long)nblocks * tiles + slots - 1) / slots;
-    return (int)(run < 1 ? 1 : run);
+    static int slots_of[4];  // workgroups the current GPU holds at once, per variant (0 = not asked yet)
+    if (slots_of[variant] == 0) {
+        int dev = 0, cus = 0, per_cu = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+            cus = 256;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)k.fn, k.threads, (size_t)lds) != hipSuccess || per_cu <= 0)
+            per_cu = 1;
+        slots_of[variant] = cus * per_cu;
+    }
+    int nruns = slots_of[variant] / tiles / PSP_XCDS * PSP_XCDS;
+    if (nruns < PSP_XCDS) nruns = PSP_XCDS;
+    const int run = (nblocks + nruns - 1) / nruns;
+    return run < 1 ? 1 : run;
 }
 
 PSP_EXPORT int psp_spmm_window_f32(const int *rowPtr_w, const int *colIdx_w, const float *val_w, const float *X, float *Y,
@@ -487,9 +495,9 @@ PSP_EXPORT int psp_spmm_window_f32(const int *rowPtr_w, const int *colIdx_w, con
         lds_raised[v] = true;
     }
     const int nblocks = psp_ceil_div(M, rb), tiles = psp_ceil_div(N, tn);
-    const int run = pspw_run_length(nblocks, tiles, k.threads);
+    const int run = pspw_run_length(nblocks, tiles, v, k, lds);
     const int nruns = psp_ceil_div(nblocks, run);
-    const psp_grid1d g = psp_xcd_grid(nruns, psp_ceil_div(8192, rb * run));
+    const psp_grid1d g = psp_xcd_grid(nruns, 1);  // long runs: neighbouring runs share two halo windows, nothing to keep in one L2
     dim3 grid(g.launch, tiles, 1), block(k.threads, 1, 1);
     hipLaunchKernelGGL(k.fn, grid, block, lds, st, rowPtr_w, colIdx_w, val_w, X, Y, mask, M, N, nnz, nruns, g.stripe, run, relu_x != 0);
     return psp_check_launch("spmm window kernel");
