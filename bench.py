@@ -145,7 +145,8 @@ def other_graph_leg(name, dims, decider, reps=10):
             b_w = algorithmic_bytes("csr", F, n, d) + 4 * (n + 1)
             row["windowed"] = {"ms": round(float(ms_w), 5), "gflops": round(2.0 * nnz * d / ms_w / 1e6, 1),
                                "alg_bytes": int(b_w), "frac": round(b_w / ms_w / 1e6 / HBM_PEAK_GBS, 4),
-                               "variant": int(ParamSpMM.window_plan(d, 0)["variant"])}
+                               "variant": int(ParamSpMM.window_plan(d, 0)["variant"]),
+                               "traffic": measured_traffic(name, [{"dim": d, "format": "window", "CF": 0, "blkWarpNum": 0}])}
         res.append(row)
         del X
     out = {"nodes": n, "nnz": int(nnz), "setup_s": round(time.time() - t0, 1), "widths": res}
@@ -562,7 +563,7 @@ def main():
     ap.add_argument("--dims", default=DEFAULT_DIMS)
     ap.add_argument("--pick", default="auto",
                     help="auto (decider if its forests are built, else sweep) | sweep | decider | "
-                         "fixed:<csr|csr_split|bcsr|bcsr_split>:<CF>:<blkWarpNum>")
+                         "fixed:<csr|csr_split|bcsr|bcsr_split>:<CF>:<blkWarpNum> | window[:<variant>] (the windowed layout)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run one plain device copy of X (known size) so a counter run can be calibrated")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -642,6 +643,13 @@ def main():
         decider = SpMMDecider()
         decider.gen_model_dict(dims)
     fixed = None
+    win_op = None
+    if pick.startswith("window"):
+        # the windowed layout at every width: window[:variant]; encoded as vec_size 0 in the configuration tuples
+        from paramspmm_ae_amd.PCSR import pcsr_spmm
+
+        win_op = pcsr_spmm(graph, vec_size=1, if_split=False, CF=0, window=True)
+        fixed = (0, 0, int(pick.split(":")[1]) if ":" in pick else 0, 0)
     if pick.startswith("fixed:"):
         _, f_fmt, f_cf, f_bw = pick.split(":")
         if "." in f_cf:  # native configuration: vectors.lanes.unroll.segments_per_wave[.e]  (0 segments = automatic)
@@ -669,6 +677,11 @@ def main():
 
     def launcher(d, ops_, chosen_):
         if_split, vec, cf, bw = chosen_[d]
+        if vec == 0:
+            X, Y = Xs[d], Ys[d]
+            w = win_op
+            return lambda: L.psp_spmm_window_f32(p(w.rowPtr_w), p(w.colIdx), p(w.val), p(X), p(Y), n, int(w.colIdx.numel()), d,
+                                                 rows, cf, 0, None, stream)
         op = ops_[(1 if if_split else 0) + (2 if vec == 2 else 0)]
         X, Y = Xs[d], Ys[d]
         a = (p(op.rowPtr), p(op.colIdx), p(op.val))
@@ -728,14 +741,16 @@ def main():
     for d in dims:
         ms = float(np.mean([a.elapsed_time(b) for a, b in events[d]]))
         if_split, vec, cf, bw = chosen[d]
-        fmt = fmt_names[(1 if if_split else 0) + (2 if vec == 2 else 0)]
-        b_alg = algorithmic_bytes(fmt, F, n, d)
+        windowed = vec == 0
+        fmt = "window" if windowed else fmt_names[(1 if if_split else 0) + (2 if vec == 2 else 0)]
+        # windowed layout: the CSR arrays and one more row pointer per row
+        b_alg = algorithmic_bytes("csr", F, n, d) + 4 * (n + 1) if windowed else algorithmic_bytes(fmt, F, n, d)
         gbs = b_alg / (ms * 1e-3) / 1e9
         # no-reuse gather volume: every stored entry fetches its row of X (what a matrix without locality moves)
         stored = F["nblk"] if fmt.startswith("bcsr") else nnz
         b_gather = b_alg - 4 * n * d + 4 * stored * d
-        per_dim.append({"dim": d, "format": fmt, "CF": cf, "config": sweep.cf_label(cf), "blkWarpNum": bw,
-                        "xcd_stripe_rows": (ops[(1 if if_split else 0) + (2 if vec == 2 else 0)].bw_flags >> 12) * 256,
+        per_dim.append({"dim": d, "format": fmt, "CF": cf, "config": "variant %d" % cf if windowed else sweep.cf_label(cf), "blkWarpNum": bw,
+                        "xcd_stripe_rows": 0 if windowed else (ops[(1 if if_split else 0) + (2 if vec == 2 else 0)].bw_flags >> 12) * 256,
                         "ms": round(ms, 5),
                         "gflops": round(2.0 * nnz * d / (ms * 1e-3) / 1e9, 1), "alg_bytes": b_alg,
                         "alg_GBps": round(gbs, 1), "frac_hbm": round(gbs / HBM_PEAK_GBS, 4),
@@ -745,6 +760,14 @@ def main():
     # symbol, which is what a rocprofv3 kernel trace averages over; take the symbol with the largest share of time.
     by_symbol = {}
     for r in per_dim:
+        if r["format"] == "window":
+            import ParamSpMM
+
+            v = int(ParamSpMM.window_plan(r["dim"], r["CF"])["variant"])
+            sym = "psp_spmm_window_kernel<%s>" % {1: "1, 2, 256", 2: "1, 3, 512", 3: "2, 3, 512"}[v]
+            r["kernel"] = sym
+            by_symbol.setdefault(sym, []).append(r)
+            continue
         plan = _capi.spmm_plan(r["dim"], r["CF"], r["blkWarpNum"])
         sym = "psp_spmm_kernel<%d, %d, %d, %d, %s, false, false>" % (plan["coarsen"], plan["vec"], plan["unroll"],
                                                        2 if r["format"].startswith("bcsr") else 1,
@@ -776,7 +799,7 @@ def main():
         "sweep": per_dim,
     }
 
-    if not args.no_extras:
+    if not args.no_extras and win_op is None:
         # ---- gather ceiling of the dominant width: the bare gathers of the same pattern and X row tiles ----------
         dom = max(rows_of, key=lambda r: r["ms"])
         plan = _capi.spmm_plan(dom["dim"], dom["CF"], dom["blkWarpNum"])

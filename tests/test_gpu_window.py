@@ -223,3 +223,44 @@ def test_window_operator_through_the_modules_and_a_gcn_layer(oracle):
             torch.testing.assert_close(y.double(), yr, rtol=1e-4, atol=1e-4)
             torch.testing.assert_close(H.grad.double(), Hr.grad, rtol=1e-4, atol=1e-4)
             torch.testing.assert_close(layer.weights.grad.double(), Wr.grad, rtol=1e-3, atol=1e-3)
+
+
+@pytest.mark.gpu
+def test_training_with_windowed_operators_follows_training_with_the_csr_operators():
+    """A community-ordered block model: most entries are local, configure_operators may keep the windowed layout
+    (decided by timing), and GCN / GIN networks built on windowed operators produce the log-probabilities and take
+    the training steps of the same networks on plain CSR operators (same seed, a few epochs)."""
+    from paramspmm_ae_amd import GNN, synth
+    from paramspmm_ae_amd.graph_input import graph_input
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+
+    n = 40000
+    r, c, n = synth.sbm(n, n // 100, 12, 1.5, seed=5)
+    rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+    g = graph_input("sbm", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val)
+    win = pcsr_spmm(g, vec_size=1, if_split=False, window=True)
+    assert win.window_local_share > 0.8
+    from paramspmm_ae_amd.decider import SpMMDecider
+
+    dec = SpMMDecider()
+    dec.gen_model_dict([16, 32])
+    ops = GNN.configure_operators(dec, g, [16, 32])
+    X = torch.randn(n, 16, device="cuda")
+    plain = pcsr_spmm(g, vec_size=1, if_split=False)
+    want = plain._spmm(X)
+    for d, op in ops.items():  # whichever layout was kept computes the product
+        got = op._spmm(torch.randn(n, d, device="cuda") * 0 + X[:, :1].expand(n, d).contiguous())[:n]
+        torch.testing.assert_close(got[:, 0], want[:, 0], rtol=1e-4, atol=1e-5)
+    for net in ("GCN", "GIN"):
+        outs = []
+        for which in ("csr", "window"):
+            op = plain if which == "csr" else win
+            torch.manual_seed(3)
+            model = GNN.build_model(net, g, {16: op, 32: op}, 16, 32, 16)
+            ms = GNN.train_profiling(model, g.y, 3)
+            assert ms > 0
+            model.eval()
+            outs.append(model().detach())
+        torch.testing.assert_close(outs[0], outs[1], rtol=2e-3, atol=2e-3)
