@@ -97,7 +97,7 @@ def measured_sddmm_traffic(graph, K, fmt, bw):
     return None
 
 
-def other_graph_leg(name, dims, decider, reps=10):
+def other_graph_leg(name, dims, decider, reps=10, reorder=None):
     """One more graph of the benchmark set at a few widths, in the decider's configuration: per width the mean
     launch duration (HIP events on the launching stream), algorithmic bytes and their fraction of the HBM roofline,
     and the measured traffic of the committed counter summary for that graph when it has the configuration."""
@@ -109,7 +109,7 @@ def other_graph_leg(name, dims, decider, reps=10):
     rowPtr, colIdx, val, n = synth.config_graph(name)
     graph = graph_input(mtx_name=name, path="")
     graph.verbose = False
-    graph.load_from_csr(rowPtr, colIdx, val)
+    graph.load_from_csr(rowPtr, colIdx, val, reorder=reorder)  # reorder: rows and columns permuted together at load time
     nnz = graph.mtx_edges
     ops = sweep.operators_of(graph)
     fmt_names = ["csr", "csr_split", "bcsr", "bcsr_split"]
@@ -137,7 +137,7 @@ def other_graph_leg(name, dims, decider, reps=10):
         row = {"dim": d, "format": fmt, "CF": cf, "config": sweep.cf_label(cf), "blkWarpNum": bw, "ms": round(float(ms), 5),
                "gflops": round(2.0 * nnz * d / ms / 1e6, 1), "alg_bytes": int(b_alg),
                "frac": round(b_alg / ms / 1e6 / HBM_PEAK_GBS, 4)}
-        row["traffic"] = measured_traffic(name, [row])
+        row["traffic"] = measured_traffic(name, [row]) if reorder is None else None
         if win is not None and d % 4 == 0:
             # the windowed layout beside it (what GNN.configure_operators would keep if it is faster): its algorithmic
             # bytes are those of the CSR product plus the second row pointer per row
@@ -967,6 +967,8 @@ def main():
                 "C3s 5-point stencil 2048^2": other_graph_leg("C3s", [64, 128], decider),
                 "C5 block model 1M nodes, community order": other_graph_leg("C5", [16, 128], decider),
                 "C5p block model 1M nodes, random order": other_graph_leg("C5p", [128], decider),
+                "C5p after the community reordering pass at load time (label propagation)":
+                    other_graph_leg("C5p", [128], decider, reorder="community"),
                 "C3 Chung-Lu 2.45M nodes": other_graph_leg("C3", [128], decider, reps=5),
             }
         # ---- GCN training epochs on the 1M-node block model (the metric's second half) ------------------------------
