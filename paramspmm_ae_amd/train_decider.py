@@ -9,6 +9,8 @@ SuiteSparse / OGB collection the reference downloads.
                 every <representation, CF, blkWarpNum> at every width 16..256 -> csv files with the reference's
                 schema: mtx_info.csv, dim<N>.csv (GFLOP/s per column), dim<N>_OP_SpMM.csv (features + arg-max
                 column = class code).
+  window (GPU)  the windowed layout (an addition of this build) timed over the same corpus -> window.csv; ``fit`` reports
+                from it where that layout beats the best swept column.
   fit    (CPU)  one RandomForestClassifier per width -> rnd_tree_<N>.pkl, and a 5-fold cross-validated report with
                 the reference's two statistics (accuracy, mean normalised performance) plus the share of
                 matrices whose pick is within 10 % of the best swept configuration.
@@ -200,6 +202,96 @@ def sweep_main(args):
                     os.path.join(args.out, "dim%d%s.csv" % (d, tag)), index=False)
 
 
+def window_main(args):
+    """The windowed layout over the same corpus (GPU): per matrix its local share and, per width, the GFLOP/s of
+    the windowed SpMM and of plain CSR with CF 1 / blkWarpNum 4 timed in the same run (the column vec1_TP_14 of the
+    sweep tables, so that the two runs can be set side by side) -> window<tag>.csv.  The forests' class space is the
+    reference's and has no windowed class; ``fit`` reports from this table where the layout beats the best swept
+    column, which is what GNN.configure_operators decides by timing on the matrix itself."""
+    import pandas as pd
+    import torch
+
+    from . import synth
+    from .graph_input import graph_input
+    from .PCSR import pcsr_spmm
+
+    assert torch.cuda.is_available(), "the sweep needs the GPU"
+    items = corpus()
+    part, nparts = (int(x) for x in args.part.split("/"))
+    items = [it for i, it in enumerate(items) if i % nparts == part]
+    if args.limit:
+        items = items[: args.limit]
+    os.makedirs(args.out, exist_ok=True)
+    tag = "" if nparts == 1 else "_part%d" % part
+    dims = [int(d) for d in args.dims.split(",")] if args.dims else DIMS
+    flush_bytes = int(args.flush_mb) << 20
+    rows_out, t_start = [], time.time()
+    for idx, (name, build) in enumerate(items):
+        r, c, n = build()
+        rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+        g = graph_input(name, "")
+        g.verbose = False
+        g.load_from_csr(rowPtr, colIdx, val)
+        nnz = g.mtx_edges
+        win = pcsr_spmm(g, vec_size=1, if_split=False, CF=0, window=True)
+        csr = pcsr_spmm(g, vec_size=1, if_split=False, CF=1, blkWarpNum=4)
+        row = {"mtx_name": name, "local_share": win.window_local_share}
+        X32 = torch.randn(n, 32, device="cuda")
+        err = (win._spmm(X32) - csr._spmm(X32)).abs().max().item()
+        assert err <= 1e-4 * (csr._spmm(X32).abs().max().item() + 1e-6), (name, err)
+        for d in dims:
+            X = torch.ones(n, d, device="cuda")
+            fb = flush_bytes if d <= 128 else 0  # as the sweep behind the forests was timed
+            row["window_TP_%d" % d] = 2.0 * nnz * d / 1e6 / win.time_ms(X, warmup=args.warmup, iters=args.iters, flush_bytes=fb)
+            row["vec1_TP_14_%d" % d] = 2.0 * nnz * d / 1e6 / csr.time_ms(X, warmup=args.warmup, iters=args.iters, flush_bytes=fb)
+        rows_out.append(row)
+        del win, csr, g
+        torch.cuda.empty_cache()
+        print("[%d/%d] %-34s n=%-8d nnz=%-9d local %.3f (total %.0fs)" % (idx + 1, len(items), name, n, nnz, row["local_share"],
+                                                                       time.time() - t_start), flush=True)
+        if (idx + 1) % 10 == 0 or idx + 1 == len(items):
+            pd.DataFrame(rows_out).to_csv(os.path.join(args.out, "window%s.csv" % tag), index=False)
+
+
+def window_report(data_dir, info, tps, dims):
+    """What the windowed layout is worth against the best swept column, from window*.csv beside the sweep tables (None
+    without them).  The two tables come from different runs: the windowed figure is scaled by the ratio of the
+    plain-CSR column both runs timed."""
+    import glob
+
+    import pandas as pd
+
+    files = sorted(glob.glob(os.path.join(data_dir, "window*.csv")))
+    if not files:
+        return None
+    win = pd.concat([pd.read_csv(f) for f in files], ignore_index=True).drop_duplicates("mtx_name").set_index("mtx_name")
+    names = [n for n in info["mtx_name"] if n in win.index]
+    sel = np.array([n in win.index for n in info["mtx_name"]])
+    share = win.loc[names, "local_share"].to_numpy()
+    from .GNN import WINDOW_MIN_LOCAL_SHARE as thr
+
+    out = {"matrices": int(len(names)), "rule": "tried when the local share is at least %.2f, kept when faster (GNN.configure_operators)" % thr,
+           "matrices_with_that_local_share": int(np.sum(share >= thr)), "per_dim": {}}
+    fams = np.array([family(n).split("_")[0] + ("_ordered" if n.startswith("sbm_") and n.split("_r")[0].endswith("_s") else
+                                                 "_permuted" if n.startswith("sbm_") else "") for n in names])
+    for d in dims:
+        TP = tps[d].to_numpy(dtype=np.float64)[sel]
+        cols = list(tps[d].columns)
+        same = TP[:, cols.index("vec1_TP_14")] / win.loc[names, "vec1_TP_14_%d" % d].to_numpy()  # run-to-run scale
+        w = win.loc[names, "window_TP_%d" % d].to_numpy() * same
+        gain = w / TP.max(axis=1)
+        wins = gain > 1.0
+        ent = {"share_of_matrices_where_windowed_beats_the_best_swept_column": float(wins.mean()),
+               "mean_gain_where_it_wins": float(gain[wins].mean()) if wins.any() else None,
+               "best_gain": float(gain.max()),
+               "of_those_share_the_rule_tries": float(np.mean(share[wins] >= thr)) if wins.any() else None,
+               "share_of_tried_matrices_where_it_wins": float(np.mean(wins[share >= thr])) if (share >= thr).any() else None,
+               "mean_gain_over_tried_matrices": float(gain[share >= thr].mean()) if (share >= thr).any() else None,
+               "mean_gain_by_family": {f: float(gain[fams == f].mean()) for f in sorted(set(fams))}}
+        out["per_dim"][str(d)] = ent
+    return out
+
+
 # ------------------------------------------------------------------------------------------------------------
 # fit (CPU)
 # ------------------------------------------------------------------------------------------------------------
@@ -379,6 +471,9 @@ def fit_main(args):
     report["share_within_10pct_mean"] = float(np.mean(allw))
     report["share_within_10pct_min"] = float(np.min(allw))
     report["per_dim"] = {str(k): report["per_dim"][k] for k in sorted(report["per_dim"], key=int)}
+    wr = window_report(args.data, info, tps, [int(k) for k in report["per_dim"] if int(k) in tps])
+    if wr is not None:
+        report["windowed_layout"] = wr
     import sklearn
 
     report["scikit_learn"] = sklearn.__version__  # a pickled forest loads under the version that wrote it (or newer)
@@ -408,12 +503,22 @@ def main(argv=None):
                         "decider.py) or every swept column")
     f.add_argument("--out", default="", help="default: models/ for --space reference, models/native/ for --space native")
     f.add_argument("--dims", default="", help="refit these widths only (comma-separated); the report keeps the others")
+    w = sub.add_parser("window")
+    w.add_argument("--out", default=os.path.join(here, "models", "train_data"))
+    w.add_argument("--part", default="0/1", help="i/n: every n-th matrix starting at i")
+    w.add_argument("--limit", type=int, default=0)
+    w.add_argument("--warmup", type=int, default=2)
+    w.add_argument("--iters", type=int, default=6)
+    w.add_argument("--dims", default="")
+    w.add_argument("--flush_mb", type=int, default=512)
     ls = sub.add_parser("list")
     args = ap.parse_args(argv)
     if args.cmd == "sweep":
         sweep_main(args)
     elif args.cmd == "fit":
         fit_main(args)
+    elif args.cmd == "window":
+        window_main(args)
     else:
         for name, _ in corpus():
             print(name)
