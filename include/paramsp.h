@@ -322,6 +322,14 @@ int psp_window_build_dev(const int *rowPtr, const int *colIdx, const float *val,
 int psp_spmm_window_plan(int N, int variant, int *tile_cols, int *rows_per_block, int *lds_bytes);
 int psp_spmm_window_f32(const int *rowPtr_w, const int *colIdx_w, const float *val_w, const float *X, float *Y, int M,
                         int nnz, int N, int rows_out, int variant, int relu_x, const float *mask, psp_stream_t stream);
+/* The same product with a small dense one folded into its epilogue (the dense product of a square GCN layer,
+ * SpCONV/SpCONV.h:43-71: torch::mm(H, W) around the sparse product): Y = mask (.) ((A f(X)) W) for transW == 0 or
+ * ((A f(X)) W^T) for transW != 0, with W[N, N] row-major, N = 16 or 32, f = max(., 0) when relu_x.  Y_raw (may be null)
+ * receives A f(X) itself.  Since A (H W) = (A H) W the forward pass of a layer is one launch, and its backward pass one
+ * launch that delivers A dY (for the weight gradient) and (A dY) W^T masked (the input gradient). */
+int psp_spmm_window_xw_f32(const int *rowPtr_w, const int *colIdx_w, const float *val_w, const float *X, const float *W,
+                           int transW, float *Y, float *Y_raw, int M, int nnz, int N, int rows_out, int relu_x,
+                           const float *mask, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: softmax over the stored entries of every CSR row (out[p] = exp(e[p]-max_r) / sum_r).

@@ -26,6 +26,11 @@
 // entries finish in plain loops (correct for any matrix, slow for matrices the format is not meant for).  Per
 // element the sum runs over the local entries in storage order, then the remote ones: within the stated fp32
 // tolerance of the reference's chain, not bit-identical to it.
+// EPI (square layers of 16 or 32 columns, one column tile): the finished row is multiplied by a small dense matrix
+// before it is stored, Y = (A f(X)) W or (A f(X)) W^T -- the dense product of a GCN layer folded into the sparse one.
+// W sits in LDS (transposed on the way in for W^T); a lane group gathers its row of A f(X) with DPP moves and each lane
+// forms its four output columns (N multiply-adds per column).  The row of A f(X) itself can be stored as well (Y_raw:
+// the backward pass needs A dY for the weight gradient and (A dY) W^T for the input gradient).
 // relu_x applies max(x, 0) to X as it enters (once per window element rather than once per gather); mask keeps an
 // output element only where mask > 0, read where the row is stored -- the two halves of a ReLU folded into the
 // product, as psp_spmm_act_f32 offers for the other formats.
@@ -66,13 +71,31 @@ template <int L> __device__ __forceinline__ int pspw_bcast_u(int x, int u, int s
     }
 }
 
-template <int C, int LOGL, int PSPW_THREADS>
+// the same for any lane of the group
+template <int L> __device__ __forceinline__ float pspw_bcast_any_f(float x, int j, int sub)
+{
+    const int v = __float_as_int(x);
+    switch (j) {
+    case 0: return __int_as_float(pspw_bcast<L, 0>(v, sub));
+    case 1: return __int_as_float(pspw_bcast<L, 1>(v, sub));
+    case 2: return __int_as_float(pspw_bcast<L, 2>(v, sub));
+    case 3: return __int_as_float(pspw_bcast<L, 3>(v, sub));
+    case 4: return __int_as_float(pspw_bcast<L, 4>(v, sub));
+    case 5: return __int_as_float(pspw_bcast<L, 5>(v, sub));
+    case 6: return __int_as_float(pspw_bcast<L, 6>(v, sub));
+    default: return __int_as_float(pspw_bcast<L, 7>(v, sub));
+    }
+}
+
+template <int C, int LOGL, int PSPW_THREADS, bool EPI = false>
 __global__ void __launch_bounds__(PSPW_THREADS)
 psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__ colIdx, const float *__restrict__ val,
                        const float *__restrict__ X, float *__restrict__ Y, const float *__restrict__ mask, int M, int N,
-                       int nnz, int nruns, int stripe, int run, int relu_x)
+                       int nnz, int nruns, int stripe, int run, int relu_x, const float *__restrict__ W, int transW,
+                       float *__restrict__ Y_raw)
 {
     constexpr int L = 1 << LOGL;
+    static_assert(!EPI || C == 1, "the dense epilogue exists for one vector per lane (one column tile of 16 or 32)");
     constexpr int TN = L * C * 4;                  // columns per tile
     constexpr int RB = PSPW_BLOCK;                 // rows per step
     constexpr int RPG = RB * L / PSPW_THREADS;     // rows per lane group
@@ -98,6 +121,13 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
     const int tile_col0 = blockIdx.y * TN;
     const int2 *rp2 = (const int2 *)rowPtr_w;
     if (tid < V4) *(psp_f32x4 *)(s_x + RING * TN + tid * 4) = (psp_f32x4){0.f, 0.f, 0.f, 0.f};
+    float *s_w = s_x + (RING + 1) * TN;  // EPI: [TN][TN], s_w[k][j] = factor of input column k in output column j
+    if constexpr (EPI) {
+        for (int idx = tid; idx < TN * TN; idx += PSPW_THREADS) {
+            const int k_ = idx / TN, j_ = idx - k_ * TN;
+            s_w[idx] = transW ? W[j_ * TN + k_] : W[idx];
+        }
+    }
 
     bool live[C];
     int off[C];
@@ -302,6 +332,25 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
                 }
             }
             const int r = j * RB + grp * RPG + k;
+            if constexpr (EPI) {
+                // the row of A f(X) is complete: store it if asked, then multiply it by the staged matrix (every lane
+                // of the wavefront takes part in the DPP moves; N == TN here, so every lane has columns)
+                const psp_f32x4 raw = acc[k][0];
+                if (Y_raw != nullptr && r < M)
+                    __builtin_nontemporal_store(raw, (psp_f32x4 *)(Y_raw + (size_t)r * (size_t)N + off[0]));
+                psp_f32x4 o = (psp_f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int j2 = 0; j2 < L; j2++) {
+#pragma unroll
+                    for (int e2 = 0; e2 < 4; e2++) {
+                        const float a_ = pspw_bcast_any_f<L>(raw[e2], j2, sub);
+                        const psp_f32x4 wv = *(const psp_f32x4 *)(s_w + ((j2 * 4 + e2) * TN + off[0]));
+#pragma unroll
+                        for (int e = 0; e < 4; e++) o[e] = __builtin_fmaf(a_, wv[e], o[e]);
+                    }
+                }
+                acc[k][0] = o;
+            }
             if (r < M) {
 #pragma unroll
                 for (int i = 0; i < C; i++) {
@@ -412,7 +461,7 @@ PSP_EXPORT int psp_window_build_dev(const int *rowPtr, const int *colIdx, const 
 
 // ---- launch -----------------------------------------------------------------------------------------------------------
 typedef void (*pspw_kernel_t)(const int *, const int *, const float *, const float *, float *, const float *, int, int,
-                              int, int, int, int, int);
+                              int, int, int, int, int, const float *, int, float *);
 
 struct pspw_variant {
     pspw_kernel_t fn;
@@ -420,8 +469,15 @@ struct pspw_variant {
 };
 
 // one row of a block per lane group: 64 groups of 4 lanes, or 64 groups of 8 lanes in a workgroup of 512
-static pspw_variant pspw_lookup(int variant)
+static pspw_variant pspw_lookup(int variant, bool epilogue = false)
 {
+    if (epilogue) {
+        switch (variant) {
+        case 1: return {psp_spmm_window_kernel<1, 2, 256, true>, 16, 256};
+        case 2: return {psp_spmm_window_kernel<1, 3, 512, true>, 32, 512};
+        default: return {nullptr, 0, 0};
+        }
+    }
     switch (variant) {
     case 1: return {psp_spmm_window_kernel<1, 2, 256>, 16, 256};  // 4 lanes x 1 vector
     case 2: return {psp_spmm_window_kernel<1, 3, 512>, 32, 512};  // 8 lanes x 1 vector
@@ -450,55 +506,82 @@ PSP_EXPORT int psp_spmm_window_plan(int N, int variant, int *tile_cols, int *row
 // is sized from the occupancy the runtime reports for the kernel: at most that many workgroups (a multiple of the
 // 8 XCDs per column tile, so that the grid holds no empty ones), each with an equal share of the blocks.
 // PSP_WINDOW_RUN overrides the choice.
-static int pspw_run_length(int nblocks, int tiles, int variant, const pspw_variant &k, int lds)
+static int pspw_run_length(int nblocks, int tiles, int slot_key, const pspw_variant &k, int lds)
 {
     static const int forced = [] {
         const char *e = getenv("PSP_WINDOW_RUN");
         return e ? atoi(e) : 0;
     }();
     if (forced > 0) return forced;
-    static int slots_of[4];  // workgroups the current GPU holds at once, per variant (0 = not asked yet)
-    if (slots_of[variant] == 0) {
+    static int slots_of[8];  // workgroups the current GPU holds at once, per kernel (0 = not asked yet)
+    if (slots_of[slot_key] == 0) {
         int dev = 0, cus = 0, per_cu = 0;
         if (hipGetDevice(&dev) != hipSuccess ||
             hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
             cus = 256;
         if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)k.fn, k.threads, (size_t)lds) != hipSuccess || per_cu <= 0)
             per_cu = 1;
-        slots_of[variant] = cus * per_cu;
+        slots_of[slot_key] = cus * per_cu;
     }
-    int nruns = slots_of[variant] / tiles / PSP_XCDS * PSP_XCDS;
+    int nruns = slots_of[slot_key] / tiles / PSP_XCDS * PSP_XCDS;
     if (nruns < PSP_XCDS) nruns = PSP_XCDS;
     const int run = (nblocks + nruns - 1) / nruns;
     return run < 1 ? 1 : run;
+}
+
+static int pspw_launch(const int *rowPtr_w, const int *colIdx_w, const float *val_w, const float *X, float *Y, int M, int nnz,
+                       int N, int rows_out, int variant, int relu_x, const float *mask, const float *W, int transW,
+                       float *Y_raw, hipStream_t st)
+{
+    const bool epi = W != nullptr;
+    int tn = 0, rb = 0, lds = 0;
+    const int v = psp_spmm_window_plan(N, variant, &tn, &rb, &lds);
+    if (v < 0) return v;
+    PSP_REQUIRE(M >= 0 && nnz >= 0 && rows_out >= M, "spmm_window: Y has %d rows, the matrix %d (%d entries)", rows_out, M, nnz);
+    PSP_REQUIRE((((size_t)X | (size_t)Y | (size_t)mask | (size_t)Y_raw) & 15) == 0, "spmm_window: X, Y and mask must be 16-byte aligned");
+    if (epi) {
+        PSP_REQUIRE(N == tn && (N == 16 || N == 32), "spmm_window: the dense epilogue exists for N = 16 and 32 (got %d)", N);
+        lds += tn * tn * 4;
+    }
+    if (nnz == 0) {  // (the kernel clamps its loads to entry nnz - 1)
+        const int rc = psp_zero_f32(Y, (size_t)rows_out * N, st);
+        return rc != PSP_OK || !Y_raw ? rc : psp_zero_f32(Y_raw, (size_t)rows_out * N, st);
+    }
+    int rc = psp_zero_f32(Y + (size_t)M * N, ((size_t)rows_out - (size_t)M) * N, st);  // rows past the matrix
+    if (rc == PSP_OK && Y_raw) rc = psp_zero_f32(Y_raw + (size_t)M * N, ((size_t)rows_out - (size_t)M) * N, st);
+    if (rc != PSP_OK || M == 0) return rc;
+    PSP_REQUIRE(rowPtr_w && colIdx_w && val_w && X && Y, "spmm_window: null pointer");
+    const pspw_variant k = pspw_lookup(v, epi);
+    const int key = v + (epi ? 4 : 0);
+    static bool lds_raised[8];
+    if (lds > 48 * 1024 && !lds_raised[key]) {
+        const hipError_t e = hipFuncSetAttribute((const void *)k.fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return psp_fail(PSP_ERR_LAUNCH, "spmm_window: %d bytes of LDS refused: %s", lds, hipGetErrorString(e));
+        lds_raised[key] = true;
+    }
+    const int nblocks = psp_ceil_div(M, rb), tiles = psp_ceil_div(N, tn);
+    const int run = pspw_run_length(nblocks, tiles, key, k, lds);
+    const int nruns = psp_ceil_div(nblocks, run);
+    const psp_grid1d g = psp_xcd_grid(nruns, 1);  // long runs: neighbouring runs share two halo windows, nothing to keep in one L2
+    dim3 grid(g.launch, tiles, 1), block(k.threads, 1, 1);
+    hipLaunchKernelGGL(k.fn, grid, block, lds, st, rowPtr_w, colIdx_w, val_w, X, Y, mask, M, N, nnz, nruns, g.stripe, run,
+                       relu_x != 0, W, transW != 0, Y_raw);
+    return psp_check_launch("spmm window kernel");
 }
 
 PSP_EXPORT int psp_spmm_window_f32(const int *rowPtr_w, const int *colIdx_w, const float *val_w, const float *X, float *Y,
                                    int M, int nnz, int N, int rows_out, int variant, int relu_x, const float *mask,
                                    psp_stream_t stream)
 {
-    int tn = 0, rb = 0, lds = 0;
-    const int v = psp_spmm_window_plan(N, variant, &tn, &rb, &lds);
-    if (v < 0) return v;
-    PSP_REQUIRE(M >= 0 && nnz >= 0 && rows_out >= M, "spmm_window: Y has %d rows, the matrix %d (%d entries)", rows_out, M, nnz);
-    PSP_REQUIRE((((size_t)X | (size_t)Y | (size_t)mask) & 15) == 0, "spmm_window: X, Y and mask must be 16-byte aligned");
-    hipStream_t st = (hipStream_t)stream;
-    if (nnz == 0) return psp_zero_f32(Y, (size_t)rows_out * N, st);  // (the kernel clamps its loads to entry nnz - 1)
-    int rc = psp_zero_f32(Y + (size_t)M * N, ((size_t)rows_out - (size_t)M) * N, st);  // rows past the matrix
-    if (rc != PSP_OK || M == 0) return rc;
-    PSP_REQUIRE(rowPtr_w && colIdx_w && val_w && X && Y, "spmm_window: null pointer");
-    const pspw_variant k = pspw_lookup(v);
-    static bool lds_raised[4];
-    if (lds > 48 * 1024 && !lds_raised[v]) {
-        const hipError_t e = hipFuncSetAttribute((const void *)k.fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return psp_fail(PSP_ERR_LAUNCH, "spmm_window: %d bytes of LDS refused: %s", lds, hipGetErrorString(e));
-        lds_raised[v] = true;
-    }
-    const int nblocks = psp_ceil_div(M, rb), tiles = psp_ceil_div(N, tn);
-    const int run = pspw_run_length(nblocks, tiles, v, k, lds);
-    const int nruns = psp_ceil_div(nblocks, run);
-    const psp_grid1d g = psp_xcd_grid(nruns, 1);  // long runs: neighbouring runs share two halo windows, nothing to keep in one L2
-    dim3 grid(g.launch, tiles, 1), block(k.threads, 1, 1);
-    hipLaunchKernelGGL(k.fn, grid, block, lds, st, rowPtr_w, colIdx_w, val_w, X, Y, mask, M, N, nnz, nruns, g.stripe, run, relu_x != 0);
-    return psp_check_launch("spmm window kernel");
+    return pspw_launch(rowPtr_w, colIdx_w, val_w, X, Y, M, nnz, N, rows_out, variant, relu_x, mask, nullptr, 0, nullptr,
+                       (hipStream_t)stream);
+}
+
+PSP_EXPORT int psp_spmm_window_xw_f32(const int *rowPtr_w, const int *colIdx_w, const float *val_w, const float *X,
+                                      const float *W, int transW, float *Y, float *Y_raw, int M, int nnz, int N, int rows_out,
+                                      int relu_x, const float *mask, psp_stream_t stream)
+{
+    PSP_REQUIRE(W != nullptr, "spmm_window_xw: W is null");
+    return pspw_launch(rowPtr_w, colIdx_w, val_w, X, Y, M, nnz, N, rows_out, 0, relu_x, mask, W, transW, Y_raw,
+                       (hipStream_t)stream);
 }

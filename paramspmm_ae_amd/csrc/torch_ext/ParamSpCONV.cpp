@@ -186,6 +186,38 @@ static Tensor aggregate_act_op(int fmt, Tensor D, Tensor rowPtr, Tensor colIdx, 
     return Y;
 }
 
+// Windowed layout, square layer of 16 or 32 columns: the dense product folded into the sparse one
+// (psp_spmm_window_xw_f32).  Returns [Y] or [Y, A f(X)]:  Y = ((A f(X)) W | W^T), kept where mask > 0 when a mask is given.
+static bool window_xw_supported(long N) { return N == 16 || N == 32; }
+static std::vector<Tensor> window_xw(Tensor X, Tensor W, bool transW, Tensor rowPtr_w, Tensor colIdx_w, Tensor values_w,
+                                     bool relu_input, c10::optional<Tensor> mask, bool want_raw)
+{
+    need_gpu(X, "input");
+    need_gpu(W, "weight");
+    Tensor Xc = X.contiguous(), Wc = W.contiguous();
+    check_spmm_args(4, Xc, rowPtr_w, colIdx_w, values_w, nullptr);
+    need_f32(Wc, "weight", 2);
+    const long N = Xc.size(1);
+    TORCH_CHECK(window_xw_supported(N) && Wc.size(0) == N && Wc.size(1) == N,
+                "window_xw: a square weight matrix of 16 or 32 columns, as wide as the input");
+    pspglue::same_device(Xc, Wc, "window_xw");
+    Tensor Mc;
+    if (mask) {
+        need_gpu(*mask, "mask");
+        TORCH_CHECK(mask->scalar_type() == torch::kFloat32 && mask->dim() == 2 && mask->size(0) == Xc.size(0) && mask->size(1) == N,
+                    "mask must be float32 with the shape of the result");
+        Mc = mask->contiguous();
+    }
+    DeviceGuard guard(Xc.device());
+    Tensor Y = torch::empty_like(Xc), R;
+    if (want_raw) R = torch::empty_like(Xc);
+    ok(psp_spmm_window_xw_f32(ip(rowPtr_w), ip(colIdx_w), fp(values_w), fp(Xc), fp(Wc), transW ? 1 : 0, fpw(Y),
+                              want_raw ? fpw(R) : nullptr, pspglue::fmt_rows(4, rowPtr_w), (int)colIdx_w.size(0), (int)N,
+                              (int)Xc.size(0), relu_input ? 1 : 0, mask ? fp(Mc) : nullptr, stream_of(Xc)));
+    if (want_raw) return {Y, R};
+    return {Y};
+}
+
 static Tensor forward_impl(int fmt, const Tensor &H, const Tensor &W, const Tensor &rowPtr, const Tensor &colIdx,
                            const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
 {
@@ -306,6 +338,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     }, "max(Z, 0)^T * G: (Z, G)");
     m.def("nll_loss_mean", &nll_loss_mean, "[loss, stats] of the mean negative log-likelihood (log-probabilities, int64 labels)");
     m.def("nll_loss_mean_backward", &nll_loss_mean_backward, "gradient w.r.t. the log-probabilities: (labels, grad_loss, stats, n, C)");
+    m.def("window_xw", &window_xw,
+          "windowed layout, dense product folded in: (X, W, transW, rowPtr_w, colIdx_w, values_w, relu_input, mask | None, want_raw) -> [Y] or [Y, A f(X)]");
+    m.def("window_xw_supported", &window_xw_supported, "widths the folded product exists for");
     m.def("aggregate", &aggregate_op, "A*D: (fmt, D, rowPtr, colIdx, values, target_row | None, CF, blkWarpNum)");
     m.def("aggregate_act", &aggregate_act_op,
           "A*max(D,0) (relu_input) and / or (A*D) where mask > 0: (fmt, D, rowPtr, colIdx, values, target_row | None, CF, blkWarpNum, relu_input, mask | None)");

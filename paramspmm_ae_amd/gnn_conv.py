@@ -40,6 +40,13 @@ def _row_ptr(op):
     return getattr(op, "spmm_rowPtr", op.rowPtr)
 
 
+def _window_xw(op, Z, weight):
+    """Does the layer A (relu(Z) W) run as one windowed launch with the dense product folded in?  A windowed operator, a
+    square weight matrix of a width the kernel has, float32."""
+    return (_fmt(op) == 4 and weight.shape[0] == weight.shape[1] == Z.shape[1] and SpCONV.window_xw_supported(int(Z.shape[1]))
+            and Z.dtype == torch.float32 and getattr(op, "fold_dense", True))
+
+
 def _aggregate(op, D):
     """A D through ``op``'s format and configuration."""
     return SpCONV.aggregate(_fmt(op), D, _row_ptr(op), op.colIdx, op.val, op.target_row if op.if_split else None, op.CF,
@@ -133,6 +140,9 @@ class GCNReLUInputFunction(torch.autograd.Function):
         ctx.save_for_backward(Z, weight)
         ctx.ParamSpMM = ParamSpMM
         op = ParamSpMM
+        if _window_xw(op, Z, weight):
+            # windowed layout, square layer: (A relu(Z)) W in one launch, the dense product in the kernel's epilogue
+            return SpCONV.window_xw(Z, weight, False, op.spmm_rowPtr, op.colIdx, op.val, True, None, False)[0]
         return SpCONV.relu_input_forward(_fmt(op), Z, weight, _row_ptr(op), op.colIdx, op.val,
                                          op.target_row if op.if_split else None, op.CF, _bw(op))
 
@@ -140,6 +150,10 @@ class GCNReLUInputFunction(torch.autograd.Function):
     def backward(ctx, d_output):
         Z, weight = ctx.saved_tensors
         op = ctx.ParamSpMM
+        if _window_xw(op, Z, weight):
+            # one launch delivers A dY (for the weight gradient) and ((A dY) W^T) where Z > 0 (the input gradient)
+            d_input, AG = SpCONV.window_xw(d_output.contiguous(), weight, True, op.spmm_rowPtr, op.colIdx, op.val, False, Z, True)
+            return d_input, SpCONV.weight_gradient_relu(Z, AG), None
         d_input, d_weight = SpCONV.relu_input_backward(_fmt(op), d_output.contiguous(), Z, weight, _row_ptr(op), op.colIdx, op.val,
                                                        op.target_row if op.if_split else None, op.CF, _bw(op))
         return d_input, d_weight, None

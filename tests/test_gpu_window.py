@@ -209,7 +209,8 @@ def test_window_operator_through_the_modules_and_a_gcn_layer(oracle):
 
     Ad = torch.from_numpy(A.toarray().astype(np.float64)).cuda()
     for cls, relu_in in ((gnn_conv.GCNConv, False), (gnn_conv.GCNConv, True), (gnn_conv.GINConv, False), (gnn_conv.GINConv, True)):
-        for in_w, out_w in ((32, 16), (16, 32)):
+        # (square layers of 16 / 32 columns with relu_input run the GCN layer as one launch, dense product folded in)
+        for in_w, out_w in ((32, 16), (16, 32), (16, 16), (32, 32)):
             layer = cls(in_w, out_w).cuda()
             H = torch.randn(n, in_w, device="cuda", requires_grad=True)
             ops = {in_w: op, out_w: op}
@@ -264,3 +265,56 @@ def test_training_with_windowed_operators_follows_training_with_the_csr_operator
             model.eval()
             outs.append(model().detach())
         torch.testing.assert_close(outs[0], outs[1], rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("N", [16, 32])
+def test_window_spmm_with_the_dense_product_folded_in(oracle, N):
+    """psp_spmm_window_xw_f32: Y = ((A f(X)) W) or ((A f(X)) W^T), masked, with A f(X) delivered beside it: the raw
+    product equals the plain windowed product bit for bit (same kernel, same order), Y a float64 restatement to
+    1e-5 of the magnitudes involved, masked elements are exact zeros; widths other than 16 / 32 are argument errors."""
+    from gpu_util import dev
+    from paramspmm_ae_amd import _capi
+    import ParamSpMM
+
+    rowPtr, colIdx, val = banded_csr(4001, 10, 40, 20 + N, far=0.15, hub=(9, 500), empty_frac=0.05)
+    M = rowPtr.size - 1
+    rp, ci, v = ParamSpMM.window_build(dev(rowPtr), dev(colIdx), dev(val))
+    import scipy.sparse as sp
+
+    A = sp.csr_matrix((val.astype(np.float64), colIdx, rowPtr), shape=(M, M))
+    rng = np.random.default_rng(N)
+    X = rng.standard_normal((M, N)).astype(np.float32)
+    W = (rng.standard_normal((N, N)) / np.sqrt(N)).astype(np.float32)
+    mask = rng.standard_normal((M, N)).astype(np.float32)
+    Xd, Wd, Md = torch.from_numpy(X).cuda(), torch.from_numpy(W).cuda(), torch.from_numpy(mask).cuda()
+    p, L = _capi.ptr, _capi.lib
+    st = torch.cuda.current_stream().cuda_stream
+    for transW in (0, 1):
+        for relu in (0, 1):
+            for use_mask in (False, True):
+                print("case xw", N, transW, relu, use_mask, flush=True)
+                Y = torch.full((M, N), float("nan"), device="cuda")
+                R = torch.full((M, N), float("nan"), device="cuda")
+                _capi.check(L.psp_spmm_window_xw_f32(p(rp), p(ci), p(v), p(Xd), p(Wd), transW, p(Y), p(R), M, int(ci.numel()), N, M,
+                                                     relu, p(Md) if use_mask else None, st))
+                torch.cuda.synchronize()
+                fX = np.maximum(X, 0) if relu else X
+                plain = _spmm_window((rp, ci, v, M), torch.from_numpy(fX).cuda())
+                assert torch.equal(R, plain)
+                AX = A @ fX.astype(np.float64)
+                want = AX @ (W.T if transW else W).astype(np.float64)
+                scale = (abs(A) @ np.abs(fX).astype(np.float64)) @ np.abs(W.T if transW else W).astype(np.float64)
+                got = Y.cpu().numpy().astype(np.float64)
+                if use_mask:
+                    assert np.all(got[mask <= 0] == 0)
+                    want = np.where(mask > 0, want, 0.0)
+                assert np.all(np.abs(got - want) <= 1e-6 + 1e-5 * scale), float(np.abs(got - want).max())
+                # without the raw output
+                Y2 = torch.full((M, N), float("nan"), device="cuda")
+                _capi.check(L.psp_spmm_window_xw_f32(p(rp), p(ci), p(v), p(Xd), p(Wd), transW, p(Y2), None, M, int(ci.numel()), N, M,
+                                                     relu, p(Md) if use_mask else None, st))
+                assert torch.equal(Y2, Y)
+    X48 = torch.zeros(M, 48, device="cuda")
+    assert L.psp_spmm_window_xw_f32(p(rp), p(ci), p(v), p(X48), p(Wd), 0, p(X48), None, M, int(ci.numel()), 48, M, 0, None, st) == -1
+    assert L.psp_spmm_window_xw_f32(p(rp), p(ci), p(v), p(Xd), None, 0, p(Xd), None, M, int(ci.numel()), N, M, 0, None, st) == -1
