@@ -481,17 +481,18 @@ def bench_sddmm(args):
 def bench_gcn(args):
     """GCN, GIN and AGNN training epochs (BASELINE.json configs[4]): 5 layers, hidden 16 / 32 / 128, 16 classes, random
     features and weights, forward + backward + Adam, on the 1M-node stochastic block model in community order
-    (C5) and randomly permuted (C5p).  --steps is the number of timed epochs (the reference times 200)."""
+    (C5) and randomly permuted (C5p).  --epochs timed epochs after one warm-up epoch (default 200, the reference's
+    protocol, GNN.py:126-151)."""
     from paramspmm_ae_amd import GNN
 
     out = {"metric": "GCN / GIN / AGNN epoch ms (5 layers, fwd+bwd+Adam), SBM 1M nodes", "unit": "ms per epoch", "n_gpus": 1,
-           "steps": args.steps, "warmup": 1, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+           "steps": args.epochs, "warmup": 1, "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
            "dtype": "f32", "data": "synthetic", "config": {"workload": "C5 / C5p, hidden 16 32 128, 16 classes"}, "epochs": []}
     graphs = [args.graph] if args.graph in ("C5", "C5p", "C1") else ["C5", "C5p"]
     for g in graphs:
         for net in ("GCN", "GIN", "AGNN"):
             argv = ["--net", net, "--synthetic", g, "--hidden_list", "16", "32", "128", "--num_classes", "16",
-                    "--num_features", "32", "--num_epoches", str(args.steps)]
+                    "--num_features", "32", "--num_epoches", str(args.epochs)]
             res = GNN.main(argv)
             # the same epochs with the training step recorded once in a HIP graph and replayed
             res_graph = GNN.main(argv + ["--hip_graph"])
@@ -559,6 +560,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--epochs", type=int, default=200, help="--workload gcn: timed epochs per network and width")
     ap.add_argument("--graph", default="C2", help="C1, C2, C3, C3s, C5, C5p (synth.config_graph)")
     ap.add_argument("--dims", default=DEFAULT_DIMS)
     ap.add_argument("--pick", default="auto",
