@@ -331,6 +331,16 @@ int psp_spmm_window_xw_f32(const int *rowPtr_w, const int *colIdx_w, const float
                            int transW, float *Y, float *Y_raw, int M, int nnz, int N, int rows_out, int relu_x,
                            const float *mask, psp_stream_t stream);
 
+/* SDDMM over the same layout: out[p] = alpha <A[row(p), :], B[col(p), :]> for every stored entry, in the layout's entry
+ * order (out is parallel to colIdx_w).  The B rows of a block's window sit in LDS; only remote entries gather.
+ * A[>= M, K], B[rows_b, K] row-major and 16-byte aligned, rows_b above every column index, K a multiple of 4 up to
+ * PSP_SDDMM_WINDOW_MAX_K.  alpha: one float in device memory, or NULL for 1.  A == B (the attention scores of a graph
+ * layer) reads the matrix once.  No counterpart in the reference (its kernels, SDDMM/sddmm_kernel.cu:917-1057, gather
+ * B[col] per entry); results agree with psp_sddmm_csr_f32 on (rowPtr_w[0::2], colIdx_w) within the fp32 tolerance. */
+#define PSP_SDDMM_WINDOW_MAX_K 128
+int psp_sddmm_window_f32(const int *rowPtr_w, const int *colIdx_w, const float *A, const float *B, const float *alpha,
+                         float *out, int M, int nnz, int K, int rows_b, psp_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: softmax over the stored entries of every CSR row (out[p] = exp(e[p]-max_r) / sum_r).
  * No counterpart in the reference (its AGNN layer applies no softmax, gnn_conv.py:136-142); it exists for

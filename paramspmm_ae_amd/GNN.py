@@ -322,10 +322,8 @@ def main(argv=None):
                 dims.append(args.num_features)  # the first layer runs its sparse product at the features' width
             if args.net == "GIN" and args.num_features not in dims and (decider is None or args.num_features in decider.model_dict):
                 dims.append(args.num_features)  # GIN aggregates its input: the first layer's product has the features' width
-            # (the attention network orders its per-entry vectors by the graph's own colIdx: it keeps the PCSR formats)
             ops = configure_operators(decider, graph, dims, None if args.config is None else tuple(args.config),
-                                      try_candidates=args.try_candidates,
-                                      try_window=not args.no_window and args.net != "AGNN")
+                                      try_candidates=args.try_candidates, try_window=not args.no_window)
             print("SpMM-decider config time: {:.3f} (ms)".format((time.perf_counter() - t1) * 1e3))
             model = build_model(args.net, graph, ops, hidden, args.num_features, args.num_classes, args.num_layers)
             if args.no_fuse_relu and hasattr(model, "fuse_relu"):

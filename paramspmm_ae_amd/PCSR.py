@@ -271,7 +271,12 @@ class pcsr_spmm(object):
         return self._spmm(X)
 
     # ---- SDDMM ------------------------------------------------------------------------------
-    def _sddmm(self, A, B, blkWarpNum):
+    def _sddmm(self, A, B, blkWarpNum, alpha=None):
+        if self.window and A.dtype == torch.float32 and SDDMM.window_sddmm_supported(int(A.size(1))):
+            # B rows of a block's window from LDS (results parallel to the layout's own colIdx)
+            return SDDMM.window_sddmm(A, B, self.rowPtr_w, self.colIdx, alpha)
+        if alpha is not None:
+            return self._sddmm(A, B, blkWarpNum) * alpha.reshape(())
         if self.vec_size == 3:  # the generic-block operators (PCSR.py:300-345)
             fn = SDDMM.vec_split_sddmm if self.if_split else SDDMM.vec_sddmm
         else:
@@ -281,11 +286,13 @@ class pcsr_spmm(object):
             blkWarpNum |= 0x100  # PSP_BW_BALANCED: divide the entries, not the rows, between the wavefronts
         return fn(A, B, *self._sparse_args(), CF, blkWarpNum | self.bw_flags)
 
-    def AGNN_sddmm(self, A):
-        """Per stored entry <A[row], A[col]>; for 2x1 blocks the result is [nblk, 2] (PCSR.py:290-320)."""
+    def AGNN_sddmm(self, A, alpha=None):
+        """Per stored entry <A[row], A[col]>; for 2x1 blocks the result is [nblk, 2] (PCSR.py:290-320).  ``alpha`` (an
+        addition of this build): a one-element tensor the results are multiplied by -- inside the kernel on a windowed
+        operator."""
         if self.vec_size != 1 and self.mask is None:
             raise ValueError("mask should be given when vec_size=2")
-        return self._sddmm(A, A, self.blkWarpNum)
+        return self._sddmm(A, A, self.blkWarpNum, alpha)
 
     def get_sddmm_result(self, dim, blkWarpNum):
         assert torch.cuda.is_available()

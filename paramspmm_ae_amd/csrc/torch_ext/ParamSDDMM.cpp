@@ -98,6 +98,40 @@ static Tensor bcsr_split_sddmm(Tensor A, Tensor B, Tensor rowPtr_bcsr_split, Ten
     return sddmm_new(3, A, B, rowPtr_bcsr_split, colIdx, values, &target_row, nullptr, CF, blkWarpNum);
 }
 
+// SDDMM over the windowed layout (ParamSpMM.window_build): out[p] = alpha <A[row], B[col]> in the layout's entry order.
+// alpha: a one-element float32 tensor on the device, or None.  Passing the same tensor for A and B reads it once.
+static bool window_sddmm_supported(long K) { return K >= 4 && K % 4 == 0 && K <= PSP_SDDMM_WINDOW_MAX_K; }
+static Tensor window_sddmm(Tensor A, Tensor B, Tensor rowPtr_w, Tensor colIdx_w, c10::optional<Tensor> alpha)
+{
+    need_gpu(A, "A");
+    need_gpu(B, "B");
+    need_gpu(rowPtr_w, "rowPtr_w");
+    need_gpu(colIdx_w, "colIdx_w");
+    need_f32(A, "A", 2);
+    need_f32(B, "B", 2);
+    need_i32(rowPtr_w, "rowPtr_w");
+    need_i32(colIdx_w, "colIdx_w");
+    same_device(A, B, "window_sddmm");
+    same_device(A, rowPtr_w, "window_sddmm");
+    same_device(A, colIdx_w, "window_sddmm");
+    TORCH_CHECK(rowPtr_w.size(0) >= 2 && rowPtr_w.size(0) % 2 == 0, "rowPtr of the windowed format has 2 M + 2 entries");
+    TORCH_CHECK(A.size(1) == B.size(1) && window_sddmm_supported(A.size(1)),
+                "window_sddmm: A and B need the same number of columns, a multiple of 4 up to ", PSP_SDDMM_WINDOW_MAX_K);
+    const long M = (rowPtr_w.size(0) - 2) / 2;
+    TORCH_CHECK(M <= A.size(0), "rowPtr_w describes more rows than A has");
+    if (alpha) {
+        need_gpu(*alpha, "alpha");
+        TORCH_CHECK(alpha->scalar_type() == torch::kFloat32 && alpha->numel() == 1, "alpha is one float32 on the device");
+        same_device(A, *alpha, "window_sddmm");
+    }
+    pspglue::DeviceGuard guard(A.device());
+    auto out = torch::empty({colIdx_w.size(0)}, A.options());
+    if (colIdx_w.numel() == 0) return out;
+    ok(psp_sddmm_window_f32(ip(rowPtr_w), ip(colIdx_w), fp(A), fp(B), alpha ? alpha->data_ptr<float>() : nullptr, fpw(out), (int)M,
+                            (int)colIdx_w.size(0), (int)A.size(1), (int)B.size(0), stream_of(A)));
+    return out;
+}
+
 // out[p] = values[p] * <A[row], B[col]>: the attention-score form (an addition of this build; the reference op
 // never multiplies the stored value in)
 static Tensor csr_sddmm_scaled(Tensor A, Tensor B, Tensor rowPtr, Tensor colIdx, Tensor values, int blkWarpNum)
@@ -344,6 +378,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     m.def("cusparse_sddmm_profile", &cusparse_sddmm_profile, "GFLOP/s of the rocSPARSE SDDMM baseline");
     m.def("genmask", &genmask, "CSR slot -> flat index into the 2x1 block values");
     // additions of this build
+    m.def("window_sddmm", &window_sddmm, "windowed CSR SDDMM (HIP, gfx950): (A, B, rowPtr_w, colIdx_w, alpha = None)", py::arg("A"),
+          py::arg("B"), py::arg("rowPtr_w"), py::arg("colIdx_w"), py::arg("alpha") = py::none());
+    m.def("window_sddmm_supported", &window_sddmm_supported, "is there a windowed SDDMM kernel for K columns?");
     m.def("csr_sddmm_scaled", &csr_sddmm_scaled, "values[p] * <A[row], B[col]>");
     m.def("csr_split_sddmm_scaled", &csr_split_sddmm_scaled, "values[p] * <A[row], B[col]> on the row-split format");
     m.def("csr_sddmm_scaled_rowmax", &csr_sddmm_scaled_rowmax, "[values[p] * <A[row], B[col]>, largest score of every row]");

@@ -202,9 +202,13 @@ class AGNNFunction(torch.autograd.Function):
         # relu_input: X holds pre-activation values; the activation and its backward ride on the dense products
         ctx.relu_input = bool(relu_input)
         X_prime = SpCONV.dense_relu_xw(X, weights) if relu_input else SpCONV.dense_xw(X, weights, False)
-        edge_feature = ParamSpMM.AGNN_sddmm(X_prime)
-        # csr: [nnz] ; 2x1 blocks: [nblk, 2] -- a single head scales both the same way
-        edge_attentions = (edge_feature * attention_w.reshape(())).contiguous()
+        if _fmt(ParamSpMM) == 4:
+            # windowed operator: the head's weight is multiplied in where the score is stored
+            edge_attentions = ParamSpMM.AGNN_sddmm(X_prime, attention_w.detach().reshape(-1)[:1])
+        else:
+            edge_feature = ParamSpMM.AGNN_sddmm(X_prime)
+            # csr: [nnz] ; 2x1 blocks: [nblk, 2] -- a single head scales both the same way
+            edge_attentions = (edge_feature * attention_w.reshape(())).contiguous()
         out = ParamSpMM.AGNN_spmm(edge_attentions, X_prime)
         ctx.save_for_backward(X, weights, edge_attentions)
         ctx.colIdx = colIdx
@@ -232,9 +236,10 @@ class AGNNFunction(torch.autograd.Function):
         # mm(d_attention[1, nnz] expanded to n_heads rows, colIdx.float()[nnz, 1])^T.  Every row of the product is the
         # same dot product over the nnz entries; as a GEMM it takes 20 ms on 2*10^7 entries (a 1 x nnz x 1 problem),
         # as a dot product some tens of microseconds.  The float copy of colIdx is made once per operator.
+        # A windowed operator keeps its entries in its own order inside the rows: its colIdx is the one that matches.
         col_f = getattr(op, "_colIdx_as_float", None)
         if col_f is None or col_f.numel() != ctx.colIdx.numel():
-            col_f = ctx.colIdx.reshape(-1).to(d_attention.dtype)
+            col_f = (op.colIdx if _fmt(op) == 4 else ctx.colIdx).reshape(-1).to(d_attention.dtype)
             op._colIdx_as_float = col_f
         d_attention_w = torch.dot(d_attention, col_f).reshape(1, 1).expand(1, n_heads)
         return d_input, d_weights, d_attention_w, None, None, None

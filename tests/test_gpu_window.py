@@ -169,6 +169,87 @@ def test_non_finite_inputs_stay_in_their_rows(oracle):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name", sorted(CASES))
+def test_window_sddmm_against_the_oracle(oracle, name):
+    """psp_sddmm_window_f32 against the oracle's CSR SDDMM on the layout's own arrays (rowPtr_w[0::2], colIdx_w is an
+    ordinary matrix with unsorted rows): 1e-6 + 1e-5 of the magnitudes summed per entry; A = B = ones gives K exactly
+    (the reference's known answer, SDDMM.py:127-128); alpha scales the result; with A == B the matrix is read once and
+    the result is bit for bit the one of two separate copies."""
+    from gpu_util import assert_close, dev
+    from paramspmm_ae_amd import _capi
+    import ParamSpMM
+
+    rowPtr, colIdx, val = CASES[name]()
+    M, nnz = rowPtr.size - 1, colIdx.size
+    rp, ci, _ = ParamSpMM.window_build(dev(rowPtr), dev(colIdx), dev(val))
+    ci_w = ci.cpu().numpy()
+    rows = np.repeat(np.arange(M), np.diff(rowPtr))
+    p, L = _capi.ptr, _capi.lib
+    st = torch.cuda.current_stream().cuda_stream
+
+    def run(A, B, K, alpha=None, rows_b=None):
+        out = torch.full((nnz,), float("nan"), device="cuda")
+        _capi.check(L.psp_sddmm_window_f32(p(rp), p(ci), p(A), p(B), p(alpha), p(out), M, nnz, K, B.shape[0] if rows_b is None else rows_b, st))
+        torch.cuda.synchronize()
+        return out
+
+    for K in (4, 16, 20, 32, 48, 64, 100, 128):
+        print("case sddmm", name, K, flush=True)
+        rng = np.random.default_rng(K)
+        A = rng.standard_normal((M + 2, K)).astype(np.float32)
+        B = rng.standard_normal((M + 5, K)).astype(np.float32)
+        want = oracle.sddmm_csr(rowPtr, ci_w, A, B)
+        scale = (np.abs(A[rows]) * np.abs(B[ci_w])).sum(1)
+        Ad, Bd = torch.from_numpy(A).cuda(), torch.from_numpy(B).cuda()
+        got = run(Ad, Bd, K)
+        assert_close(got, want, what="%s K=%d" % (name, K), scale=scale)
+        alpha = torch.tensor([-0.75], device="cuda")
+        assert torch.equal(run(Ad, Bd, K, alpha), got * -0.75)
+        # one matrix on both sides: its rows come from the ring
+        same = run(Bd, Bd, K)
+        assert_close(same, oracle.sddmm_csr(rowPtr, ci_w, B, B), what="%s K=%d, A == B" % (name, K),
+                     scale=(np.abs(B[rows]) * np.abs(B[ci_w])).sum(1))
+        assert torch.equal(same, run(Bd.clone(), Bd, K))
+        ones = torch.ones(M, K, device="cuda")
+        assert bool((run(ones, ones, K) == K).all())
+    # argument errors
+    X = torch.zeros(M, 18, device="cuda")
+    out = torch.zeros(max(nnz, 1), device="cuda")
+    assert L.psp_sddmm_window_f32(p(rp), p(ci), p(X), p(X), None, p(out), M, nnz, 18, M, st) == -1
+    assert L.psp_sddmm_window_f32(p(rp), p(ci), p(X), p(X), None, p(out), M, nnz, 132, M, st) == -1
+    assert L.psp_sddmm_window_f32(p(rp), p(ci), p(X), p(X), None, p(out), M, nnz, 16, M - 1, st) == -1  # A == B, too few rows
+
+
+@pytest.mark.gpu
+def test_window_sddmm_non_finite_rows_stay_in_their_entries(oracle):
+    from gpu_util import dev
+    from paramspmm_ae_amd import _capi
+    import ParamSpMM
+
+    rowPtr, colIdx, val = banded_csr(1500, 9, 30, 9, far=0.2, hub=(3, 400))
+    M, nnz = rowPtr.size - 1, colIdx.size
+    rp, ci, _ = ParamSpMM.window_build(dev(rowPtr), dev(colIdx), dev(val))
+    ci_w = ci.cpu().numpy()
+    rows = np.repeat(np.arange(M), np.diff(rowPtr))
+    for K in (16, 64):
+        X = np.random.default_rng(K).standard_normal((M, K)).astype(np.float32)
+        X[colIdx[5]] = np.inf
+        X[colIdx[colIdx.size // 2], 3] = np.nan
+        X[0] = np.inf       # the rows the clamped loads and the padding point at
+        X[M - 1] = np.inf
+        Xd = torch.from_numpy(X).cuda()
+        out = torch.zeros(nnz, device="cuda")
+        _capi.check(_capi.lib.psp_sddmm_window_f32(_capi.ptr(rp), _capi.ptr(ci), _capi.ptr(Xd), _capi.ptr(Xd), None, _capi.ptr(out), M,
+                                                   nnz, K, M, torch.cuda.current_stream().cuda_stream))
+        got = out.cpu().numpy()
+        touched = ~np.isfinite(X).all(1)
+        clean = ~touched[rows] & ~touched[ci_w]
+        assert np.isfinite(got[clean]).all() and not np.isfinite(got[~clean]).any()
+        want = oracle.sddmm_csr(rowPtr, ci_w, X, X)
+        np.testing.assert_allclose(got[clean], want[clean], rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.gpu
 def test_window_operator_through_the_modules_and_a_gcn_layer(oracle):
     """pcsr_spmm(window=True): SpMM, the fused forward / backward, the SDDMM on the permuted arrays, and a GCN layer's
     gradients against dense autograd."""
@@ -227,6 +308,51 @@ def test_window_operator_through_the_modules_and_a_gcn_layer(oracle):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("width", [16, 32, 20])
+def test_agnn_layer_on_a_windowed_operator(width):
+    """The attention layer on a windowed operator: forward against dense algebra, backward against the reference's
+    literal formulas (gnn_conv.py:153-180) -- the per-entry vectors follow the operator's own entry order, which
+    leaves every one of those sums unchanged.  Width 20 is not a width of the windowed SpMM's fused forms but is one
+    of the SDDMM's; all of them take the windowed kernels."""
+    from paramspmm_ae_amd.graph_input import graph_input
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from paramspmm_ae_amd.gnn_conv import AGNNConv
+
+    n = 700
+    rowPtr, colIdx, val = banded_csr(n, 7, 25, 31, far=0.2, hub=(11, 300))
+    g = graph_input("t", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val)
+    op = pcsr_spmm(g, vec_size=1, if_split=False, window=True)
+    rows = torch.from_numpy(np.repeat(np.arange(n), np.diff(rowPtr))).cuda()
+    pattern = torch.zeros(n, n, device="cuda")
+    pattern[rows, torch.from_numpy(colIdx.astype(np.int64)).cuda()] = 1.0
+    torch.manual_seed(1)
+    layer = AGNNConv(24, width).cuda()
+    X = torch.randn(n, 24, device="cuda", requires_grad=True)
+    ci = g.csr_data.colIdx.cuda().unsqueeze(-1)  # what the driver hands to the layer: the graph's own order
+    y = layer(X, {width: op}, ci)
+    Xp = X.detach() @ layer.weights.detach()
+    att = pattern * (Xp @ Xp.t()) * layer.attention_w.detach().reshape(())
+    torch.testing.assert_close(y, att @ Xp, rtol=1e-4, atol=1e-4)
+    dY = torch.randn_like(y)
+    y.backward(dY)
+    d_in_prime = att @ dY
+    torch.testing.assert_close(X.grad, d_in_prime @ layer.weights.detach().t(), rtol=1e-3, atol=1e-3)
+    torch.testing.assert_close(layer.weights.grad, X.detach().t() @ d_in_prime, rtol=1e-3, atol=1e-3)
+    d_att = (dY[rows] * dY[g.csr_data.colIdx.cuda().long()]).sum(1)
+    want = (d_att[None, :].double() @ ci.double()).t()
+    torch.testing.assert_close(layer.attention_w.grad.double(), want, rtol=1e-3, atol=1e-1)
+    # the scores themselves, against the CSR kernel on the same arrays
+    import ParamSDDMM
+
+    Xp = Xp.contiguous()
+    e = op.AGNN_sddmm(Xp)
+    ref = ParamSDDMM.csr_sddmm(Xp, Xp, op.rowPtr, op.colIdx, op.val, 1, 4)
+    torch.testing.assert_close(e, ref, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.gpu
 def test_training_with_windowed_operators_follows_training_with_the_csr_operators():
     """A community-ordered block model: most entries are local, configure_operators may keep the windowed layout
     (decided by timing), and GCN / GIN networks built on windowed operators produce the log-probabilities and take
@@ -265,6 +391,42 @@ def test_training_with_windowed_operators_follows_training_with_the_csr_operator
             model.eval()
             outs.append(model().detach())
         torch.testing.assert_close(outs[0], outs[1], rtol=2e-3, atol=2e-3)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("hidden", [16, 64])
+def test_attention_network_on_windowed_operators_equals_the_one_on_csr_operators(hidden):
+    """The five-layer attention network (GNN.py:82-101) on windowed operators: loss and every gradient of one training
+    step equal those of the same network (same seed, same dropout mask) on plain CSR operators."""
+    from paramspmm_ae_amd import GNN, synth
+    from paramspmm_ae_amd.graph_input import graph_input
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+    from paramspmm_ae_amd.gnn_conv import nll_loss_mean
+
+    r, c, n = synth.sbm(20000, 200, 12, 1.5, seed=6)
+    rowPtr, colIdx, val = synth.to_gcn_csr(r, c, n)
+    g = graph_input("sbm", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val)
+    ops = {"csr": pcsr_spmm(g, vec_size=1, if_split=False, CF=1, blkWarpNum=4), "window": pcsr_spmm(g, vec_size=1, if_split=False, window=True)}
+    torch.manual_seed(0)
+    x = torch.randn(n, 32, device="cuda")
+    labels = torch.randint(0, 16, (n,), device="cuda")
+    res = {}
+    for which, op in ops.items():
+        torch.manual_seed(1)
+        model = GNN.AGNN(16, 32, x, {16: op, 32: op, hidden: op}, hidden, g.csr_data.colIdx.cuda().unsqueeze(-1)).cuda()
+        with torch.no_grad():  # keep the attention scores of five stacked layers in range
+            for q in model.parameters():
+                q.mul_(0.3)
+        model.train()
+        torch.manual_seed(123)  # the dropout mask
+        loss = nll_loss_mean(model(), labels)
+        loss.backward()
+        res[which] = (loss.item(), [q.grad.clone() for q in model.parameters()])
+    assert abs(res["csr"][0] - res["window"][0]) <= 1e-4 * abs(res["csr"][0])
+    for a, b in zip(res["window"][1], res["csr"][1]):
+        torch.testing.assert_close(a, b, rtol=2e-3, atol=1e-4 * float(b.abs().max()) + 1e-6)
 
 
 @pytest.mark.gpu
