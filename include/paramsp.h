@@ -341,6 +341,22 @@ int psp_spmm_window_xw_f32(const int *rowPtr_w, const int *colIdx_w, const float
 int psp_sddmm_window_f32(const int *rowPtr_w, const int *colIdx_w, const float *A, const float *B, const float *alpha,
                          float *out, int M, int nnz, int K, int rows_b, psp_stream_t stream);
 
+/* One attention layer's sparse work over the same layout, the SDDMM and the SpMM of a direction in one pass over the
+ * window (the layer of gnn_conv.py:128-180 runs them as separate operators; no counterpart in the reference).
+ * X, dY: [>= M, K] row-major, 16-byte aligned; the matrix is square (every column index below M); K a multiple of 4 up
+ * to PSP_ATTN_WINDOW_MAX_K; Y, G: [rows_out, K], rows past M are cleared.
+ *   forward:  att[p] = alpha <X[row(p)], X[col(p)]> (alpha: one float on the device, or NULL for 1) in the layout's
+ *             entry order, Y[i] = sum_p att[p] X[col(p)].
+ *   backward: G[i] = sum_p att[p] dY[col(p)] and *wsum = sum_p <dY[row(p)], dY[col(p)]> (float)col(p), the reference's
+ *             literal formula for the gradient of the attention weight (gnn_conv.py:166-172: the SDDMM of the gradient
+ *             with itself times colIdx as floats); *wsum (device memory) is overwritten, the per-entry products are
+ *             never stored.  Workgroups add their shares to *wsum atomically, in no fixed order. */
+#define PSP_ATTN_WINDOW_MAX_K 64
+int psp_attn_window_forward_f32(const int *rowPtr_w, const int *colIdx_w, const float *X, const float *alpha, float *att,
+                                float *Y, int M, int nnz, int K, int rows_out, psp_stream_t stream);
+int psp_attn_window_backward_f32(const int *rowPtr_w, const int *colIdx_w, const float *att, const float *dY, float *G,
+                                 float *wsum, int M, int nnz, int K, int rows_out, psp_stream_t stream);
+
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: softmax over the stored entries of every CSR row (out[p] = exp(e[p]-max_r) / sum_r).
  * No counterpart in the reference (its AGNN layer applies no softmax, gnn_conv.py:136-142); it exists for

@@ -218,6 +218,60 @@ static std::vector<Tensor> window_xw(Tensor X, Tensor W, bool transW, Tensor row
     return {Y};
 }
 
+// ---- attention layer on the windowed layout: SDDMM and SpMM of a direction in one launch ---------------------------------
+static bool attn_window_supported(long K) { return K >= 4 && K % 4 == 0 && K <= PSP_ATTN_WINDOW_MAX_K; }
+
+static void check_attn_window(const Tensor &X, const Tensor &rowPtr_w, const Tensor &colIdx_w, const char *what)
+{
+    need_gpu(X, what);
+    need_gpu(rowPtr_w, "rowPtr_w");
+    need_gpu(colIdx_w, "colIdx_w");
+    need_f32(X, what, 2);
+    need_i32(rowPtr_w, "rowPtr_w");
+    need_i32(colIdx_w, "colIdx_w");
+    pspglue::same_device(X, rowPtr_w, "attn_window");
+    pspglue::same_device(X, colIdx_w, "attn_window");
+    TORCH_CHECK(rowPtr_w.size(0) >= 2 && rowPtr_w.size(0) % 2 == 0, "rowPtr of the windowed format has 2 M + 2 entries");
+    TORCH_CHECK(attn_window_supported(X.size(1)), "attn_window: the width must be a multiple of 4 up to ", PSP_ATTN_WINDOW_MAX_K);
+    TORCH_CHECK((rowPtr_w.size(0) - 2) / 2 <= X.size(0), "rowPtr_w describes more rows than the dense operand has");
+}
+
+// (X, rowPtr_w, colIdx_w, alpha | None) -> [att = alpha <X_i, X_j> per stored entry, Y = att-weighted sum of the X rows]
+static std::vector<Tensor> attn_window_forward(Tensor X, Tensor rowPtr_w, Tensor colIdx_w, c10::optional<Tensor> alpha)
+{
+    check_attn_window(X, rowPtr_w, colIdx_w, "X");
+    if (alpha) {
+        need_gpu(*alpha, "alpha");
+        TORCH_CHECK(alpha->scalar_type() == torch::kFloat32 && alpha->numel() == 1, "alpha is one float32 on the device");
+        pspglue::same_device(X, *alpha, "attn_window");
+    }
+    pspglue::DeviceGuard guard(X.device());
+    Tensor att = torch::empty({colIdx_w.size(0)}, X.options());
+    Tensor Y = torch::empty_like(X);
+    const float *a = alpha ? alpha->data_ptr<float>() : nullptr;
+    ok(psp_attn_window_forward_f32(ip(rowPtr_w), ip(colIdx_w), fp(X), a, colIdx_w.numel() ? fpw(att) : nullptr, fpw(Y),
+                                   (int)(rowPtr_w.size(0) - 2) / 2, (int)colIdx_w.size(0), (int)X.size(1), (int)X.size(0),
+                                   stream_of(X)));
+    return {att, Y};
+}
+
+// (dY, att, rowPtr_w, colIdx_w) -> [G = att-weighted sum of the dY rows, sum_p <dY_i, dY_j> float(col(p)) as a 1-element tensor]
+static std::vector<Tensor> attn_window_backward(Tensor dY, Tensor att, Tensor rowPtr_w, Tensor colIdx_w)
+{
+    check_attn_window(dY, rowPtr_w, colIdx_w, "dY");
+    need_gpu(att, "att");
+    need_f32(att, "att", 1);
+    TORCH_CHECK(att.size(0) == colIdx_w.size(0), "att has one value per stored entry");
+    pspglue::same_device(dY, att, "attn_window");
+    pspglue::DeviceGuard guard(dY.device());
+    Tensor G = torch::empty_like(dY);
+    Tensor wsum = torch::empty({1}, dY.options());
+    ok(psp_attn_window_backward_f32(ip(rowPtr_w), ip(colIdx_w), att.numel() ? fp(att) : nullptr, fp(dY), fpw(G), wsum.data_ptr<float>(),
+                                    (int)(rowPtr_w.size(0) - 2) / 2, (int)colIdx_w.size(0), (int)dY.size(1), (int)dY.size(0),
+                                    stream_of(dY)));
+    return {G, wsum};
+}
+
 static Tensor forward_impl(int fmt, const Tensor &H, const Tensor &W, const Tensor &rowPtr, const Tensor &colIdx,
                            const Tensor &values, const Tensor *target_row, int CF, int blkWarpNum)
 {
@@ -338,6 +392,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     }, "max(Z, 0)^T * G: (Z, G)");
     m.def("nll_loss_mean", &nll_loss_mean, "[loss, stats] of the mean negative log-likelihood (log-probabilities, int64 labels)");
     m.def("nll_loss_mean_backward", &nll_loss_mean_backward, "gradient w.r.t. the log-probabilities: (labels, grad_loss, stats, n, C)");
+    m.def("attn_window_forward", &attn_window_forward,
+          "attention layer on the windowed layout: (X, rowPtr_w, colIdx_w, alpha | None) -> [att, Y]");
+    m.def("attn_window_backward", &attn_window_backward,
+          "attention layer on the windowed layout: (dY, att, rowPtr_w, colIdx_w) -> [G, weight-gradient sum]");
+    m.def("attn_window_supported", &attn_window_supported, "is there a fused attention kernel for this width?");
     m.def("window_xw", &window_xw,
           "windowed layout, dense product folded in: (X, W, transW, rowPtr_w, colIdx_w, values_w, relu_input, mask | None, want_raw) -> [Y] or [Y, A f(X)]");
     m.def("window_xw_supported", &window_xw_supported, "widths the folded product exists for");

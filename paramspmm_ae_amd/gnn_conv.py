@@ -202,14 +202,20 @@ class AGNNFunction(torch.autograd.Function):
         # relu_input: X holds pre-activation values; the activation and its backward ride on the dense products
         ctx.relu_input = bool(relu_input)
         X_prime = SpCONV.dense_relu_xw(X, weights) if relu_input else SpCONV.dense_xw(X, weights, False)
-        if _fmt(ParamSpMM) == 4:
-            # windowed operator: the head's weight is multiplied in where the score is stored
-            edge_attentions = ParamSpMM.AGNN_sddmm(X_prime, attention_w.detach().reshape(-1)[:1])
+        ctx.fused = (_fmt(ParamSpMM) == 4 and X_prime.dtype == torch.float32
+                     and SpCONV.attn_window_supported(int(X_prime.shape[1])))
+        if ctx.fused:
+            # windowed operator: scores (the head's weight multiplied in) and their aggregation in one launch
+            edge_attentions, out = SpCONV.attn_window_forward(X_prime, ParamSpMM.spmm_rowPtr, ParamSpMM.colIdx,
+                                                              attention_w.detach().reshape(-1)[:1])
         else:
-            edge_feature = ParamSpMM.AGNN_sddmm(X_prime)
-            # csr: [nnz] ; 2x1 blocks: [nblk, 2] -- a single head scales both the same way
-            edge_attentions = (edge_feature * attention_w.reshape(())).contiguous()
-        out = ParamSpMM.AGNN_spmm(edge_attentions, X_prime)
+            if _fmt(ParamSpMM) == 4:
+                edge_attentions = ParamSpMM.AGNN_sddmm(X_prime, attention_w.detach().reshape(-1)[:1])
+            else:
+                edge_feature = ParamSpMM.AGNN_sddmm(X_prime)
+                # csr: [nnz] ; 2x1 blocks: [nblk, 2] -- a single head scales both the same way
+                edge_attentions = (edge_feature * attention_w.reshape(())).contiguous()
+            out = ParamSpMM.AGNN_spmm(edge_attentions, X_prime)
         ctx.save_for_backward(X, weights, edge_attentions)
         ctx.colIdx = colIdx
         ctx.ParamSpMM = ParamSpMM
@@ -220,7 +226,11 @@ class AGNNFunction(torch.autograd.Function):
         op = ctx.ParamSpMM
         X, weights, edge_attentions = ctx.saved_tensors
         d_output = d_output.contiguous()
-        d_input_prime = op.AGNN_spmm(edge_attentions, d_output)
+        if ctx.fused:
+            # A_att dY and the reference's sum for the attention weight (below) in one launch
+            d_input_prime, d_attention_w = SpCONV.attn_window_backward(d_output, edge_attentions, op.spmm_rowPtr, op.colIdx)
+        else:
+            d_input_prime = op.AGNN_spmm(edge_attentions, d_output)
         if not ctx.needs_input_grad[0]:
             d_input = None
         elif ctx.relu_input:
@@ -229,6 +239,8 @@ class AGNNFunction(torch.autograd.Function):
             d_input = SpCONV.dense_xw(d_input_prime, weights, True)
         # X^T * d_input_prime (relu(X)^T when the layer reads X through the activation)
         d_weights = SpCONV.weight_gradient_relu(X, d_input_prime) if ctx.relu_input else SpCONV.weight_gradient(X, d_input_prime)
+        if ctx.fused:
+            return d_input, d_weights, d_attention_w.reshape(1, 1).expand(1, n_heads), None, None, None
         d_attention = op.AGNN_sddmm(d_output)
         if d_attention.dim() != 1:
             d_attention = d_attention.view(-1)[op.mask]  # block layout -> CSR slots

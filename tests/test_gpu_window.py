@@ -221,6 +221,67 @@ def test_window_sddmm_against_the_oracle(oracle, name):
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("name", ["banded", "banded_hub", "wide_band", "random", "tiny"])
+def test_attention_passes_against_the_oracle(oracle, name):
+    """psp_attn_window_forward_f32 / _backward_f32 against the oracle's SDDMM followed by its SpMM on the layout's own
+    arrays: scores to 1e-6 + 1e-5 of the magnitudes summed per entry, the aggregated rows to twice that of the
+    magnitudes summed per row (two chained roundings), the weight-gradient sum against float64."""
+    from gpu_util import assert_close, dev
+    from paramspmm_ae_amd import _capi
+    import ParamSpMM
+
+    rowPtr, colIdx, val = CASES[name]()
+    M, nnz = rowPtr.size - 1, colIdx.size
+    rp, ci, _ = ParamSpMM.window_build(dev(rowPtr), dev(colIdx), dev(val))
+    ci_w = ci.cpu().numpy()
+    rows = np.repeat(np.arange(M), np.diff(rowPtr))
+    p, L = _capi.ptr, _capi.lib
+    st = torch.cuda.current_stream().cuda_stream
+    for K in (4, 16, 20, 32, 48, 64):
+        print("case attn", name, K, flush=True)
+        rng = np.random.default_rng(K)
+        X = (rng.standard_normal((M + 3, K)) / np.sqrt(K)).astype(np.float32)
+        alpha = np.float32(-1.25)
+        e = oracle.sddmm_csr(rowPtr, ci_w, X, X)
+        att_want = (e * alpha).astype(np.float32)
+        e_scale = (np.abs(X[rows]) * np.abs(X[ci_w])).sum(1) * abs(alpha)
+        Y_want = oracle.spmm_csr(rowPtr, ci_w, att_want, X, rows_out=M + 3)
+        Y_scale = oracle.spmm_csr(rowPtr, ci_w, e_scale.astype(np.float32), np.abs(X), rows_out=M + 3)
+        Xd = torch.from_numpy(X).cuda()
+        att = torch.full((nnz,), float("nan"), device="cuda")
+        Y = torch.full((M + 3, K), float("nan"), device="cuda")
+        _capi.check(L.psp_attn_window_forward_f32(p(rp), p(ci), p(Xd), p(torch.tensor([alpha], device="cuda")), p(att), p(Y), M, nnz, K,
+                                                  M + 3, st))
+        torch.cuda.synchronize()
+        assert_close(att, att_want, what="scores %s K=%d" % (name, K), scale=e_scale)
+        assert_close(Y, Y_want, rtol=2e-5, what="aggregate %s K=%d" % (name, K), scale=Y_scale)
+        assert bool((Y[M:] == 0).all())
+        # the scores equal the windowed SDDMM's bit for bit when both sum a score the same way (same lane group shape)
+        sd = torch.empty(nnz, device="cuda")
+        _capi.check(L.psp_sddmm_window_f32(p(rp), p(ci), p(Xd), p(Xd), p(torch.tensor([alpha], device="cuda")), p(sd), M, nnz, K, M + 3, st))
+        assert_close(sd, att.cpu().numpy(), what="scores vs windowed SDDMM", scale=e_scale)
+        # backward: G = sum att dY[col]; wsum = sum <dY_i, dY_j> float(col)
+        dY = (rng.standard_normal((M + 3, K)) / np.sqrt(K)).astype(np.float32)
+        att_in = rng.standard_normal(nnz).astype(np.float32)
+        G_want = oracle.spmm_csr(rowPtr, ci_w, att_in, dY, rows_out=M + 3)
+        G_scale = oracle.spmm_csr(rowPtr, ci_w, np.abs(att_in), np.abs(dY), rows_out=M + 3)
+        d = (dY[rows].astype(np.float64) * dY[ci_w].astype(np.float64)).sum(1)
+        w_want = float((d * ci_w.astype(np.float32).astype(np.float64)).sum())
+        w_scale = float(((np.abs(dY[rows]).astype(np.float64) * np.abs(dY[ci_w])).sum(1) * ci_w).sum())
+        G = torch.full((M + 3, K), float("nan"), device="cuda")
+        wsum = torch.full((1,), float("nan"), device="cuda")
+        dYd, att_d = torch.from_numpy(dY).cuda(), torch.from_numpy(att_in).cuda()
+        _capi.check(L.psp_attn_window_backward_f32(p(rp), p(ci), p(att_d), p(dYd), p(G), p(wsum), M, nnz, K, M + 3, st))
+        torch.cuda.synchronize()
+        assert_close(G, G_want, what="gradient aggregate %s K=%d" % (name, K), scale=G_scale)
+        assert bool((G[M:] == 0).all())
+        assert abs(float(wsum.item()) - w_want) <= 1e-6 + 2e-5 * w_scale, (float(wsum.item()), w_want, w_scale)
+    X = torch.zeros(M, 72, device="cuda")
+    assert L.psp_attn_window_forward_f32(p(rp), p(ci), p(X), None, p(att), p(X), M, nnz, 72, M, st) == -1   # wider than the kernel covers
+    assert L.psp_attn_window_backward_f32(p(rp), p(ci), p(att), p(X), p(X), None, M, nnz, 16, M, st) == -1   # no place for the sum
+
+
+@pytest.mark.gpu
 def test_window_sddmm_non_finite_rows_stay_in_their_entries(oracle):
     from gpu_util import dev
     from paramspmm_ae_amd import _capi
@@ -308,12 +369,12 @@ def test_window_operator_through_the_modules_and_a_gcn_layer(oracle):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("width", [16, 32, 20])
+@pytest.mark.parametrize("width", [16, 32, 20, 64, 96])
 def test_agnn_layer_on_a_windowed_operator(width):
     """The attention layer on a windowed operator: forward against dense algebra, backward against the reference's
     literal formulas (gnn_conv.py:153-180) -- the per-entry vectors follow the operator's own entry order, which
-    leaves every one of those sums unchanged.  Width 20 is not a width of the windowed SpMM's fused forms but is one
-    of the SDDMM's; all of them take the windowed kernels."""
+    leaves every one of those sums unchanged.  Up to 64 columns a direction is one launch (scores and aggregation
+    together, psp_attn_window_*); 96 runs the windowed SDDMM and SpMM one after the other."""
     from paramspmm_ae_amd.graph_input import graph_input
     from paramspmm_ae_amd.PCSR import pcsr_spmm
     from paramspmm_ae_amd.gnn_conv import AGNNConv
