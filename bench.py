@@ -19,7 +19,7 @@ The JSON line also carries
   sddmm            one SDDMM width (K = 64) on the same pattern with its own roofline;
   other_graphs     the other graphs of the benchmark set in the decider's configuration: 5-point stencil 2048^2 at
                    N = 64 / 128, block model (community order and random order) at N = 128, Chung-Lu 2.45M at N = 128;
-  gcn_epoch_ms     GCN / GIN training epochs (5 layers, hidden 16 / 32 / 128, 16 classes) on the 1M-node block model,
+  gcn_epoch_ms     GCN / GIN / AGNN training epochs (5 layers, hidden 16 / 32 / 128, 16 classes) on the 1M-node block model,
                    1 warm-up + 200 timed epochs as in GNN.py:126-151;
   cpu_baseline     torch.sparse.mm on the host cores (the product the reference verifies against, verification.py:18-46)
                    on a bounded sample of the widths; cpu_scalar_port is the oracle's one-thread C restatement, which also
@@ -979,12 +979,12 @@ def main():
         epochs = {}
         n_epochs = 200  # the reference's protocol: 1 warm-up epoch + 200 timed ones (GNN.py:126-151)
         with contextlib.redirect_stdout(sys.stderr):
-            for net in ("GCN", "GIN"):
+            for net in ("GCN", "GIN", "AGNN"):
                 res = GNN.main(["--net", net, "--synthetic", "C5", "--hidden_list", "16", "32", "128", "--num_classes", "16",
                                 "--num_features", "32", "--num_epoches", str(n_epochs)])
                 epochs[net] = {str(h): round(float(ms), 3) for (_, h), ms in res.items()}
         out["gcn_epoch_ms"] = {"value": epochs["GCN"]["16"], "unit": "ms per epoch", "epochs": n_epochs,
-                               "by_hidden": epochs["GCN"], "gin_by_hidden": epochs["GIN"],
+                               "by_hidden": epochs["GCN"], "gin_by_hidden": epochs["GIN"], "agnn_by_hidden": epochs["AGNN"],
                                "config": "5 layers, hidden 16 / 32 / 128 (value: GCN, hidden 16), 16 classes, 32 features, "
                                          "fwd+bwd+Adam, SBM 1M nodes (community order), decider-picked operators"}
 
