@@ -97,6 +97,21 @@ def measured_sddmm_traffic(graph, K, fmt, bw):
     return None
 
 
+def _event_ms(fn, warmup, iters):
+    """Mean milliseconds per call of ``fn`` (HIP events on the current stream, which is the one the operators launch on)."""
+    import torch
+
+    for _ in range(warmup):
+        fn()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / iters
+
+
 def other_graph_leg(name, dims, decider, reps=10, reorder=None):
     """One more graph of the benchmark set at a few widths, in the decider's configuration: per width the mean
     launch duration (HIP events on the launching stream), algorithmic bytes and their fraction of the HBM roofline,
@@ -152,6 +167,20 @@ def other_graph_leg(name, dims, decider, reps=10, reorder=None):
     out = {"nodes": n, "nnz": int(nnz), "setup_s": round(time.time() - t0, 1), "widths": res}
     if win is not None:
         out["window_local_share"] = round(win.window_local_share, 4)
+        # the SDDMM <X_i, X_j> (the attention scores) on the same matrix: the CSR kernel and the windowed one.
+        # Algorithmic bytes: row pointers, columns, the feature matrix once, one float per entry.
+        out["sddmm"] = []
+        csr = ops[0]
+        for K in dims:
+            if K % 4:
+                continue
+            X = torch.randn(rows, K, device="cuda", generator=gen)
+            ms_c = _event_ms(lambda: csr.AGNN_sddmm(X), 3, reps)
+            ms_w = _event_ms(lambda: win.AGNN_sddmm(X), 3, reps)
+            b_alg = 4 * (n + 1) + 8 * nnz + 4 * n * K
+            out["sddmm"].append({"K": K, "csr_ms": round(ms_c, 5), "windowed_ms": round(ms_w, 5),
+                                 "alg_bytes": int(b_alg), "windowed_frac": round(b_alg / ms_w / 1e6 / HBM_PEAK_GBS, 4)})
+            del X
     del ops, graph, win
     torch.cuda.empty_cache()
     return out
