@@ -25,7 +25,7 @@ int psp_fail(int code, const char *fmt, ...)
 }
 
 // Library-wide options: defaults, overridden once by the environment (PSP_XCD_STRIPE_ROWS, PSP_ALIGN_PCT,
-// PSP_SPLIT_CLEAR_MIN, PSP_WHOLE_ROWS) when the library is first used, and afterwards only through psp_set_option.
+// PSP_SPLIT_CLEAR_MIN, PSP_WHOLE_ROWS, PSP_DENSE_SPLIT) when the library is first used, and afterwards only through psp_set_option.
 psp_options &psp_opts(void)
 {
     static psp_options o = [] {
@@ -34,6 +34,7 @@ psp_options &psp_opts(void)
         d.align_pct = 50;
         d.split_clear_min = (long long)4 << 20;
         d.whole_rows = 0;
+        d.dense_split = 1;
         if (const char *e = getenv("PSP_XCD_STRIPE_ROWS")) {
             if (atoi(e) > 0) d.stripe_rows = atoi(e);
         }
@@ -44,6 +45,7 @@ psp_options &psp_opts(void)
             if (atoll(e) >= 0) d.split_clear_min = atoll(e);
         }
         if (const char *e = getenv("PSP_WHOLE_ROWS")) d.whole_rows = atoi(e) != 0;
+        if (const char *e = getenv("PSP_DENSE_SPLIT")) d.dense_split = atoi(e) != 0;
         return d;
     }();
     return o;
@@ -66,6 +68,9 @@ PSP_EXPORT int psp_set_option(const char *name, long long value)
     } else if (!strcmp(name, "whole_rows")) {
         PSP_REQUIRE(value == 0 || value == 1, "set_option: whole_rows is 0 or 1");
         o.whole_rows = (int)value;
+    } else if (!strcmp(name, "dense_split")) {
+        PSP_REQUIRE(value == 0 || value == 1, "set_option: dense_split is 0 or 1");
+        o.dense_split = (int)value;
     } else {
         return psp_fail(PSP_ERR_ARG, "set_option: unknown option '%s'", name);
     }
@@ -80,6 +85,7 @@ PSP_EXPORT long long psp_get_option(const char *name)
     if (!strcmp(name, "align_pct")) return o.align_pct;
     if (!strcmp(name, "split_clear_min")) return o.split_clear_min;
     if (!strcmp(name, "whole_rows")) return o.whole_rows;
+    if (!strcmp(name, "dense_split")) return o.dense_split;
     return psp_fail(PSP_ERR_ARG, "get_option: unknown option '%s'", name);
 }
 

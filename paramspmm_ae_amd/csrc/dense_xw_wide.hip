@@ -22,6 +22,7 @@
 // gfx950 only, whose CUs have 160 KB, and two workgroups per CU (the launch shape) need 132 KB of it.  The grid is sized
 // to the GPU and every wavefront walks blocks of 32 rows with the next block's loads in flight.
 #include "psp_common.h"
+#include <cstdlib>
 
 typedef float psp_f32x4 __attribute__((ext_vector_type(4)));
 
@@ -139,6 +140,159 @@ psp_xw_wide_kernel(const float *__restrict__ X, const float *__restrict__ W, flo
     }
 }
 
+// ---- the 128 x 128 product on the bf16 matrix-core path -----------------------------------------------------------------
+// At 128 x 128 the fp32 instruction above needs as long for its 32 kflop per row as the memory system needs for the row's
+// 1 KB.  gfx950 multiplies bf16 sixteen times as fast, and an fp32 number is the exact sum of three bf16 numbers
+// (x = hi + mid + lo, 8 + 8 + 8 significant bits), so x w = sum of nine bf16 products, of which the six with at least
+// 16 significant bits between them (hi hi, hi mid, mid hi, mid mid, hi lo, lo hi) carry the product to 2^-23 of |x||w|
+// -- the rounding level of an fp32 product -- and are accumulated in fp32 by v_mfma_f32_16x16x32_bf16.  Six instructions
+// of 16 cycles replace eight of 32: the kernel is bound by its 1 KB per row again.  Same transposed form and the same
+// lane roles as above; a contraction step covers 32 columns: lane (r, q) supplies the eight values of its float4 pair
+// (2s, 2s + 1), i.e. columns 32s + 16 (i / 4) + 4q + i % 4 stand for k = 8q + i, and the W fragments in LDS follow the same
+// rule: [s][tile j][hi | mid | lo][lane][8 bf16], one 16-byte read per fragment.  An infinite input turns its products
+// into NaN (inf - inf in the split) instead of +-inf; NaN stays NaN.
+typedef __bf16 psp_bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 psp_bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int psp_u32x4 __attribute__((ext_vector_type(4)));
+typedef float psp_f32x2 __attribute__((ext_vector_type(2)));
+
+// two floats -> their three bf16 terms, packed in pairs (low half = first float)
+__device__ __forceinline__ void psp_split3(float a, float b, unsigned &hi, unsigned &mid, unsigned &lo)
+{
+    psp_f32x2 v = {a, b};
+    hi = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
+    v[0] = a - __uint_as_float(hi << 16);
+    v[1] = b - __uint_as_float(hi & 0xffff0000u);
+    mid = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
+    v[0] -= __uint_as_float(mid << 16);
+    v[1] -= __uint_as_float(mid & 0xffff0000u);
+    lo = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
+}
+
+template <bool RELU_X, bool MASK>
+__global__ void __launch_bounds__(512)
+psp_xw_wide_split_kernel(const float *__restrict__ X, const float *__restrict__ W, float *__restrict__ Y, long long n,
+                         const float *__restrict__ mask, int transW, long long nblocks)
+{
+    constexpr int K1 = 128, K2 = 128;
+    constexpr int T = K2 / 16;   // column tiles
+    constexpr int KT = K1 / 16;  // float4 loads per lane and row block
+    constexpr int KS = K1 / 32;  // contraction steps
+    extern __shared__ __align__(16) unsigned short Wb[];  // [KS][T][3][64][8]
+
+    for (int idx = threadIdx.x; idx < K1 * K2; idx += blockDim.x) {
+        const int i = idx & 7, l = (idx >> 3) & 63, sj = idx >> 9;  // sj = s * T + j
+        const int j = sj % T, st = sj / T;
+        const int r_ = l & 15, q_ = l >> 4;
+        const int k = 32 * st + 16 * (i >> 2) + 4 * q_ + (i & 3), c = 16 * j + r_;
+        const float w = transW ? W[c * K1 + k] : W[k * K2 + c];
+        unsigned hi, mid, lo;
+        psp_split3(w, 0.0f, hi, mid, lo);
+        unsigned short *at = Wb + ((size_t)(sj * 3) * 64 + l) * 8 + i;
+        at[0] = (unsigned short)hi;
+        at[64 * 8] = (unsigned short)mid;
+        at[2 * 64 * 8] = (unsigned short)lo;
+    }
+    __syncthreads();
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 15, q = lane >> 4;
+    const int waves = blockDim.x >> 6;
+    const long long stride = (long long)gridDim.x * waves;
+    long long blk = (long long)blockIdx.x * waves + wave;
+    if (blk >= nblocks) return;
+
+    psp_f32x4 xa[2][KT], xb[2][KT];
+    auto load_block = [&](long long b, psp_f32x4 (&x)[2][KT]) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            long long row = b * XWW_ROWS + 16 * h + r;
+            if (row >= n) row = n - 1;  // loaded and computed, never stored
+            const psp_f32x4 *xr = (const psp_f32x4 *)(X + row * K1) + q;
+#pragma unroll
+            for (int t = 0; t < KT; t++) x[h][t] = xr[4 * t];
+        }
+    };
+    auto compute_block = [&](long long b, psp_f32x4 (&x)[2][KT]) {
+        psp_f32x4 acc[2][T];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int j = 0; j < T; j++) acc[h][j] = psp_f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int st = 0; st < KS; st++) {
+            psp_u32x4 xh[2], xm[2], xl[2];
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    float a = x[h][2 * st + (g >> 1)][2 * (g & 1)], c = x[h][2 * st + (g >> 1)][2 * (g & 1) + 1];
+                    if constexpr (RELU_X) {
+                        a = a < 0.0f ? 0.0f : a;  // NaN stays NaN
+                        c = c < 0.0f ? 0.0f : c;
+                    }
+                    unsigned h_, m_, l_;
+                    psp_split3(a, c, h_, m_, l_);
+                    xh[h][g] = h_, xm[h][g] = m_, xl[h][g] = l_;
+                }
+            const psp_u32x4 *wf = (const psp_u32x4 *)Wb + (size_t)(st * T * 3) * 64 + lane;
+#pragma unroll
+            for (int jp = 0; jp < T; jp += 2) {
+                psp_u32x4 w[2][3];
+#pragma unroll
+                for (int u = 0; u < 2; u++)
+#pragma unroll
+                    for (int p = 0; p < 3; p++) w[u][p] = wf[((jp + u) * 3 + p) * 64];
+                // small terms first; four independent accumulators between two instructions on the same one
+#define XWS_TERM(WP_, XV_)                                                                                          \
+    _Pragma("unroll") for (int u = 0; u < 2; u++) _Pragma("unroll") for (int h = 0; h < 2; h++)                       \
+        acc[h][jp + u] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(psp_bf16x8, w[u][WP_]),           \
+                                                                 __builtin_bit_cast(psp_bf16x8, XV_[h]), acc[h][jp + u], 0, 0, 0);
+                XWS_TERM(2, xh)
+                XWS_TERM(0, xl)
+                XWS_TERM(1, xm)
+                XWS_TERM(1, xh)
+                XWS_TERM(0, xm)
+                XWS_TERM(0, xh)
+#undef XWS_TERM
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const long long row = b * XWW_ROWS + 16 * h + r;
+            if (row >= n) continue;
+            psp_f32x4 *yr = (psp_f32x4 *)(Y + row * K2) + q;
+            const psp_f32x4 *mr = (const psp_f32x4 *)(mask + row * K2) + q;
+#pragma unroll
+            for (int j = 0; j < T; j++) {
+                psp_f32x4 o = acc[h][j];
+                if constexpr (MASK) {
+                    const psp_f32x4 m = mr[4 * j];
+#pragma unroll
+                    for (int c = 0; c < 4; c++) o[c] = m[c] > 0.0f ? o[c] : 0.0f;
+                }
+                yr[4 * j] = o;
+            }
+        }
+    };
+
+    load_block(blk, xa);
+    while (true) {
+        long long nxt = blk + stride;
+        if (nxt < nblocks) load_block(nxt, xb);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_block(blk, xa);
+        if (nxt >= nblocks) break;
+        blk = nxt;
+        nxt = blk + stride;
+        if (nxt < nblocks) load_block(nxt, xa);
+        __builtin_amdgcn_sched_barrier(0);
+        compute_block(blk, xb);
+        if (nxt >= nblocks) break;
+        blk = nxt;
+    }
+}
+
 typedef void (*psp_xw_wide_kernel_t)(const float *, const float *, float *, long long, const float *, int, long long);
 
 static psp_xw_wide_kernel_t xw_wide_lookup(int K1, int K2, bool relu_x, bool mask)
@@ -176,6 +330,24 @@ int psp_xw_wide_launch(const float *X, const float *W, float *Y, long long n, in
     psp_xw_wide_kernel_t k = xw_wide_lookup(K1, K2, relu_x != 0, mask != nullptr);
     if (!k) return psp_fail(PSP_ERR_ARG, "gemm_xw: unsupported widths %d x %d", K1, K2);
     const long long nblocks = (n + XWW_ROWS - 1) / XWW_ROWS;
+    if (K1 == 128 && K2 == 128 && psp_opts().dense_split) {
+        psp_xw_wide_kernel_t ks = mask ? psp_xw_wide_split_kernel<false, true>
+                                       : (relu_x ? psp_xw_wide_split_kernel<true, false> : psp_xw_wide_split_kernel<false, false>);
+        const int lds = (K1 / 32) * (K2 / 16) * 3 * 64 * 16;  // 96 KB: one workgroup of eight wavefronts per CU
+        static bool raised[3];
+        const int which = mask ? 0 : (relu_x ? 1 : 2);
+        if (!raised[which]) {
+            const hipError_t e = hipFuncSetAttribute((const void *)ks, hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+            if (e != hipSuccess) return psp_fail(PSP_ERR_LAUNCH, "gemm_xw: %d bytes of LDS refused: %s", lds, hipGetErrorString(e));
+            raised[which] = true;
+        }
+        // eight wavefronts per workgroup, one workgroup per CU (measured against four and six: 267 / 278 / 283 us at 10^6 rows)
+        const int wv = 8;
+        const long long want_s = (nblocks + wv - 1) / wv;
+        const int grid_s = (int)(want_s < 256 ? want_s : 256);
+        hipLaunchKernelGGL(ks, dim3(grid_s), dim3(64 * wv), lds, stream, X, W, Y, n, mask, transW, nblocks);
+        return psp_check_launch("gemm_xw wide split kernel");
+    }
     // 4 wavefronts per workgroup, two workgroups per CU (two copies of W in LDS side by side); measured against 6 and 8
     // wavefronts per workgroup and one to four workgroups per CU at 10^6 rows: nothing faster
     const int waves = 4;

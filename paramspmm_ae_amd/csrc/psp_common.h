@@ -58,6 +58,7 @@ struct psp_options {
     int align_pct;              // whole segments per lane group when that costs at most this many percent more steps
     long long split_clear_min;  // row-split outputs of at least this many floats are cleared selectively
     int whole_rows;             // SpMM: a lane group always takes whole segments (reference summation order)
+    int dense_split;            // 128 x 128 layer products: fp32 operands as three bf16 terms on the bf16 matrix-core path
 };
 psp_options &psp_opts(void);
 int psp_stripe_rows(void);

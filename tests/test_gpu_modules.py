@@ -531,6 +531,45 @@ def test_dense_xw_matches_torch(K1, K2):
     assert torch.all((small.double() - want[:100]).abs() <= 1e-5 * scale[:100] + 1e-6)
 
 
+@pytest.mark.parametrize("n", [31, 100_003])
+def test_the_128_wide_dense_product_on_either_matrix_core_path(n):
+    """psp_gemm_xw_act_f32 at 128 x 128 with the option dense_split on (three bf16 terms per operand, six bf16
+    matrix-core products) and off (the fp32 instruction): both within 1e-6 + 1e-5 |X||W| of float64, all three forms
+    (plain, ReLU on the input, masked output, W and W^T); a non-finite input stays in its row on both paths."""
+    from paramspmm_ae_amd import _capi
+
+    L, p = _capi.lib, _capi.ptr
+    g = torch.Generator(device="cuda").manual_seed(n)
+    X = torch.randn(n, 128, device="cuda", generator=g) * torch.logspace(-3, 3, 128, device="cuda")  # a wide range of magnitudes
+    W = torch.randn(128, 128, device="cuda", generator=g)
+    Z = torch.randn(n, 128, device="cuda", generator=g)
+    Wt = W.t().contiguous()
+    st = torch.cuda.current_stream().cuda_stream
+    scale = X.abs().double() @ W.abs().double()
+    assert L.psp_get_option(b"dense_split") == 1
+    try:
+        for split in (1, 0):
+            _capi.check(L.psp_set_option(b"dense_split", split))
+            for transW, relu, mask in ((0, 0, None), (1, 0, None), (0, 1, None), (1, 0, Z)):
+                Y = torch.full((n, 128), float("nan"), device="cuda")
+                _capi.check(L.psp_gemm_xw_act_f32(p(X), p(Wt if transW else W), p(Y), n, 128, 128, transW, relu, p(mask), st))
+                want = (torch.relu(X) if relu else X).double() @ W.double()
+                if mask is not None:
+                    want = want * (Z > 0)
+                    assert bool((Y[Z <= 0] == 0).all())
+                assert torch.all((Y.double() - want).abs() <= 1e-5 * scale + 1e-6), (split, transW, relu, mask is not None)
+            Xn = X.clone()
+            Xn[7, 100] = float("inf")
+            Xn[n - 3, 5] = float("nan")
+            Y = torch.empty(n, 128, device="cuda")
+            _capi.check(L.psp_gemm_xw_act_f32(p(Xn), p(W), p(Y), n, 128, 128, 0, 0, None, st))
+            bad = (~torch.isfinite(Y)).any(dim=1)
+            assert bool(bad[7]) and bool(bad[n - 3]) and int(bad.sum()) == 2
+    finally:
+        _capi.check(L.psp_set_option(b"dense_split", 1))
+    assert L.psp_set_option(b"dense_split", 2) == -1
+
+
 @pytest.mark.parametrize("vec_size", [2, 3])
 def test_sddmm_sweep_harness(tmp_path, vec_size):
     """SDDMM.py's facade and sweep (SDDMM.py:46-383) on the reference's pubmed pattern read from a .mtx file and on a
