@@ -94,9 +94,9 @@ int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan);
  *                      order, which is the summation order of the reference's one-warp-per-row kernels
  *                      (SpMM/SpMM_kernel.cu:1157-1212, 1362-1440): results repeat the sequential chain bit for bit.
  *                      Default 0: rows may be cut between lane groups and summed piecewise (faster on skewed rows).
- *   "dense_split"      1 (default): psp_gemm_xw(_act)_f32 at 128 x 128 forms every fp32 product from the three bf16
+ *   "dense_split"      1 (default): psp_gemm_xw(_act)_f32 and psp_gemm_atb(_ws)(_act)_f32 at 128 x 128 form every fp32 product from the three bf16
  *                      terms of each operand (six bf16 matrix-core products, fp32 accumulation: error 2^-23 of |x||w|
- *                      per product, the rounding level of fp32) and is bound by its memory traffic; an infinite input
+ *                      per product, the rounding level of fp32) and are bound by their memory traffic; an infinite input
  *                      turns its row into NaN.  0: the fp32 matrix-core instruction, 25-40 % slower at that shape.
  * The environment (PSP_XCD_STRIPE_ROWS, PSP_ALIGN_PCT, PSP_SPLIT_CLEAR_MIN, PSP_WHOLE_ROWS, PSP_DENSE_SPLIT) sets the
  * initial values, once.

@@ -232,6 +232,141 @@ psp_atb_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B, fl
     }
 }
 
+// The 128 x 128 product on the bf16 matrix-core path (option dense_split).  At that shape the fp32 instruction above
+// needs as long for its flops as the memory system needs for the two operands; with every fp32 operand taken apart
+// into its three bf16 terms (exact: 8 + 8 + 8 significant bits) and the six term products that matter (error 2^-23 of
+// |a||b| per product) accumulated in fp32 by v_mfma_f32_16x16x32_bf16, the kernel is bound by its traffic again.
+// The instruction contracts 32 rows; operand lane (c, kk) = (lane % 16, lane / 16) supplies eight of them, rows
+// 8 kk + i of the chunk, for output index c.  A lane loads, from each of its eight rows, two float4 of A (columns
+// 64 t + 4 c ..: tile 4 t + e takes element e) and one float2 of its wavefront's quarter of B (columns col0 + 2 c + q:
+// tile q), so one load instruction covers 256 (128) contiguous bytes of four rows.  The four wavefronts of a workgroup
+// share a chunk and own a quarter of B's columns each, as in the JSPLIT = 4 form above.  Rows past n enter as zeros.
+typedef __bf16 psp_bf16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 psp_bf16x8 __attribute__((ext_vector_type(8)));
+typedef unsigned int psp_u32x4 __attribute__((ext_vector_type(4)));
+
+// two floats -> their three bf16 terms, packed in pairs (low half = first float)
+__device__ __forceinline__ void psp_atb_split3(float a, float b, unsigned &hi, unsigned &mid, unsigned &lo)
+{
+    psp_f32x2 v = {a, b};
+    hi = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
+    v[0] = a - __uint_as_float(hi << 16);
+    v[1] = b - __uint_as_float(hi & 0xffff0000u);
+    mid = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
+    v[0] -= __uint_as_float(mid << 16);
+    v[1] -= __uint_as_float(mid & 0xffff0000u);
+    lo = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
+}
+
+#define ATB_SPLIT_WGS 256  // one workgroup per CU (the kernel's 410 registers allow no more): as many partial products to add
+
+template <bool RELU_A>
+__global__ void __launch_bounds__(256)
+psp_atb_split_kernel(const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, long long n,
+                     float *__restrict__ partial)
+{
+    constexpr int K1 = 128, K2 = 128, RM = 8, RNW = 2;
+    const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const int kk = lane >> 4, c = lane & 15;
+    const int col0 = w * 32;
+    psp_mfma_acc acc[RM][RNW];
+#pragma unroll
+    for (int m = 0; m < RM; m++)
+#pragma unroll
+        for (int q = 0; q < RNW; q++) acc[m][q] = psp_mfma_acc{0.f, 0.f, 0.f, 0.f};
+
+    const long long chunks = (n + 31) >> 5;
+    psp_f32x4 a0[8][2], a1[8][2];
+    psp_f32x2 b0[8], b1[8];
+    // unconditional loads from clamped rows; what lies past n is cleared where it is used
+    auto fetch = [&](long long ch, psp_f32x4 (&fa)[8][2], psp_f32x2 (&fb)[8]) {
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            long long row = ch * 32 + 8 * kk + i;
+            row = row < n ? row : n - 1;
+            fa[i][0] = *(const psp_f32x4 *)(A + row * K1 + 4 * c);
+            fa[i][1] = *(const psp_f32x4 *)(A + row * K1 + 64 + 4 * c);
+            fb[i] = *(const psp_f32x2 *)(B + row * K2 + col0 + 2 * c);
+        }
+    };
+    auto multiply = [&](long long ch, psp_f32x4 (&fa)[8][2], psp_f32x2 (&fb)[8]) {
+        if (ch * 32 + 32 > n) {  // the last chunk of the matrix
+#pragma unroll
+            for (int i = 0; i < 8; i++)
+                if (ch * 32 + 8 * kk + i >= n) {
+                    fa[i][0] = fa[i][1] = psp_f32x4{0.f, 0.f, 0.f, 0.f};
+                    fb[i] = psp_f32x2{0.f, 0.f};
+                }
+        }
+        psp_u32x4 bh[RNW], bm[RNW], bl[RNW];
+#pragma unroll
+        for (int q = 0; q < RNW; q++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                unsigned h_, m_, l_;
+                psp_atb_split3(fb[2 * g][q], fb[2 * g + 1][q], h_, m_, l_);
+                bh[q][g] = h_, bm[q][g] = m_, bl[q][g] = l_;
+            }
+#pragma unroll
+        for (int m = 0; m < RM; m++) {
+            psp_u32x4 ah, am, al;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                float x = fa[2 * g][m >> 2][m & 3], y = fa[2 * g + 1][m >> 2][m & 3];
+                if constexpr (RELU_A) {
+                    x = x < 0.0f ? 0.0f : x;
+                    y = y < 0.0f ? 0.0f : y;
+                }
+                unsigned h_, m_, l_;
+                psp_atb_split3(x, y, h_, m_, l_);
+                ah[g] = h_, am[g] = m_, al[g] = l_;
+            }
+            // small terms first; the two column tiles alternate, so no instruction waits for the one before it
+#define ATBS_TERM(AV_, BV_)                                                                                            \
+    _Pragma("unroll") for (int q = 0; q < RNW; q++) acc[m][q] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(               \
+        __builtin_bit_cast(psp_bf16x8, AV_), __builtin_bit_cast(psp_bf16x8, BV_[q]), acc[m][q], 0, 0, 0);
+            ATBS_TERM(al, bh)
+            ATBS_TERM(ah, bl)
+            ATBS_TERM(am, bm)
+            ATBS_TERM(am, bh)
+            ATBS_TERM(ah, bm)
+            ATBS_TERM(ah, bh)
+#undef ATBS_TERM
+        }
+    };
+    long long ch = blockIdx.x;
+    const long long step = gridDim.x;
+    if (ch < chunks) {
+        fetch(ch, a0, b0);
+        while (true) {
+            long long nxt = ch + step;
+            if (nxt < chunks) fetch(nxt, a1, b1);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(ch, a0, b0);
+            if (nxt >= chunks) break;
+            ch = nxt;
+            nxt = ch + step;
+            if (nxt < chunks) fetch(nxt, a0, b0);
+            __builtin_amdgcn_sched_barrier(0);
+            multiply(ch, a1, b1);
+            if (nxt >= chunks) break;
+            ch = nxt;
+        }
+    }
+    // accumulator register v of lane (c, kk), tile (m, q) is C[64 (m / 4) + 4 (4 kk + v) + m % 4][col0 + 2 c + q]
+    float *dst = partial ? partial + (size_t)blockIdx.x * (K1 * K2) : C;
+#pragma unroll
+    for (int m = 0; m < RM; m++)
+#pragma unroll
+        for (int q = 0; q < RNW; q++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                float *d = &dst[(64 * (m >> 2) + 4 * (4 * kk + v) + (m & 3)) * K2 + col0 + 2 * c + q];
+                if (partial) *d = acc[m][q][v];
+                else unsafeAtomicAdd(d, acc[m][q][v]);
+            }
+}
+
 // C[e] = sum over the P workgroup slots of partial[p][e].  A workgroup of 1024 lanes takes 16 elements; lane t adds the
 // slots t / 16, t / 16 + 64, ... of element t % 16 (all loads independent, so one memory latency covers them), then
 // the 64 sums of an element meet in LDS.
@@ -314,7 +449,11 @@ static int atb_atomic(const float *A, const float *B, float *C, long long n, int
     if (rc != PSP_OK || n == 0) return rc;
     int jsplit = 1;
     if (psp_atb_mfma_kernel_t km = atb_mfma_lookup(K1, K2, &jsplit, relu_a)) {
-        const long long wgs = atb_mfma_grid(n, jsplit, K1 * K2);
+        long long wgs = atb_mfma_grid(n, jsplit, K1 * K2);
+        if (K1 == 128 && K2 == 128 && psp_opts().dense_split) {
+            km = relu_a ? psp_atb_split_kernel<true> : psp_atb_split_kernel<false>;
+            wgs = wgs < ATB_SPLIT_WGS ? wgs : ATB_SPLIT_WGS;
+        }
         hipLaunchKernelGGL(km, dim3((unsigned)wgs), dim3(256), 0, stream, A, B, C, n, (float *)nullptr);
         return psp_check_launch("gemm_atb mfma kernel");
     }
@@ -348,9 +487,13 @@ PSP_EXPORT int psp_gemm_atb_ws_act_f32(const float *A, const float *B, float *C,
     psp_atb_mfma_kernel_t km = atb_mfma_lookup(K1, K2, &jsplit, relu_a != 0);
     if (!km || n <= 0) return atb_atomic(A, B, C, n, K1, K2, relu_a != 0, (hipStream_t)stream);  // shapes of the LDS-tiled kernel; n = 0
     PSP_REQUIRE(A && B && C, "gemm_atb_ws: null pointer");
-    const long long wgs = atb_mfma_grid(n, jsplit, K1 * K2);
+    long long wgs = atb_mfma_grid(n, jsplit, K1 * K2);
     PSP_REQUIRE(workspace && workspace_floats >= wgs * K1 * K2, "gemm_atb_ws: the workspace holds %lld floats, %lld needed",
                 workspace_floats, wgs * K1 * K2);
+    if (K1 == 128 && K2 == 128 && psp_opts().dense_split) {
+        km = relu_a ? psp_atb_split_kernel<true> : psp_atb_split_kernel<false>;
+        wgs = wgs < ATB_SPLIT_WGS ? wgs : ATB_SPLIT_WGS;  // (uses the first slots of the workspace)
+    }
     hipStream_t st = (hipStream_t)stream;
     hipLaunchKernelGGL(km, dim3((unsigned)wgs), dim3(256), 0, st, A, B, C, n, workspace);
     int rc = psp_check_launch("gemm_atb mfma kernel");
