@@ -94,10 +94,11 @@ int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan);
  *                      order, which is the summation order of the reference's one-warp-per-row kernels
  *                      (SpMM/SpMM_kernel.cu:1157-1212, 1362-1440): results repeat the sequential chain bit for bit.
  *                      Default 0: rows may be cut between lane groups and summed piecewise (faster on skewed rows).
- *   "dense_split"      1 (default): psp_gemm_xw(_act)_f32 and psp_gemm_atb(_ws)(_act)_f32 at 128 x 128 form every fp32 product from the three bf16
- *                      terms of each operand (six bf16 matrix-core products, fp32 accumulation: error 2^-23 of |x||w|
- *                      per product, the rounding level of fp32) and are bound by their memory traffic; an infinite input
- *                      turns its row into NaN.  0: the fp32 matrix-core instruction, 25-40 % slower at that shape.
+ *   "dense_split"      1 (default): the dense layer products (the gemm_xw and gemm_atb entry points) at 128 x 128 form
+ *                      every fp32 product from the three bf16 terms of each operand (six bf16 matrix-core products,
+ *                      fp32 accumulation: error 2^-23 of |x||w| per product, the rounding level of fp32) and are
+ *                      bound by their memory traffic; an infinite input turns its row into NaN.  0: the fp32
+ *                      matrix-core instruction, 25-40 % slower at that shape.
  * The environment (PSP_XCD_STRIPE_ROWS, PSP_ALIGN_PCT, PSP_SPLIT_CLEAR_MIN, PSP_WHOLE_ROWS, PSP_DENSE_SPLIT) sets the
  * initial values, once.
  * psp_get_option returns the value, or a negative psp_status for an unknown name.  Not synchronised with running
@@ -318,7 +319,7 @@ int psp_sddmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b, const flo
  * (local entries are summed before remote ones), they are not bit-identical to it.
  * ------------------------------------------------------------------------------------------- */
 #define PSP_WINDOW_BLOCK 64
-#define PSP_WINDOW_HALO 64
+#define PSP_WINDOW_HALO 88
 int psp_window_build(const int *rowPtr, const int *colIdx, const float *val, int M, int *rowPtr_w, int *colIdx_w,
                      float *val_w);
 int psp_window_build_dev(const int *rowPtr, const int *colIdx, const float *val, int M, int *rowPtr_w, int *colIdx_w,

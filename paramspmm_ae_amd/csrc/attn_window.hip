@@ -34,7 +34,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
     constexpr int V4 = TN / 4;
     constexpr int FPT = RB * V4 / THREADS;
     static_assert(RB * L == THREADS, "one row of the block per lane group");
-    static_assert(RB * V4 % THREADS == 0 && (RING & (RING - 1)) == 0 && UR <= L && UR == 4, "shape");
+    static_assert(RB * V4 % THREADS == 0 && UR <= L && UR == 4, "shape");
     extern __shared__ __align__(16) float s_x[];  // [RING + 1][TN]: the ring and a row of zeros
     constexpr int ZERO_OFF = RING * TN * 4;
     __shared__ float s_part[THREADS / 64];
@@ -95,7 +95,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         for (int i = 0; i < FPT; i++) {
             const int q = i * THREADS + tid;
             const int wr = q / V4, c4 = q - wr * V4;
-            *(psp_f32x4 *)(s_x + (((first + wr + RING) & (RING - 1)) * TN + c4 * 4)) = w[i];
+            *(psp_f32x4 *)(s_x + (pspw_slot<RING>(first + wr) * TN + c4 * 4)) = w[i];
         }
     };
     auto gather_remote = [&](int cr, psp_f32x4(&xr)[UR][C]) {
@@ -116,7 +116,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
                 cf[t] = ok ? (float)cl[t] : 0.0f;
                 vl[t] = ok ? vl[t] : 0.0f;
             }
-            cl[t] = ok ? ((cl[t] + RING) & (RING - 1)) * (TN * 4) : ZERO_OFF;
+            cl[t] = ok ? pspw_slot<RING>(cl[t]) * (TN * 4) : ZERO_OFF;
         }
     };
     auto dot = [&](const psp_f32x4(&x)[C], const psp_f32x4(&ar)[C]) {
@@ -143,7 +143,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
     load_bounds(j0, a, m, b);
     load_bounds(j0 + 1, an, mn, bn);
 #pragma unroll 1
-    for (int piece = 0; piece < 3; piece++) {
+    for (int piece = 0; piece < PSPW_FIRST_PIECES; piece++) {
         fill_load(j0 * RB - PSPW_HALO + piece * RB, w);
         fill_store(j0 * RB - PSPW_HALO + piece * RB, w);
     }
@@ -161,7 +161,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         const int r = j * RB + grp;
         {
             // the group's own row (a row past the matrix has no entries; its slot holds the nearest valid row)
-            const int slot = (r & (RING - 1)) * TN;
+            const int slot = pspw_slot<RING>(r) * TN;
 #pragma unroll
             for (int i = 0; i < C; i++) {
                 ar[i] = *(const psp_f32x4 *)(s_x + slot + off[i]);
@@ -216,7 +216,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         // local entries beyond the ones fetched up front
         for (int p = a + T * L; p < m; p++) {
             const int c_ = colIdx[p];
-            const int slot = ((c_ + RING) & (RING - 1)) * TN;
+            const int slot = pspw_slot<RING>(c_) * TN;
             psp_f32x4 x_[C];
 #pragma unroll
             for (int i = 0; i < C; i++) x_[i] = *(const psp_f32x4 *)(s_x + (slot + off[i]));

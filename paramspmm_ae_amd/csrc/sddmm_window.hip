@@ -32,7 +32,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
     constexpr int V4 = TN / 4;                     // 16-byte pieces per window row
     constexpr int FPT = RB * V4 / THREADS;         // pieces per lane when 64 rows enter
     static_assert(RB * L == THREADS, "one row of the block per lane group");
-    static_assert(RB * V4 % THREADS == 0 && (RING & (RING - 1)) == 0 && UR <= L && UR == 4, "shape");
+    static_assert(RB * V4 % THREADS == 0 && UR <= L && UR == 4, "shape");
     // [RING + 1][TN]: the ring and a row of zeros for the padding of a row's entry registers
     extern __shared__ __align__(16) float s_x[];
     constexpr int ZERO_OFF = RING * TN * 4;
@@ -85,7 +85,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
         for (int i = 0; i < FPT; i++) {
             const int q = i * THREADS + tid;
             const int wr = q / V4, c4 = q - wr * V4;
-            *(psp_f32x4 *)(s_x + (((first + wr + RING) & (RING - 1)) * TN + c4 * 4)) = w[i];
+            *(psp_f32x4 *)(s_x + (pspw_slot<RING>(first + wr) * TN + c4 * 4)) = w[i];
         }
     };
     auto gather_remote = [&](int cr, psp_f32x4(&xr)[UR][C]) {
@@ -104,7 +104,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
     // local columns -> byte offsets of the B rows in the ring (the zero row for a slot past the row's local part)
     auto to_ring = [&](int a, int m, int(&cl)[T]) {
 #pragma unroll
-        for (int t = 0; t < T; t++) cl[t] = a + t * L + sub < m ? ((cl[t] + RING) & (RING - 1)) * (TN * 4) : ZERO_OFF;
+        for (int t = 0; t < T; t++) cl[t] = a + t * L + sub < m ? pspw_slot<RING>(cl[t]) * (TN * 4) : ZERO_OFF;
     };
     auto dot = [&](const psp_f32x4(&x)[C], const psp_f32x4(&ar)[C]) {
         float s = 0.0f;
@@ -123,7 +123,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
     load_bounds(j0, a, m, b);
     load_bounds(j0 + 1, an, mn, bn);
 #pragma unroll 1
-    for (int piece = 0; piece < 3; piece++) {
+    for (int piece = 0; piece < PSPW_FIRST_PIECES; piece++) {
         fill_load(j0 * RB - PSPW_HALO + piece * RB, w);
         fill_store(j0 * RB - PSPW_HALO + piece * RB, w);
     }
@@ -141,7 +141,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
         fill_load((j + 1) * RB + PSPW_HALO, w);  // the rows that enter with block j + 1
         if constexpr (SAME) {
             // (a row past the matrix has no entries; its slot holds the nearest valid row)
-            const int slot = ((j * RB + grp) & (RING - 1)) * TN;
+            const int slot = pspw_slot<RING>(j * RB + grp) * TN;
 #pragma unroll
             for (int i = 0; i < C; i++) ar[i] = *(const psp_f32x4 *)(s_x + slot + off[i]);
         } else {
@@ -185,7 +185,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
 #undef PSPW_DOT
         // local entries beyond the ones fetched up front
         for (int p = a + T * L; p < m; p++) {
-            const int c_ = (colIdx[p] + RING) & (RING - 1);
+            const int c_ = pspw_slot<RING>(colIdx[p]);
             psp_f32x4 x_[C];
 #pragma unroll
             for (int i = 0; i < C; i++) x_[i] = *(const psp_f32x4 *)(s_x + (c_ * TN + off[i]));

@@ -5,16 +5,17 @@
 // sparse rows gather as well.
 //
 // Format (psp_window_build / psp_window_build_dev).  The rows are cut into blocks of PSP_WINDOW_BLOCK = 64; the
-// window of a block is the row range [64 b - 64, 64 b + 128), i.e. the block and PSP_WINDOW_HALO = 64 rows either
-// side.  An entry is *local* when its column lies inside its row's window.  Every row keeps its entries, local ones
+// window of a block is the row range [64 b - 88, 64 b + 152), i.e. the block and PSP_WINDOW_HALO = 88 rows either
+// side (the widest halo with which two workgroups of the 64-column variant still share a CU's 160 KB of LDS: every
+// remote entry costs a gather of its own and, past the few whose rows are prefetched, a wait).  An entry is *local* when its column lies inside its row's window.  Every row keeps its entries, local ones
 // first (each part in the original order), and rowPtr_w[2M + 2] holds for row i the start of the row at 2i and the
 // start of its remote part at 2i + 1; entries 2M and 2M + 1 hold nnz.  Columns stay absolute, so any CSR kernel can
 // read (rowPtr_w[0::2], colIdx_w, val_w) as an ordinary matrix with unsorted rows.
 //
 // Kernel.  A workgroup of 256 lanes walks a run of consecutive 64-row blocks for one column tile of TN = 16 / 32 / 64
-// floats.  The X rows of the current block's window sit in LDS in a ring of 256 rows (row g in slot (g + 256) % 256):
-// the windows of neighbouring blocks overlap by 128 rows, so a step to the next block loads only the 64 rows that
-// enter -- and they land in the slots of the 64 rows that the block after next no longer needs, so the ring never
+// floats.  The X rows of the current block's window sit in LDS in a ring of 64 + 2 * 88 + 64 = 304 rows (row g in slot
+// g mod 304): the windows of neighbouring blocks differ by 64 rows, so a step to the next block loads only the 64 rows
+// that enter -- and they land in the slots of the 64 rows that the block after next no longer needs, so the ring never
 // overwrites a row that is still being read and one barrier per block is enough.  A lane group of L = 4 or 8 lanes
 // owns L / 4 rows of a block.  The walk is software-pipelined, so that after the first block of a run no lane waits for
 // a load it has just issued: while block j is summed from LDS, the loads in flight are
@@ -58,7 +59,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
     constexpr int UR = PSPW_UR;
     constexpr int V4 = TN / 4;                     // 16-byte pieces per window row
     constexpr int FPT = RB * V4 / PSPW_THREADS;    // pieces per lane when 64 rows enter
-    static_assert(RPG >= 1 && RB * V4 % PSPW_THREADS == 0 && (RING & (RING - 1)) == 0, "shape");
+    static_assert(RPG >= 1 && RB * V4 % PSPW_THREADS == 0, "shape");
     static_assert(UR <= L, "one lane per prefetched remote entry");
     // [RING + 1][TN]: the ring and one row of zeros, which the padding of a row's entry registers points at (value 0
     // times a zero, so the summing loop needs no predicate and a padding slot can never bring an Inf or NaN in)
@@ -145,7 +146,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
 #pragma unroll
                 for (int e = 0; e < 4; e++) w[i][e] = w[i][e] < 0.0f ? 0.0f : w[i][e];
             }
-            *(psp_f32x4 *)(s_x + (((first + wr + RING) & (RING - 1)) * TN + c4 * 4)) = w[i];
+            *(psp_f32x4 *)(s_x + (pspw_slot<RING>(first + wr) * TN + c4 * 4)) = w[i];
         }
     };
     auto gather_remote = [&](const int(&cr)[RPG], psp_f32x4(&xr)[RPG][UR][C]) {
@@ -169,7 +170,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
 #pragma unroll
             for (int t = 0; t < T; t++) {
                 const bool ok = a[k] + t * L + sub < m[k];
-                cl[k][t] = ok ? ((cl[k][t] + RING) & (RING - 1)) * (TN * 4) : ZERO_OFF;
+                cl[k][t] = ok ? pspw_slot<RING>(cl[k][t]) * (TN * 4) : ZERO_OFF;
                 vl[k][t] = ok ? vl[k][t] : 0.0f;
             }
     };
@@ -183,7 +184,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
     load_bounds(j0, a, m, b);
     load_bounds(j0 + 1, an, mn, bn);
 #pragma unroll 1
-    for (int piece = 0; piece < 3; piece++) {
+    for (int piece = 0; piece < PSPW_FIRST_PIECES; piece++) {
         fill_load(j0 * RB - PSPW_HALO + piece * RB, w);
         fill_store(j0 * RB - PSPW_HALO + piece * RB, w);
     }
@@ -239,7 +240,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
             }
             // local entries beyond the ones fetched up front
             for (int p = a[k] + T * L; p < m[k]; p++) {
-                const int c_ = (colIdx[p] + RING) & (RING - 1);
+                const int c_ = pspw_slot<RING>(colIdx[p]);
                 const float v_ = val[p];
 #pragma unroll
                 for (int i = 0; i < C; i++) {

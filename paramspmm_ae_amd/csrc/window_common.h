@@ -8,8 +8,13 @@ typedef float psp_f32x4 __attribute__((ext_vector_type(4)));
 
 #define PSPW_BLOCK PSP_WINDOW_BLOCK
 #define PSPW_HALO PSP_WINDOW_HALO
+// pieces of PSPW_BLOCK rows that cover a block's whole window (loaded before the first block of a run)
+#define PSPW_FIRST_PIECES ((PSPW_BLOCK + 2 * PSPW_HALO + PSPW_BLOCK - 1) / PSPW_BLOCK)
 #define PSPW_UR 4        // remote entries per row whose X tiles are prefetched into registers
 #define PSPW_LOCAL 32    // local entries per row fetched up front (T = 32 / L chunks)
+
+// slot of matrix row g (>= -PSPW_HALO) in a ring of RING rows
+template <int RING> __device__ __forceinline__ int pspw_slot(int g) { return (int)((unsigned)(g + RING) % (unsigned)RING); }
 
 // value of lane j of the caller's lane group (L = 4 or 8 consecutive lanes), j a compile-time constant: DPP moves on
 // the vector ALU, which this kernel leaves idle, instead of ds_bpermute on the LDS pipeline, which it keeps busy

@@ -105,7 +105,7 @@ class csr_data(object):
 
     def window_format(self, device="cuda"):
         """(rowPtr_w, colIdx_w, val_w, local share) of this CSR matrix in the windowed layout of the library
-        (psp_window_build: every row's entries reordered so that the ones whose column lies within 64 rows of the
+        (psp_window_build: every row's entries reordered so that the ones whose column lies within PSP_WINDOW_HALO rows of the
         row's 64-row block come first), built on ``device`` once and kept.  No counterpart in the reference; the
         CSR arrays must be the plain (vec_size 1) ones."""
         import ParamSpMM

@@ -10,7 +10,7 @@ import torch
 
 from conftest import random_csr
 
-BLOCK, HALO = 64, 64
+BLOCK, HALO = 64, 88
 
 
 def banded_csr(n, per_row, width, seed, far=0.0, hub=None, empty_frac=0.0):
