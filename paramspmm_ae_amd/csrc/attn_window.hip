@@ -31,6 +31,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
     constexpr int RING = RB + 2 * PSPW_HALO + RB;
     constexpr int T = PSPW_LOCAL / L;
     constexpr int UR = PSPW_UR;
+    constexpr int REM = L == 8 ? 2 * UR : UR;      // remote entries per row whose pairs sit in registers (entry e in lane e)
     constexpr int V4 = TN / 4;
     constexpr int FPT = RB * V4 / THREADS;
     static_assert(RB * L == THREADS, "one row of the block per lane group");
@@ -69,7 +70,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         m = am.y;
         b = rp2[min(r + 1, M)].x;
     };
-    // lane s takes the row's local entries a + tL + s (t < T) and, s < UR, remote entry m + s
+    // lane s takes the row's local entries a + tL + s (t < T) and remote entry m + s
     auto load_entries = [&](int a, int m, int(&cl)[T], float(&vl)[T], int &cr, float &vr) {
 #pragma unroll
         for (int t = 0; t < T; t++) {
@@ -77,7 +78,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
             cl[t] = colIdx[p];
             if constexpr (BWD) vl[t] = att_in[p];
         }
-        const int p = min(m + (sub & (UR - 1)), nnz - 1);
+        const int p = min(m + sub, nnz - 1);  // remote entry e in lane e
         cr = colIdx[p];
         if constexpr (BWD) vr = att_in[p];
     };
@@ -98,10 +99,10 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
             *(psp_f32x4 *)(s_x + (pspw_slot<RING>(first + wr) * TN + c4 * 4)) = w[i];
         }
     };
-    auto gather_remote = [&](int cr, psp_f32x4(&xr)[UR][C]) {
+    auto gather_remote = [&](int cr, int first, psp_f32x4(&xr)[UR][C]) {
 #pragma unroll
         for (int u = 0; u < UR; u++) {
-            const int c = pspw_bcast_u<L>(cr, u, sub);
+            const int c = pspw_remote<L>(cr, first + u, sub);
 #pragma unroll
             for (int i = 0; i < C; i++) xr[u][i] = *(const psp_f32x4 *)(X + (size_t)c * (size_t)K + min(off[i], K - 4));
         }
@@ -148,7 +149,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         fill_store(j0 * RB - PSPW_HALO + piece * RB, w);
     }
     load_entries(a, m, cl, vl, cr, vr);
-    gather_remote(cr, xr);
+    gather_remote(cr, 0, xr);
     to_ring(a, m, cl, vl, cf);
     __syncthreads();
 
@@ -232,23 +233,35 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         }
 
         // ---- remote entries ----------------------------------------------------------------------------------------------
+        // first round: entries 0 .. 3, whose rows were gathered while the previous block was processed; second round:
+        // entries 4 .. 7 of lane groups of 8 (columns already in lanes 4 .. 7), gathered together when some row of the
+        // wavefront has that many
+        auto remote_round = [&](int first, const psp_f32x4(&x)[UR][C]) {
 #pragma unroll
-        for (int u = 0; u < UR; u++) {
-            // (the moves between lanes stay outside the branch: every lane of the group takes part in them)
-            const float vu = BWD ? __int_as_float(pspw_bcast_u<L>(__float_as_int(vr), u, sub)) : 0.0f;
-            float s_ = pspw_reduce_all<L>(dot(xr[u], ar));
-            if (m + u < b) {
-                if constexpr (BWD) {
-                    if (sub == u) wsum = __builtin_fmaf(s_, (float)cr, wsum);
-                    axpy(vu, xr[u], acc);
-                } else {
-                    s_ *= alpha;
-                    if (sub == u) att_out[m + u] = s_;
-                    axpy(s_, xr[u], acc);
+            for (int u = 0; u < UR; u++) {
+                // (the moves between lanes stay outside the branch: every lane of the group takes part in them)
+                const int e = first + u;
+                const float vu = BWD ? pspw_remote_f<L>(vr, e, sub) : 0.0f;
+                float s_ = pspw_reduce_all<L>(dot(x[u], ar));
+                if (m + e < b) {
+                    if constexpr (BWD) {
+                        if (sub == e) wsum = __builtin_fmaf(s_, (float)cr, wsum);
+                        axpy(vu, x[u], acc);
+                    } else {
+                        s_ *= alpha;
+                        if (sub == e) att_out[m + e] = s_;
+                        axpy(s_, x[u], acc);
+                    }
                 }
             }
+        };
+        remote_round(0, xr);
+        if (REM > UR && __builtin_amdgcn_ballot_w64(m + UR < b) != 0ull) {
+            psp_f32x4 x2[UR][C];
+            gather_remote(cr, UR, x2);
+            remote_round(UR, x2);
         }
-        for (int p = m + UR; p < b; p++) {
+        for (int p = m + REM; p < b; p++) {
             const int c_ = colIdx[p];
             psp_f32x4 x_[C];
 #pragma unroll
@@ -270,7 +283,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         }
 
         // ---- hand over to block j + 1 ---------------------------------------------------------------------------------
-        gather_remote(crn, xr);                     // in flight while block j + 1 is processed
+        gather_remote(crn, 0, xr);                     // in flight while block j + 1 is processed
         fill_store((j + 1) * RB + PSPW_HALO, w);    // slots no row of block j's or j + 1's window occupies
         a = an, m = mn, b = bn;
         an = a2, mn = m2, bn = b2;

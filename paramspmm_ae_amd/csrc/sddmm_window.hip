@@ -29,6 +29,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
     constexpr int RING = RB + 2 * PSPW_HALO + RB;  // window + the rows that enter with the next block
     constexpr int T = PSPW_LOCAL / L;
     constexpr int UR = PSPW_UR;
+    constexpr int REM = L == 8 ? 2 * UR : UR;      // remote entries per row whose pairs sit in registers (entry e in lane e)
     constexpr int V4 = TN / 4;                     // 16-byte pieces per window row
     constexpr int FPT = RB * V4 / THREADS;         // pieces per lane when 64 rows enter
     static_assert(RB * L == THREADS, "one row of the block per lane group");
@@ -65,11 +66,11 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
         m = am.y;
         b = rp2[min(r + 1, M)].x;
     };
-    // lane s takes the row's local entries a + tL + s (t < T) and, s < UR, remote entry m + s
+    // lane s takes the row's local entries a + tL + s (t < T) and remote entry m + s
     auto load_cols = [&](int a, int m, int(&cl)[T], int &cr) {
 #pragma unroll
         for (int t = 0; t < T; t++) cl[t] = colIdx[min(a + t * L + sub, nnz - 1)];
-        cr = colIdx[min(m + (sub & (UR - 1)), nnz - 1)];
+        cr = colIdx[min(m + sub, nnz - 1)];  // remote entry e in lane e
     };
     auto fill_load = [&](int first, psp_f32x4(&w)[FPT]) {
 #pragma unroll
@@ -88,10 +89,10 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
             *(psp_f32x4 *)(s_x + (pspw_slot<RING>(first + wr) * TN + c4 * 4)) = w[i];
         }
     };
-    auto gather_remote = [&](int cr, psp_f32x4(&xr)[UR][C]) {
+    auto gather_remote = [&](int cr, int first, psp_f32x4(&xr)[UR][C]) {
 #pragma unroll
         for (int u = 0; u < UR; u++) {
-            const int c = pspw_bcast_u<L>(cr, u, sub);
+            const int c = pspw_remote<L>(cr, first + u, sub);
 #pragma unroll
             for (int i = 0; i < C; i++) xr[u][i] = *(const psp_f32x4 *)(B + (size_t)c * (size_t)K + min(off[i], K - 4));
         }
@@ -128,7 +129,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
         fill_store(j0 * RB - PSPW_HALO + piece * RB, w);
     }
     load_cols(a, m, cl, cr);
-    gather_remote(cr, xr);
+    gather_remote(cr, 0, xr);
     if constexpr (!SAME) load_row(j0, arn);
     to_ring(a, m, cl);
     __syncthreads();
@@ -202,7 +203,19 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
             const int p = m + sub;
             if (sub < UR && p < b) out[p] = alpha * r;
         }
-        for (int p = m + UR; p < b; p++) {
+        // second round (lane groups of 8): remote entries 4 .. 7 (columns already in lanes 4 .. 7), gathered together
+        // when some row of the wavefront has that many
+        if (REM > UR && __builtin_amdgcn_ballot_w64(m + UR < b) != 0ull) {
+            psp_f32x4 x2[UR][C];
+            gather_remote(cr, UR, x2);
+            float part[UR];
+#pragma unroll
+            for (int u = 0; u < UR; u++) part[u] = dot(x2[u], ar);
+            const float r = pspw_reduce_transposed4<L>(part, sub);
+            const int p = m + UR + sub;
+            if (sub < UR && p < b) out[p] = alpha * r;
+        }
+        for (int p = m + REM; p < b; p++) {
             const int c_ = colIdx[p];
             psp_f32x4 x_[C];
 #pragma unroll
@@ -212,7 +225,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
         }
 
         // ---- hand over to block j + 1 ---------------------------------------------------------------------------------
-        gather_remote(crn, xr);                     // in flight while block j + 1 is processed
+        gather_remote(crn, 0, xr);                     // in flight while block j + 1 is processed
         fill_store((j + 1) * RB + PSPW_HALO, w);    // slots no row of block j's or j + 1's window occupies
         a = an, m = mn, b = bn;
         an = a2, mn = m2, bn = b2;

@@ -57,6 +57,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
     constexpr int RING = RB + 2 * PSPW_HALO + RB;  // window + the rows that enter with the next block
     constexpr int T = PSPW_LOCAL / L;
     constexpr int UR = PSPW_UR;
+    constexpr int REM = L == 8 ? 2 * UR : UR;      // remote entries per row whose pairs sit in registers (entry e in lane e)
     constexpr int V4 = TN / 4;                     // 16-byte pieces per window row
     constexpr int FPT = RB * V4 / PSPW_THREADS;    // pieces per lane when 64 rows enter
     static_assert(RPG >= 1 && RB * V4 % PSPW_THREADS == 0, "shape");
@@ -110,7 +111,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
     // it is used.  A load under a condition would meet its "not loaded" value in a register copy right behind the
     // load, and the copy would wait for the load: the pipeline of this kernel lives on loads that stay in flight.
     //
-    // lane s takes the rows' local entries a + tL + s (t < T) and, s < UR, remote entry m + s
+    // lane s takes the rows' local entries a + tL + s (t < T) and remote entry m + s
     auto load_pairs = [&](const int(&a)[RPG], const int(&m)[RPG], int(&cl)[RPG][T], float(&vl)[RPG][T], int(&cr)[RPG],
                           float(&vr)[RPG]) {
 #pragma unroll
@@ -121,7 +122,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
                 cl[k][t] = colIdx[p];
                 vl[k][t] = val[p];
             }
-            const int p = min(m[k] + (sub & (UR - 1)), nnz - 1);
+            const int p = min(m[k] + sub, nnz - 1);  // remote entry e in lane e
             cr[k] = colIdx[p];
             vr[k] = val[p];
         }
@@ -154,7 +155,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         for (int k = 0; k < RPG; k++) {
 #pragma unroll
             for (int u = 0; u < UR; u++) {
-                const int c = pspw_bcast_u<L>(cr[k], u, sub);
+                const int c = pspw_remote<L>(cr[k], u, sub);
 #pragma unroll
                 for (int i = 0; i < C; i++)
                     xr[k][u][i] = *(const psp_f32x4 *)(X + (size_t)c * (size_t)N + min(tile_col0 + off[i], N - 4));
@@ -257,7 +258,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         for (int k = 0; k < RPG; k++) {
 #pragma unroll
             for (int u = 0; u < UR; u++) {
-                const float v = __int_as_float(pspw_bcast_u<L>(__float_as_int(vr[k]), u, sub));
+                const float v = pspw_remote_f<L>(vr[k], u, sub);
                 if (m[k] + u < b[k]) {
 #pragma unroll
                     for (int i = 0; i < C; i++) {
@@ -271,7 +272,38 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
                     }
                 }
             }
-            for (int p = m[k] + UR; p < b[k]; p++) {
+            // Second round (lane groups of 8): remote entries 4 .. 7, whose columns and values lanes 4 .. 7 already hold.
+            // Their X rows are gathered together, into the registers the first round has just left, only when some row of
+            // the wavefront has that many -- one wait instead of two dependent ones per entry in the loop below.
+            if constexpr (REM > UR) {
+                if (__builtin_amdgcn_ballot_w64(m[k] + UR < b[k]) != 0ull) {
+                    psp_f32x4 x2[UR][C];
+#pragma unroll
+                    for (int u = 0; u < UR; u++) {
+                        const int c = pspw_remote<L>(cr[k], UR + u, sub);
+#pragma unroll
+                        for (int i = 0; i < C; i++)
+                            x2[u][i] = *(const psp_f32x4 *)(X + (size_t)c * (size_t)N + min(tile_col0 + off[i], N - 4));
+                    }
+#pragma unroll
+                    for (int u = 0; u < UR; u++) {
+                        const float v = pspw_remote_f<L>(vr[k], UR + u, sub);
+                        if (m[k] + UR + u < b[k]) {
+#pragma unroll
+                            for (int i = 0; i < C; i++) {
+                                psp_f32x4 x_ = x2[u][i];
+                                if (relu_x) {
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) x_[e] = x_[e] < 0.0f ? 0.0f : x_[e];
+                                }
+#pragma unroll
+                                for (int e = 0; e < 4; e++) acc[k][i][e] = __builtin_fmaf(v, x_[e], acc[k][i][e]);
+                            }
+                        }
+                    }
+                }
+            }
+            for (int p = m[k] + REM; p < b[k]; p++) {
                 const int c_ = colIdx[p];
                 const float v_ = val[p];
 #pragma unroll

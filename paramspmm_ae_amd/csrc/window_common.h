@@ -43,6 +43,28 @@ template <int L> __device__ __forceinline__ int pspw_bcast_u(int x, int u, int s
     default: return pspw_bcast<L, 3>(x, sub);
     }
 }
+// A lane group keeps the (column, value) pairs of a row's first L remote entries in registers, entry e in lane e.  The X
+// rows of the first PSPW_UR = 4 are gathered a block ahead; groups of 8 lanes gather the other four together, in a
+// second round, when some row of the wavefront has that many.  (Groups of 4 lanes -- 16 rows per wavefront, of which
+// some row nearly always has a fifth entry -- were slower with a second round than with the plain loop.)
+// Entry e (a constant after unrolling) for every lane of the group:
+template <int L> __device__ __forceinline__ int pspw_remote(int x, int e, int sub)
+{
+    switch (e) {
+    case 0: return pspw_bcast<L, 0>(x, sub);
+    case 1: return pspw_bcast<L, 1>(x, sub);
+    case 2: return pspw_bcast<L, 2>(x, sub);
+    case 3: return pspw_bcast<L, 3>(x, sub);
+    case 4: return pspw_bcast<L, 4>(x, sub);
+    case 5: return pspw_bcast<L, 5>(x, sub);
+    case 6: return pspw_bcast<L, 6>(x, sub);
+    default: return pspw_bcast<L, 7>(x, sub);
+    }
+}
+template <int L> __device__ __forceinline__ float pspw_remote_f(float x, int e, int sub)
+{
+    return __int_as_float(pspw_remote<L>(__float_as_int(x), e, sub));
+}
 
 // the same for any lane of the group
 template <int L> __device__ __forceinline__ float pspw_bcast_any_f(float x, int j, int sub)
