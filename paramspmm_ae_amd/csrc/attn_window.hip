@@ -99,10 +99,12 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
             *(psp_f32x4 *)(s_x + (pspw_slot<RING>(first + wr) * TN + c4 * 4)) = w[i];
         }
     };
-    auto gather_remote = [&](int cr, int first, psp_f32x4(&xr)[UR][C]) {
+    // (a slot past the row's remote part reads row 0: the same address for every such lane of the wavefront, which the
+    // memory pipeline serves as one request, where the clamped column would cost a request of its own)
+    auto gather_remote = [&](int cr, int m, int b, int first, psp_f32x4(&xr)[UR][C]) {
 #pragma unroll
         for (int u = 0; u < UR; u++) {
-            const int c = pspw_remote<L>(cr, first + u, sub);
+            const int c = m + first + u < b ? pspw_remote<L>(cr, first + u, sub) : 0;
 #pragma unroll
             for (int i = 0; i < C; i++) xr[u][i] = *(const psp_f32x4 *)(X + (size_t)c * (size_t)K + min(off[i], K - 4));
         }
@@ -149,7 +151,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         fill_store(j0 * RB - PSPW_HALO + piece * RB, w);
     }
     load_entries(a, m, cl, vl, cr, vr);
-    gather_remote(cr, 0, xr);
+    gather_remote(cr, m, b, 0, xr);
     to_ring(a, m, cl, vl, cf);
     __syncthreads();
 
@@ -258,7 +260,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         remote_round(0, xr);
         if (REM > UR && __builtin_amdgcn_ballot_w64(m + UR < b) != 0ull) {
             psp_f32x4 x2[UR][C];
-            gather_remote(cr, UR, x2);
+            gather_remote(cr, m, b, UR, x2);
             remote_round(UR, x2);
         }
         for (int p = m + REM; p < b; p++) {
@@ -283,7 +285,7 @@ psp_attn_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         }
 
         // ---- hand over to block j + 1 ---------------------------------------------------------------------------------
-        gather_remote(crn, 0, xr);                     // in flight while block j + 1 is processed
+        gather_remote(crn, mn, bn, 0, xr);                     // in flight while block j + 1 is processed
         fill_store((j + 1) * RB + PSPW_HALO, w);    // slots no row of block j's or j + 1's window occupies
         a = an, m = mn, b = bn;
         an = a2, mn = m2, bn = b2;

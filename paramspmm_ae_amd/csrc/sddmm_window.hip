@@ -89,10 +89,12 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
             *(psp_f32x4 *)(s_x + (pspw_slot<RING>(first + wr) * TN + c4 * 4)) = w[i];
         }
     };
-    auto gather_remote = [&](int cr, int first, psp_f32x4(&xr)[UR][C]) {
+    // (a slot past the row's remote part reads row 0: the same address for every such lane of the wavefront, which the
+    // memory pipeline serves as one request, where the clamped column would cost a request of its own)
+    auto gather_remote = [&](int cr, int m, int b, int first, psp_f32x4(&xr)[UR][C]) {
 #pragma unroll
         for (int u = 0; u < UR; u++) {
-            const int c = pspw_remote<L>(cr, first + u, sub);
+            const int c = m + first + u < b ? pspw_remote<L>(cr, first + u, sub) : 0;
 #pragma unroll
             for (int i = 0; i < C; i++) xr[u][i] = *(const psp_f32x4 *)(B + (size_t)c * (size_t)K + min(off[i], K - 4));
         }
@@ -129,7 +131,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
         fill_store(j0 * RB - PSPW_HALO + piece * RB, w);
     }
     load_cols(a, m, cl, cr);
-    gather_remote(cr, 0, xr);
+    gather_remote(cr, m, b, 0, xr);
     if constexpr (!SAME) load_row(j0, arn);
     to_ring(a, m, cl);
     __syncthreads();
@@ -207,7 +209,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
         // when some row of the wavefront has that many
         if (REM > UR && __builtin_amdgcn_ballot_w64(m + UR < b) != 0ull) {
             psp_f32x4 x2[UR][C];
-            gather_remote(cr, UR, x2);
+            gather_remote(cr, m, b, UR, x2);
             float part[UR];
 #pragma unroll
             for (int u = 0; u < UR; u++) part[u] = dot(x2[u], ar);
@@ -225,7 +227,7 @@ psp_sddmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict_
         }
 
         // ---- hand over to block j + 1 ---------------------------------------------------------------------------------
-        gather_remote(crn, 0, xr);                     // in flight while block j + 1 is processed
+        gather_remote(crn, mn, bn, 0, xr);                     // in flight while block j + 1 is processed
         fill_store((j + 1) * RB + PSPW_HALO, w);    // slots no row of block j's or j + 1's window occupies
         a = an, m = mn, b = bn;
         an = a2, mn = m2, bn = b2;

@@ -150,12 +150,14 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
             *(psp_f32x4 *)(s_x + (pspw_slot<RING>(first + wr) * TN + c4 * 4)) = w[i];
         }
     };
-    auto gather_remote = [&](const int(&cr)[RPG], psp_f32x4(&xr)[RPG][UR][C]) {
+    // (a slot past the row's remote part reads row 0: the same address for every such lane of the wavefront, which the
+    // memory pipeline serves as one request, where the clamped column would cost a request of its own)
+    auto gather_remote = [&](const int(&cr)[RPG], const int(&m)[RPG], const int(&b)[RPG], psp_f32x4(&xr)[RPG][UR][C]) {
 #pragma unroll
         for (int k = 0; k < RPG; k++) {
 #pragma unroll
             for (int u = 0; u < UR; u++) {
-                const int c = pspw_remote<L>(cr[k], u, sub);
+                const int c = m[k] + u < b[k] ? pspw_remote<L>(cr[k], u, sub) : 0;
 #pragma unroll
                 for (int i = 0; i < C; i++)
                     xr[k][u][i] = *(const psp_f32x4 *)(X + (size_t)c * (size_t)N + min(tile_col0 + off[i], N - 4));
@@ -190,7 +192,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         fill_store(j0 * RB - PSPW_HALO + piece * RB, w);
     }
     load_pairs(a, m, cl, vl, cr, vr);
-    gather_remote(cr, xr);
+    gather_remote(cr, m, b, xr);
     to_ring(a, m, cl, vl);
     __syncthreads();
 
@@ -355,7 +357,7 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
         }
 
         // ---- hand over to block j + 1 ---------------------------------------------------------------------------------
-        gather_remote(crn, xr);                     // in flight while block j + 1 is summed from the ring
+        gather_remote(crn, mn, bn, xr);                     // in flight while block j + 1 is summed from the ring
         fill_store((j + 1) * RB + PSPW_HALO, w);    // slots no row of block j's or j + 1's window occupies
 #pragma unroll
         for (int k = 0; k < RPG; k++) {
