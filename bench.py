@@ -419,11 +419,19 @@ def bench_sddmm(args):
         torch.cuda.synchronize()
         return e0.elapsed_time(e1) / args.steps
 
+    # the windowed layout beside the PCSR formats when the matrix has the locality it is made for
+    from paramspmm_ae_amd.GNN import WINDOW_MIN_LOCAL_SHARE
+
+    rp_w, ci_w, _, local_share = c.window_format(dev)
+    windowed = local_share >= WINDOW_MIN_LOCAL_SHARE
+
     per_K = []
     for K in (16, 32, 64, 128):
         A = torch.randn(rows, K, device=dev, generator=gen)
         Bm = torch.randn(rows, K, device=dev, generator=gen)
         cands = {}
+        if windowed:
+            cands[("window", 0)] = lambda: ParamSDDMM.window_sddmm(A, Bm, rp_w, ci_w, None)
         for bw in (4, 8):
             # each format with the XCD stripe graph_input chose for it (flag bits of blkWarpNum)
             cands[("csr", bw)] = lambda bw=bw: ParamSDDMM.csr_sddmm(A, Bm, C["rowPtr"], C["colIdx"], C["val"], 1, bw | stripe[0])
@@ -435,7 +443,9 @@ def bench_sddmm(args):
             cands[("bcsr_split", bw)] = lambda bw=bw: ParamSDDMM.bcsr_split_sddmm(A, Bm, Bf["rowPtr_split"], Bf["colIdx"], Bf["val"], Bf["target_row"], 1, bw | stripe[3])
         times = {k: timed(f) for k, f in cands.items()}
         (fmt, bw), ms = min(times.items(), key=lambda kv: kv[1])
-        if fmt.startswith("bcsr"):
+        if fmt == "window":
+            alg = 4 * rp_w.numel() + 4 * nnz + 8 * n * K + 4 * nnz
+        elif fmt.startswith("bcsr"):
             alg = 4 * (Bf["rowPtr_split" if "split" in fmt else "rowPtr"].numel()) + 12 * nblk + 8 * n * K + 8 * nblk
         else:
             alg = 4 * (C["rowPtr_split" if "split" in fmt else "rowPtr"].numel()) + 4 * nnz + 8 * n * K + 4 * nnz
