@@ -37,9 +37,11 @@ const char *psp_last_error(void);
  * buffers that the library fills have grown between versions under unchanged symbol names --
  *   200: psp_spmm_plan gained log_segs_per_wave, even_split, xcd_stripe_rows (10 ints; 7 before);
  *        psp_nll_loss_mean_f32 writes 3 + 3*1024 floats of `stats` (2 before);
- *   300: option "whole_rows"; the windowed-CSR entry points.
+ *   300: option "whole_rows"; the windowed-CSR entry points;
+ *   310: PSP_WINDOW_HALO is 88 (64 before: windowed arrays built by a 300 library do not match these kernels -- build
+ *        them again); psp_sddmm_window_f32, psp_attn_window_forward_f32 / _backward_f32; option "dense_split".
  * The extension modules and the ctypes loader of this package check it when they are imported. */
-#define PSP_ABI_VERSION 300
+#define PSP_ABI_VERSION 310
 int psp_version(void);
 
 /* How a (N, CF, blkWarpNum) request of the Python layer maps onto the wave64 kernels.

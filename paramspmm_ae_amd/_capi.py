@@ -115,7 +115,7 @@ for _name, _args in SIGNATURES.items():
 lib.psp_last_error.argtypes = []
 lib.psp_last_error.restype = ctypes.c_char_p
 
-ABI_VERSION = 300  # PSP_ABI_VERSION of include/paramsp.h: the struct layouts and buffer sizes this module assumes
+ABI_VERSION = 310  # PSP_ABI_VERSION of include/paramsp.h: the struct layouts and buffer sizes this module assumes
 if lib.psp_version() < ABI_VERSION:
     raise ImportError("%s is version %d, this package needs %d: rebuild it (paramspmm_ae_amd/build_param.sh)"
                       % (LIB_PATH, lib.psp_version(), ABI_VERSION))

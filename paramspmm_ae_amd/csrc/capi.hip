@@ -90,7 +90,7 @@ PSP_EXPORT long long psp_get_option(const char *name)
 }
 
 PSP_EXPORT const char *psp_last_error(void) { return g_err; }
-PSP_EXPORT int psp_version(void) { return 300; }
+PSP_EXPORT int psp_version(void) { return PSP_ABI_VERSION; }
 
 // ------------------------------------------------------------------------------------------------
 // (N, CF, blkWarpNum) -> wave64 launch plan
