@@ -204,6 +204,102 @@ def test_gcn_operators_at_full_size():
         torch.cuda.empty_cache()
 
 
+def test_windowed_operators_at_full_size(oracle):
+    """The windowed layout on the SBM graph in community order (1 M rows, 20.9 M entries, nine entries in ten local):
+      * SpMM: X = ones -> row sums (the reference's known answer, verification.py:26-46) against float64; the oracle on
+        a row sample; agreement with the plain CSR kernel at N = 16 / 32 / 64 / 128, with the activation and the mask
+        folded in, and with the dense product folded in (N = 16, 32);
+      * SDDMM: A = B = ones -> K exactly (SDDMM.py:127-128); agreement with the CSR kernel on the same arrays, with one
+        matrix on both sides and with two;
+      * the attention passes: scores and aggregate against the SDDMM followed by the SpMM, the weight-gradient sum
+        against a float64 dot product."""
+    import paramspmm_ae_amd  # noqa: F401
+    import ParamSDDMM
+    import ParamSpCONV
+    import ParamSpMM
+    from gpu_util import assert_close
+    from paramspmm_ae_amd import synth
+    from paramspmm_ae_amd.graph_input import graph_input
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+
+    rowPtr, colIdx, val, n = synth.config_graph("C5")
+    g = graph_input("C5", "")
+    g.verbose = False
+    g.load_from_csr(rowPtr, colIdx, val)
+    win = pcsr_spmm(g, vec_size=1, if_split=False, window=True)
+    csr = pcsr_spmm(g, vec_size=1, if_split=False, CF=1, blkWarpNum=4)
+    assert win.window_local_share > 0.85
+    ci_w = win.colIdx.cpu().numpy()
+    v_w = win.val.cpu().numpy()
+    # the layout is a permutation inside the rows
+    assert np.array_equal(win.rowPtr_w.cpu().numpy()[0:2 * n:2], rowPtr[:-1])
+    sample = sample_rows(rowPtr)
+    for r in sample[:: max(1, sample.size // 200)]:
+        a, b = rowPtr[r], rowPtr[r + 1]
+        assert sorted(zip(ci_w[a:b].tolist(), v_w[a:b].tolist())) == sorted(zip(colIdx[a:b].tolist(), val[a:b].tolist()))
+    row_sums = np.add.reduceat(val.astype(np.float64), rowPtr[:-1])
+    gen = torch.Generator(device="cuda").manual_seed(11)
+    for N in (16, 32, 64, 128):
+        print("case window spmm", N, flush=True)
+        ones = torch.ones(n, N, device="cuda")
+        got = win._spmm(ones).cpu().numpy()
+        assert np.all(np.abs(got - row_sums[:, None]) <= 1e-6 + 1e-5 * np.abs(row_sums[:, None]))
+        X = torch.randn(n, N, device="cuda", generator=gen)
+        Y = win._spmm(X)
+        ref = csr._spmm(X)
+        A_abs = torch.sparse_csr_tensor(csr.rowPtr, csr.colIdx, csr.val.abs(), size=(n, n))
+        scale = torch.sparse.mm(A_abs, X.abs())
+        assert torch.all((Y - ref).abs() <= 2e-6 + 2e-5 * scale)  # two roundings: each kernel against the exact sum
+        rp_s, ci_s, v_s = sub_csr(rowPtr, colIdx, val, sample)
+        Xh = X.cpu().numpy()
+        want = oracle.spmm_csr(rp_s, ci_s, v_s, Xh, rows_out=sample.size)
+        sc = oracle.spmm_csr(rp_s, ci_s, np.abs(v_s), np.abs(Xh), rows_out=sample.size)
+        assert_close(Y[torch.from_numpy(sample).cuda()], want, what="window vs oracle N=%d" % N, scale=sc)
+        M = torch.randn(n, N, device="cuda", generator=gen)
+        Ya = ParamSpCONV.aggregate_act(4, X, win.rowPtr_w, win.colIdx, win.val, None, 0, 4, True, M)
+        plain = win._spmm(torch.relu(X))
+        assert torch.equal(Ya, torch.where(M > 0, plain, torch.zeros_like(plain)))
+        if N <= 32:
+            W = torch.randn(N, N, device="cuda", generator=gen) / N ** 0.5
+            out, raw = ParamSpCONV.window_xw(X, W, False, win.rowPtr_w, win.colIdx, win.val, True, None, True)
+            assert torch.equal(raw, plain)
+            want_xw = plain.double() @ W.double()
+            sc_xw = plain.abs().double() @ W.abs().double()
+            assert torch.all((out.double() - want_xw).abs() <= 1e-6 + 1e-5 * sc_xw)
+    for K in (16, 64, 128):
+        print("case window sddmm", K, flush=True)
+        ones = torch.ones(n, K, device="cuda")
+        assert bool((win.AGNN_sddmm(ones) == K).all())
+        X = torch.nn.functional.normalize(torch.randn(n, K, device="cuda", generator=gen), dim=1).contiguous()
+        Z = torch.nn.functional.normalize(torch.randn(n, K, device="cuda", generator=gen), dim=1).contiguous()
+        for A_, B_ in ((X, X), (X, Z)):
+            e = ParamSDDMM.window_sddmm(A_, B_, win.rowPtr_w, win.colIdx, None)
+            ref = ParamSDDMM.csr_sddmm(A_, B_, win.rowPtr, win.colIdx, win.val, 1, 4)
+            rows_t = torch.repeat_interleave(torch.arange(n, device="cuda"), torch.from_numpy(np.diff(rowPtr)).cuda())
+            sc = (A_[rows_t].abs() * B_[win.colIdx.long()].abs()).sum(1)
+            assert torch.all((e - ref).abs() <= 2e-6 + 2e-5 * sc)
+    for K in (16, 64):
+        print("case window attention", K, flush=True)
+        X = torch.nn.functional.normalize(torch.randn(n, K, device="cuda", generator=gen), dim=1).contiguous()
+        alpha = torch.tensor([0.7], device="cuda")
+        att, Y = ParamSpCONV.attn_window_forward(X, win.rowPtr_w, win.colIdx, alpha)
+        e = ParamSDDMM.window_sddmm(X, X, win.rowPtr_w, win.colIdx, alpha)
+        assert torch.all((att - e).abs() <= 2e-6 + 2e-5 * 0.7)  # |<x, y>| <= 1 for unit rows
+        Yref = ParamSpMM.window_spmm(X, win.rowPtr_w, win.colIdx, att, 0)
+        A_att = torch.sparse_csr_tensor(win.rowPtr, win.colIdx, att.abs(), size=(n, n))
+        assert torch.all((Y - Yref).abs() <= 2e-6 + 2e-5 * torch.sparse.mm(A_att, X.abs()))
+        dY = torch.randn(n, K, device="cuda", generator=gen) / K ** 0.5
+        G, wsum = ParamSpCONV.attn_window_backward(dY, att, win.rowPtr_w, win.colIdx)
+        Gref = ParamSpMM.window_spmm(dY, win.rowPtr_w, win.colIdx, att, 0)
+        assert torch.all((G - Gref).abs() <= 2e-6 + 2e-5 * torch.sparse.mm(A_att, dY.abs()))
+        d = ParamSDDMM.window_sddmm(dY, dY, win.rowPtr_w, win.colIdx, None).double()
+        colf = win.colIdx.float().double()
+        want_w = float((d * colf).sum().item())
+        # the reference forms this sum in fp32 (gnn_conv.py:172); so does the kernel, per lane and per workgroup: the
+        # bound is that of a tree of fp32 additions over the magnitudes
+        assert abs(float(wsum.item()) - want_w) <= 1e-4 * float((d.abs() * colf).sum().item())
+
+
 @pytest.mark.parametrize("K", [32, 64])
 def test_attention_layer_on_the_headline_pattern_at_full_size(K):
     """The attention layer of the R-MAT 2^20 workload (out_e = A_e <X_i, Y_j> with row-normalised X, Y; softmax over
