@@ -12,6 +12,7 @@
 //                        fp32 atomics.
 #include "psp_common.h"
 #include "spmm_kernel.h"
+#include "bf16_split.h"
 
 // RELU_A (both kernels): A enters the product as max(a, 0) -- the weight gradient of a layer whose input is the
 // activation of the previous layer's output, without that activation ever being stored.
@@ -241,23 +242,6 @@ psp_atb_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B, fl
 // 64 t + 4 c ..: tile 4 t + e takes element e) and one float2 of its wavefront's quarter of B (columns col0 + 2 c + q:
 // tile q), so one load instruction covers 256 (128) contiguous bytes of four rows.  The four wavefronts of a workgroup
 // share a chunk and own a quarter of B's columns each, as in the JSPLIT = 4 form above.  Rows past n enter as zeros.
-typedef __bf16 psp_bf16x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 psp_bf16x8 __attribute__((ext_vector_type(8)));
-typedef unsigned int psp_u32x4 __attribute__((ext_vector_type(4)));
-
-// two floats -> their three bf16 terms, packed in pairs (low half = first float)
-__device__ __forceinline__ void psp_atb_split3(float a, float b, unsigned &hi, unsigned &mid, unsigned &lo)
-{
-    psp_f32x2 v = {a, b};
-    hi = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
-    v[0] = a - __uint_as_float(hi << 16);
-    v[1] = b - __uint_as_float(hi & 0xffff0000u);
-    mid = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
-    v[0] -= __uint_as_float(mid << 16);
-    v[1] -= __uint_as_float(mid & 0xffff0000u);
-    lo = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
-}
-
 #define ATB_SPLIT_WGS 256  // one workgroup per CU (the kernel's 410 registers allow no more): as many partial products to add
 
 template <bool RELU_A>
@@ -304,7 +288,7 @@ psp_atb_split_kernel(const float *__restrict__ A, const float *__restrict__ B, f
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 unsigned h_, m_, l_;
-                psp_atb_split3(fb[2 * g][q], fb[2 * g + 1][q], h_, m_, l_);
+                psp_split3(fb[2 * g][q], fb[2 * g + 1][q], h_, m_, l_);
                 bh[q][g] = h_, bm[q][g] = m_, bl[q][g] = l_;
             }
 #pragma unroll
@@ -318,7 +302,7 @@ psp_atb_split_kernel(const float *__restrict__ A, const float *__restrict__ B, f
                     y = y < 0.0f ? 0.0f : y;
                 }
                 unsigned h_, m_, l_;
-                psp_atb_split3(x, y, h_, m_, l_);
+                psp_split3(x, y, h_, m_, l_);
                 ah[g] = h_, am[g] = m_, al[g] = l_;
             }
             // small terms first; the two column tiles alternate, so no instruction waits for the one before it

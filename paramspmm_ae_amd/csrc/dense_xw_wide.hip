@@ -22,6 +22,7 @@
 // gfx950 only, whose CUs have 160 KB, and two workgroups per CU (the launch shape) need 132 KB of it.  The grid is sized
 // to the GPU and every wavefront walks blocks of 32 rows with the next block's loads in flight.
 #include "psp_common.h"
+#include "bf16_split.h"
 #include <cstdlib>
 
 typedef float psp_f32x4 __attribute__((ext_vector_type(4)));
@@ -151,23 +152,6 @@ psp_xw_wide_kernel(const float *__restrict__ X, const float *__restrict__ W, flo
 // (2s, 2s + 1), i.e. columns 32s + 16 (i / 4) + 4q + i % 4 stand for k = 8q + i, and the W fragments in LDS follow the same
 // rule: [s][tile j][hi | mid | lo][lane][8 bf16], one 16-byte read per fragment.  An infinite input turns its products
 // into NaN (inf - inf in the split) instead of +-inf; NaN stays NaN.
-typedef __bf16 psp_bf16x2 __attribute__((ext_vector_type(2)));
-typedef __bf16 psp_bf16x8 __attribute__((ext_vector_type(8)));
-typedef unsigned int psp_u32x4 __attribute__((ext_vector_type(4)));
-typedef float psp_f32x2 __attribute__((ext_vector_type(2)));
-
-// two floats -> their three bf16 terms, packed in pairs (low half = first float)
-__device__ __forceinline__ void psp_split3(float a, float b, unsigned &hi, unsigned &mid, unsigned &lo)
-{
-    psp_f32x2 v = {a, b};
-    hi = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
-    v[0] = a - __uint_as_float(hi << 16);
-    v[1] = b - __uint_as_float(hi & 0xffff0000u);
-    mid = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
-    v[0] -= __uint_as_float(mid << 16);
-    v[1] -= __uint_as_float(mid & 0xffff0000u);
-    lo = __builtin_bit_cast(unsigned, __builtin_convertvector(v, psp_bf16x2));
-}
 
 template <bool RELU_X, bool MASK>
 __global__ void __launch_bounds__(512)
