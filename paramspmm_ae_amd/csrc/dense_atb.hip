@@ -242,10 +242,10 @@ psp_atb_mfma_kernel(const float *__restrict__ A, const float *__restrict__ B, fl
 // 64 t + 4 c ..: tile 4 t + e takes element e) and one float2 of its wavefront's quarter of B (columns col0 + 2 c + q:
 // tile q), so one load instruction covers 256 (128) contiguous bytes of four rows.  The four wavefronts of a workgroup
 // share a chunk and own a quarter of B's columns each, as in the JSPLIT = 4 form above.  Rows past n enter as zeros.
-#define ATB_SPLIT_WGS 256  // one workgroup per CU (the kernel's 410 registers allow no more): as many partial products to add
+#define ATB_SPLIT_WGS 512  // two workgroups per CU (three, at 168 registers with spills, were slower): as many partial products to add
 
 template <bool RELU_A>
-__global__ void __launch_bounds__(256)
+__global__ void __launch_bounds__(256, 2)
 psp_atb_split_kernel(const float *__restrict__ A, const float *__restrict__ B, float *__restrict__ C, long long n,
                      float *__restrict__ partial)
 {
@@ -260,8 +260,8 @@ psp_atb_split_kernel(const float *__restrict__ A, const float *__restrict__ B, f
         for (int q = 0; q < RNW; q++) acc[m][q] = psp_mfma_acc{0.f, 0.f, 0.f, 0.f};
 
     const long long chunks = (n + 31) >> 5;
-    psp_f32x4 a0[8][2], a1[8][2];
-    psp_f32x2 b0[8], b1[8];
+    psp_f32x4 a0[8][2];
+    psp_f32x2 b0[8];
     // unconditional loads from clamped rows; what lies past n is cleared where it is used
     auto fetch = [&](long long ch, psp_f32x4 (&fa)[8][2], psp_f32x2 (&fb)[8]) {
 #pragma unroll
@@ -318,24 +318,11 @@ psp_atb_split_kernel(const float *__restrict__ A, const float *__restrict__ B, f
 #undef ATBS_TERM
         }
     };
-    long long ch = blockIdx.x;
-    const long long step = gridDim.x;
-    if (ch < chunks) {
+    // one set of operand registers: two workgroups share a CU (256 registers per lane each), and while one waits for
+    // its chunk the other takes its own apart and multiplies
+    for (long long ch = blockIdx.x; ch < chunks; ch += gridDim.x) {
         fetch(ch, a0, b0);
-        while (true) {
-            long long nxt = ch + step;
-            if (nxt < chunks) fetch(nxt, a1, b1);
-            __builtin_amdgcn_sched_barrier(0);
-            multiply(ch, a0, b0);
-            if (nxt >= chunks) break;
-            ch = nxt;
-            nxt = ch + step;
-            if (nxt < chunks) fetch(nxt, a0, b0);
-            __builtin_amdgcn_sched_barrier(0);
-            multiply(ch, a1, b1);
-            if (nxt >= chunks) break;
-            ch = nxt;
-        }
+        multiply(ch, a0, b0);
     }
     // accumulator register v of lane (c, kk), tile (m, q) is C[64 (m / 4) + 4 (4 kk + v) + m % 4][col0 + 2 c + q]
     float *dst = partial ? partial + (size_t)blockIdx.x * (K1 * K2) : C;
