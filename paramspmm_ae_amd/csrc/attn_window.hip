@@ -11,8 +11,9 @@
 //
 // A lane group of L = 4 or 8 lanes owns one row and covers the whole width (K <= 4 C L).  Per local entry: one
 // ds_read_b128 per lane and vector, 4 C multiply-adds for the partial dot product, log2(L) DPP additions to complete
-// it in every lane, 4 C multiply-adds into the row's sum.  Remote entries (up to 4 per row prefetched into registers,
-// the rest in a plain loop) go the same way from global memory.
+// it in every lane, 4 C multiply-adds into the row's sum.  Remote entries go the same way from global memory: the
+// first four of a row from registers filled a block ahead, entries 4 .. 7 of lane groups of 8 in a second round when
+// some row of the wavefront has them, the rest in a plain loop.
 // Summation order: a score is summed inside a lane over k = s, s + L, ..., then across the lanes; a row of Y over its
 // local entries in storage order, then the remote ones.  Within the stated fp32 tolerance of the two reference
 // operators, not bit-identical to them.  *wsum is accumulated with one atomic addition per workgroup.

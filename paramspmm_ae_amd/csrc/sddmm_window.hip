@@ -6,11 +6,12 @@
 // only the remote ones gather.
 //
 // A workgroup walks a run of consecutive 64-row blocks; a lane group of L = 4 or 8 lanes owns one row of the block and
-// holds that row of A in registers, 4 C floats per lane (K <= 16 C L / 4 ... the whole of K is covered by one lane
-// group: TN = 4 C L >= K).  Per chunk of L local entries the group forms L partial dot products (one ds_read_b128 of
+// holds that row of A in registers, 4 C floats per lane (the whole of K is covered by one lane group: 4 C L >= K).
+// Per chunk of L local entries the group forms L partial dot products (one ds_read_b128 of
 // the B row and 4 C multiply-adds per lane and entry) and sums them across the lanes with L - 1 DPP additions, after
-// which lane s holds entry s of the chunk and the group stores L consecutive floats.  The remote entries' B rows (up
-// to 4 per row) were gathered into registers while the previous block was processed; longer rows finish in plain
+// which lane s holds entry s of the chunk and the group stores L consecutive floats.  The B rows of a row's first four
+// remote entries were gathered into registers while the previous block was processed; lane groups of 8 gather those
+// of entries 4 .. 7 together in a second round when some row of the wavefront has them; longer rows finish in plain
 // loops.  SAME: A and B are the same matrix (the attention scores of a graph layer, <X_i, X_j>), so the row of A is
 // read from the ring as well and X is read from HBM once.
 // Per entry the products are summed in the order k = s, s + L, ... inside a lane, then across the lanes: within the

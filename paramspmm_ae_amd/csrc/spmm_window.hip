@@ -17,14 +17,17 @@
 // g mod 304): the windows of neighbouring blocks differ by 64 rows, so a step to the next block loads only the 64 rows
 // that enter -- and they land in the slots of the 64 rows that the block after next no longer needs, so the ring never
 // overwrites a row that is still being read and one barrier per block is enough.  A lane group of L = 4 or 8 lanes
-// owns L / 4 rows of a block.  The walk is software-pipelined, so that after the first block of a run no lane waits for
+// owns one row of a block (workgroups of 512 lanes for L = 8).  The walk is software-pipelined, so that after the first block of a run no lane waits for
 // a load it has just issued: while block j is summed from LDS, the loads in flight are
 //   * the X row tiles of block j's remote entries (up to UR = 4 per row, gathered from global memory into registers,
 //     issued when block j - 1 was finished),
 //   * the 64 new window rows, the (column, value) pairs and the row bounds of the blocks that follow.
 // Local entries are read with ds_read_b128 -- no global gather instruction in that loop; the (column, value) pairs
-// travel round the lane group with DPP moves, not through the LDS crossbar.  Rows with more than 32 local or 4 remote
-// entries finish in plain loops (correct for any matrix, slow for matrices the format is not meant for).  Per
+// travel round the lane group with DPP moves, not through the LDS crossbar.  A lane group of 8 keeps the pairs of a
+// row's first eight remote entries (entry e in lane e) and gathers the rows of entries 4 .. 7 together, in a second
+// round, when some row of the wavefront has that many; prefetch slots past a row's remote part read one shared address.
+// Rows with more than 32 local or 8 (groups of 4 lanes: 4) remote entries finish in plain loops (correct for any
+// matrix, slow for matrices the format is not meant for).  Per
 // element the sum runs over the local entries in storage order, then the remote ones: within the stated fp32
 // tolerance of the reference's chain, not bit-identical to it.
 // EPI (square layers of 16 or 32 columns, one column tile): the finished row is multiplied by a small dense matrix
