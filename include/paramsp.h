@@ -39,7 +39,8 @@ const char *psp_last_error(void);
  *        psp_nll_loss_mean_f32 writes 3 + 3*1024 floats of `stats` (2 before);
  *   300: option "whole_rows"; the windowed-CSR entry points;
  *   310: PSP_WINDOW_HALO is 88 (64 before: windowed arrays built by a 300 library do not match these kernels -- build
- *        them again); psp_sddmm_window_f32, psp_attn_window_forward_f32 / _backward_f32; option "dense_split".
+ *        them again); psp_sddmm_window_f32, psp_attn_window_forward_f32 / _backward_f32, psp_softmax_nll_mean_f32 (+ backward);
+ *        option "dense_split".
  * The extension modules and the ctypes loader of this package check it when they are imported. */
 #define PSP_ABI_VERSION 310
 int psp_version(void);
@@ -445,6 +446,16 @@ int psp_nll_loss_mean_f32(const float *logp, const long long *labels, long long 
                           psp_stream_t stream);
 int psp_nll_loss_mean_backward_f32(const long long *labels, const float *grad_loss, const float *stats, long long n,
                                    int C, float *grad_logp, psp_stream_t stream);
+
+/* The same loss from the logits: F.nll_loss(F.log_softmax(x, 1), labels) (GNN.py:61,78,101 with 131-146) in one pass
+ * over x instead of five over the [n, C] matrix.  C a multiple of 4 up to 64 (psp_softmax_nll_supported), x 16-byte
+ * aligned; loss and stats as above (stats[0] is the sum of the log-probabilities of the labels).  The backward call
+ * writes d loss / d x = (softmax(x) - onehot(label)) * grad_loss / count for rows that count, 0 for the others. */
+int psp_softmax_nll_supported(int C);
+int psp_softmax_nll_mean_f32(const float *logits, const long long *labels, long long n, int C, float *loss, float *stats,
+                             psp_stream_t stream);
+int psp_softmax_nll_mean_backward_f32(const float *logits, const long long *labels, const float *grad_loss,
+                                      const float *stats, long long n, int C, float *grad_logits, psp_stream_t stream);
 
 /* ---------------------------------------------------------------------------------------------
  * DEVICE: double precision.  The reference dispatches its SpMM / SDDMM kernels for double as well

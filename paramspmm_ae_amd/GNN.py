@@ -17,7 +17,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .decider import SpMMDecider, DEFAULT_PICKLE_PATH
-from .gnn_conv import AGNNConv, GCNConv, GINConv, nll_loss_mean
+from .gnn_conv import AGNNConv, GCNConv, GINConv, nll_loss_mean, softmax_nll_loss_mean
 from .graph_input import graph_input
 from .PCSR import pcsr_spmm
 
@@ -35,17 +35,21 @@ class Net_5layers(torch.nn.Module):
         )
         self.fuse_relu = True  # False: F.relu between the layers as separate passes, as the reference's driver does
 
-    def forward(self):
+    def logits(self):
+        """The network up to, and without, its log-softmax (what loss_of_step folds into the loss)."""
         if not self.fuse_relu:
             x = self.x
             for conv in (self.conv1, self.conv2, self.conv3, self.conv4):
                 x = F.relu(conv(x, self.spmm_dict))
-            return F.log_softmax(self.conv5(x, self.spmm_dict), dim=1)
+            return self.conv5(x, self.spmm_dict)
         # the same network with every ReLU applied by the layer that reads it (no activation passes)
         z = self.conv1(self.x, self.spmm_dict)
         for conv in (self.conv2, self.conv3, self.conv4, self.conv5):
             z = conv(z, self.spmm_dict, relu_input=True)
-        return F.log_softmax(z, dim=1)
+        return z
+
+    def forward(self):
+        return F.log_softmax(self.logits(), dim=1)
 
 
 class GIN(torch.nn.Module):
@@ -62,17 +66,21 @@ class GIN(torch.nn.Module):
 
         self.fuse_relu = True  # False: F.relu between the layers as separate passes, as the reference's driver does
 
-    def forward(self):
+    def logits(self):
+        """The network up to, and without, its log-softmax (what loss_of_step folds into the loss)."""
         if not self.fuse_relu:
             x = self.x
             for conv in (self.conv1, self.conv2, self.conv3, self.conv4):
                 x = F.relu(conv(x, self.spmm_dict))
-            return F.log_softmax(self.conv5(x, self.spmm_dict), dim=1)
+            return self.conv5(x, self.spmm_dict)
         # the same network with every ReLU applied inside the sparse product of the layer that reads it
         z = self.conv1(self.x, self.spmm_dict)
         for conv in (self.conv2, self.conv3, self.conv4, self.conv5):
             z = conv(z, self.spmm_dict, relu_input=True)
-        return F.log_softmax(z, dim=1)
+        return z
+
+    def forward(self):
+        return F.log_softmax(self.logits(), dim=1)
 
 
 class AGNN(torch.nn.Module):
@@ -89,13 +97,14 @@ class AGNN(torch.nn.Module):
         self.relu = nn.ReLU()
         self.fuse_relu = True  # False: ReLU between the layers as separate passes, as the reference's driver does
 
-    def forward(self):
+    def logits(self):
+        """The network up to, and without, its log-softmax (what loss_of_step folds into the loss)."""
         if not self.fuse_relu:
             x = self.relu(self.conv1(self.x, self.spmm_dict, self.colIdx))
             x = F.dropout(x, training=self.training)
             for conv in self.hidden_layers:
                 x = self.relu(conv(x, self.spmm_dict, self.colIdx))
-            return F.log_softmax(self.conv2(x, self.spmm_dict, self.colIdx), dim=1)
+            return self.conv2(x, self.spmm_dict, self.colIdx)
         # The same network with every ReLU applied by the layer that reads it.  Dropout scales by a non-negative
         # mask, so it commutes with the activation: dropping the pre-activation values and activating afterwards
         # gives what the reference's order gives, with the same random mask.
@@ -103,7 +112,19 @@ class AGNN(torch.nn.Module):
         z = F.dropout(z, training=self.training)
         for conv in self.hidden_layers:
             z = conv(z, self.spmm_dict, self.colIdx, relu_input=True)
-        return F.log_softmax(self.conv2(z, self.spmm_dict, self.colIdx, relu_input=True), dim=1)
+        return self.conv2(z, self.spmm_dict, self.colIdx, relu_input=True)
+
+    def forward(self):
+        return F.log_softmax(self.logits(), dim=1)
+
+
+def loss_of_step(model, labels):
+    """F.nll_loss(model(), labels) of the reference's training step (GNN.py:131-146).  The networks end in a
+    log-softmax; with ``model.fuse_loss`` (the default) it is folded into the loss -- one pass over the logits instead
+    of a softmax, a loss and their two backward passes."""
+    if getattr(model, "fuse_loss", True) and hasattr(model, "logits"):
+        return softmax_nll_loss_mean(model.logits(), labels)
+    return nll_loss_mean(model(), labels)
 
 
 def capture_training_step(model, labels, optimizer, warmup=3):
@@ -118,13 +139,13 @@ def capture_training_step(model, labels, optimizer, warmup=3):
     with torch.cuda.stream(side):
         for _ in range(warmup):
             optimizer.zero_grad(set_to_none=True)
-            nll_loss_mean(model(), labels).backward()
+            loss_of_step(model, labels).backward()
             optimizer.step()
     torch.cuda.current_stream().wait_stream(side)
     optimizer.zero_grad(set_to_none=True)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        loss = nll_loss_mean(model(), labels)
+        loss = loss_of_step(model, labels)
         loss.backward()
         optimizer.step()
     return graph, loss
@@ -138,7 +159,7 @@ def train_profiling(model, labels, num_epoches, verbose=False, progress=False, h
     def epoch():
         model.train()
         optimizer.zero_grad()
-        loss = nll_loss_mean(model(), labels)
+        loss = loss_of_step(model, labels)
         loss.backward()
         optimizer.step()
         return loss
@@ -285,6 +306,8 @@ def main(argv=None):
                         "are generated in the new order")
     p.add_argument("--no_aggregate_first", action="store_true",
                    help="GCN: always A (H W), also for the first layer when it widens its input (the reference's order)")
+    p.add_argument("--no_fuse_loss", action="store_true",
+                   help="run the networks' log-softmax and the loss as operators of their own, as the reference's driver does")
     p.add_argument("--no_fuse_relu", action="store_true",
                    help="apply the ReLU between the layers as passes of their own, as the reference's driver does")
     p.add_argument("--try_candidates", type=int, default=0, metavar="K",
@@ -327,6 +350,8 @@ def main(argv=None):
                                       try_candidates=args.try_candidates, try_window=not args.no_window)
             print("SpMM-decider config time: {:.3f} (ms)".format((time.perf_counter() - t1) * 1e3))
             model = build_model(args.net, graph, ops, hidden, args.num_features, args.num_classes, args.num_layers)
+            if args.no_fuse_loss:
+                model.fuse_loss = False
             if args.no_fuse_relu and hasattr(model, "fuse_relu"):
                 model.fuse_relu = False
             torch.cuda.synchronize()

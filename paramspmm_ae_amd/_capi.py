@@ -91,6 +91,9 @@ SIGNATURES = {
     "psp_window_build_dev": [_vp, _vp, _vp, _i, _vp, _vp, _vp, _vp],
     "psp_spmm_window_plan": [_i, _i, ctypes.POINTER(_i), ctypes.POINTER(_i), ctypes.POINTER(_i)],
     "psp_spmm_window_f32": [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp],
+    "psp_softmax_nll_supported": [_i],
+    "psp_softmax_nll_mean_f32": [_vp, _vp, ctypes.c_longlong, _i, _vp, _vp, _vp],
+    "psp_softmax_nll_mean_backward_f32": [_vp, _vp, _vp, _vp, ctypes.c_longlong, _i, _vp, _vp],
     "psp_sddmm_window_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "psp_attn_window_forward_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],
     "psp_attn_window_backward_f32": [_vp, _vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp],

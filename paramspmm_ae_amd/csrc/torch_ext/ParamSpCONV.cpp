@@ -329,6 +329,32 @@ static Tensor nll_loss_mean_backward(Tensor labels, Tensor grad_loss, Tensor sta
     return grad;
 }
 
+// the same loss from the logits (log-softmax folded in): [loss, stats]; and its gradient w.r.t. the logits
+static bool softmax_nll_supported(long C) { return psp_softmax_nll_supported((int)C) != 0; }
+static std::vector<Tensor> softmax_nll_mean(Tensor logits, Tensor labels)
+{
+    check_loss_args(logits, labels);
+    TORCH_CHECK(softmax_nll_supported(logits.size(1)), "softmax_nll_mean: the class count must be a multiple of 4 up to 64");
+    DeviceGuard guard(logits.device());
+    Tensor loss = torch::empty({}, logits.options()), stats = torch::empty({(long)psp_nll_loss_stats_floats()}, logits.options());
+    ok(psp_softmax_nll_mean_f32(fp(logits), (const long long *)labels.data_ptr<int64_t>(), logits.size(0), (int)logits.size(1),
+                                loss.data_ptr<float>(), stats.data_ptr<float>(), stream_of(logits)));
+    return {loss, stats};
+}
+static Tensor softmax_nll_mean_backward(Tensor logits, Tensor labels, Tensor grad_loss, Tensor stats)
+{
+    check_loss_args(logits, labels);
+    need_gpu(grad_loss, "grad_loss");
+    need_gpu(stats, "stats");
+    TORCH_CHECK(grad_loss.scalar_type() == torch::kFloat32 && grad_loss.numel() == 1, "grad_loss must hold one float");
+    TORCH_CHECK(stats.scalar_type() == torch::kFloat32 && stats.numel() >= 2 && stats.is_contiguous(), "bad stats");
+    DeviceGuard guard(logits.device());
+    Tensor grad = torch::empty_like(logits);
+    ok(psp_softmax_nll_mean_backward_f32(fp(logits), (const long long *)labels.data_ptr<int64_t>(), grad_loss.data_ptr<float>(),
+                                         stats.data_ptr<float>(), logits.size(0), (int)logits.size(1), fpw(grad), stream_of(logits)));
+    return grad;
+}
+
 #define PSP_CONV(NAME, FMT)                                                                                       \
     static Tensor NAME##_forward(Tensor H, Tensor W, Tensor rowPtr, Tensor colIdx, Tensor values, int CF, int bw)  \
     {                                                                                                             \
@@ -392,6 +418,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m)
     }, "max(Z, 0)^T * G: (Z, G)");
     m.def("nll_loss_mean", &nll_loss_mean, "[loss, stats] of the mean negative log-likelihood (log-probabilities, int64 labels)");
     m.def("nll_loss_mean_backward", &nll_loss_mean_backward, "gradient w.r.t. the log-probabilities: (labels, grad_loss, stats, n, C)");
+    m.def("softmax_nll_supported", &softmax_nll_supported, "is there a fused log-softmax + NLL kernel for this class count?");
+    m.def("softmax_nll_mean", &softmax_nll_mean, "[loss, stats] of nll_loss(log_softmax(logits), labels), mean over the rows");
+    m.def("softmax_nll_mean_backward", &softmax_nll_mean_backward, "gradient w.r.t. the logits: (logits, labels, grad_loss, stats)");
     m.def("attn_window_forward", &attn_window_forward,
           "attention layer on the windowed layout: (X, rowPtr_w, colIdx_w, alpha | None) -> [att, Y]");
     m.def("attn_window_backward", &attn_window_backward,

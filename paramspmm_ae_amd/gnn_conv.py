@@ -79,6 +79,31 @@ def nll_loss_mean(logp, labels):
     return torch.nn.functional.nll_loss(logp, labels)
 
 
+class _SoftmaxNllMean(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, logits, labels):
+        loss, stats = SpCONV.softmax_nll_mean(logits, labels)
+        ctx.save_for_backward(logits, labels, stats)
+        return loss
+
+    @staticmethod
+    def backward(ctx, grad_loss):
+        logits, labels, stats = ctx.saved_tensors
+        return SpCONV.softmax_nll_mean_backward(logits, labels, grad_loss.contiguous(), stats), None
+
+
+def softmax_nll_loss_mean(logits, labels):
+    """``F.nll_loss(F.log_softmax(logits, dim=1), labels)`` -- the end of the reference's networks and the loss of its
+    training step (GNN.py:61,78,101 and 131-146) -- as one function of the logits: one pass over the [n, C] matrix
+    forward, one read and one write backward, where the two separate operators make five.  Class counts other than a
+    multiple of 4 up to 64, and anything but contiguous float32 CUDA logits with int64 labels, take the separate
+    operators."""
+    if (logits.is_cuda and logits.dtype == torch.float32 and logits.dim() == 2 and labels.dtype == torch.int64
+            and labels.dim() == 1 and SpCONV.softmax_nll_supported(int(logits.shape[1]))):
+        return _SoftmaxNllMean.apply(logits.contiguous(), labels.contiguous())
+    return nll_loss_mean(torch.nn.functional.log_softmax(logits, dim=1), labels)
+
+
 class GCNFunction(torch.autograd.Function):
     """forward A(HW); backward dH = (A dY) W^T, dW = H^T (A dY) -- A is symmetric (gnn_conv.py:13-107)."""
 

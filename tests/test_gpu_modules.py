@@ -570,6 +570,64 @@ def test_the_128_wide_dense_product_on_either_matrix_core_path(n):
     assert L.psp_set_option(b"dense_split", 2) == -1
 
 
+@pytest.mark.parametrize("n,C", [(1, 16), (257, 4), (100_003, 16), (50_001, 32), (20_000, 64), (3000, 10)])
+def test_loss_from_the_logits_equals_log_softmax_then_nll(n, C):
+    """softmax_nll_loss_mean(x, y) against F.nll_loss(F.log_softmax(x.double(), 1), y): the loss to 1e-6 relative, the
+    gradient to 1e-6 + 1e-5 |g| of the float64 one; labels outside [0, C) (PyTorch's -100 among them) do not count and get
+    a zero gradient row; a class count the kernel does not take (10) runs the two separate operators."""
+    from paramspmm_ae_amd import gnn_conv
+
+    g = torch.Generator(device="cuda").manual_seed(n + C)
+    x = (torch.randn(n, C, device="cuda", generator=g) * 3.0).requires_grad_(True)
+    y = torch.randint(0, C, (n,), device="cuda", generator=g)
+    if n > 100:
+        y[5] = -100
+        y[n - 2] = -100
+    loss = gnn_conv.softmax_nll_loss_mean(x, y)
+    loss.backward(torch.tensor(1.7, device="cuda"))
+    xd = x.detach().double().requires_grad_(True)
+    want = torch.nn.functional.nll_loss(torch.nn.functional.log_softmax(xd, dim=1), y)
+    want.backward(torch.tensor(1.7, device="cuda", dtype=torch.float64))
+    assert abs(loss.item() - want.item()) <= 1e-6 * abs(want.item()) + 1e-7
+    assert torch.all((x.grad.double() - xd.grad).abs() <= 1e-6 / max(n, 1) + 1e-5 * xd.grad.abs())
+    if n > 100:
+        assert bool((x.grad[5] == 0).all()) and bool((x.grad[n - 2] == 0).all())
+    # large logits do not overflow
+    xb = torch.full((max(n, 2), C), 80.0, device="cuda")
+    xb[:, 0] = 120.0
+    yb = torch.zeros(max(n, 2), dtype=torch.int64, device="cuda")
+    lb = gnn_conv.softmax_nll_loss_mean(xb, yb)
+    assert bool(torch.isfinite(lb)) and lb.item() < 1e-6
+
+
+def test_networks_train_the_same_with_the_loss_folded_in():
+    """The GCN network's training step with the log-softmax folded into the loss (GNN.loss_of_step, the default) and with
+    the two as operators of their own: same loss, same gradients (fp32 rounding apart)."""
+    from paramspmm_ae_amd import GNN
+    from paramspmm_ae_amd.PCSR import pcsr_spmm
+
+    n = 20000
+    g, rowPtr, colIdx, val = sym_graph(n, 9)
+    op = pcsr_spmm(g, vec_size=1, if_split=False, CF=1, blkWarpNum=4)
+    torch.manual_seed(0)
+    x = torch.randn(n, 32, device="cuda")
+    labels = torch.randint(0, 16, (n,), device="cuda")
+    model = GNN.Net_5layers(16, 32, x, {16: op, 32: op}, 32).cuda()
+    res = {}
+    for fused in (True, False):
+        model.fuse_loss = fused
+        model.zero_grad(set_to_none=True)
+        loss = GNN.loss_of_step(model, labels)
+        loss.backward()
+        res[fused] = (loss.item(), [p.grad.clone() for p in model.parameters()])
+    assert abs(res[True][0] - res[False][0]) <= 1e-5 * abs(res[False][0])
+    for a, b in zip(res[True][1], res[False][1]):
+        torch.testing.assert_close(a, b, rtol=1e-3, atol=1e-5 * float(b.abs().max()) + 1e-7)
+    model.eval()
+    out = model()
+    torch.testing.assert_close(out.exp().sum(1), torch.ones(n, device="cuda"), rtol=1e-4, atol=1e-4)
+
+
 @pytest.mark.parametrize("vec_size", [2, 3])
 def test_sddmm_sweep_harness(tmp_path, vec_size):
     """SDDMM.py's facade and sweep (SDDMM.py:46-383) on the reference's pubmed pattern read from a .mtx file and on a
