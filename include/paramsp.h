@@ -308,12 +308,13 @@ int psp_sddmm_vec_split_f32(const int *rowPtr_bs, const int *colIdx_b, const flo
 /* ---------------------------------------------------------------------------------------------
  * Windowed CSR: a fifth representation, for matrices whose entries cluster around the diagonal (community-ordered
  * graphs, meshes, banded matrices).  No counterpart in the reference.  Rows are cut into blocks of PSP_WINDOW_BLOCK;
- * an entry is local when its column lies in [block start - PSP_WINDOW_HALO, block end + PSP_WINDOW_HALO).  The format
+ * an entry is local when its column lies in [block start - PSP_WINDOW_HALO, block end + PSP_WINDOW_HALO) and below M.  The format
  * keeps every row's entries, local ones first (each part in its original order), columns absolute:
  *   rowPtr_w[2M + 2]: 2i = start of row i, 2i + 1 = start of its remote part; 2M and 2M + 1 = nnz;
  *   colIdx_w[nnz], val_w[nnz]: the permuted entries.
  * psp_window_build fills them on the host, psp_window_build_dev on the device (same result).
- * psp_spmm_window_f32: Y[0..M) = A X (square A with nnz = rowPtr_w[2M] stored entries, X with at least M rows),
+ * psp_spmm_window_f32: Y[0..M) = A X (A with M rows and nnz = rowPtr_w[2M] stored entries, X with a row for every
+ * column and at least M of them),
  * Y[M..rows_out) = 0.  The X rows of a workgroup's window are staged in LDS and the local entries read them there;
  * only remote entries gather from global memory.  N must be a multiple of 4.  variant: 0 automatic, 1 / 2 / 3 = column tiles of 16 / 32 / 64 floats
  * (psp_spmm_window_plan reports tile width, rows per workgroup and LDS bytes, and returns the variant chosen).

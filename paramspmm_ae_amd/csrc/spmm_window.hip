@@ -376,10 +376,12 @@ psp_spmm_window_kernel(const int *__restrict__ rowPtr_w, const int *__restrict__
 }
 
 // ---- format construction ----------------------------------------------------------------------------------------
-__device__ __host__ static inline bool pspw_is_local(int row, int col)
+// (a column past the last row is never local: the kernels stage rows 0 .. M - 1 of the dense operand, and a matrix with
+// more columns than rows reaches the rest through the gathers)
+__device__ __host__ static inline bool pspw_is_local(int row, int col, int M)
 {
     const int lo = row / PSPW_BLOCK * PSPW_BLOCK - PSPW_HALO;
-    return col >= lo && col < lo + PSPW_BLOCK + 2 * PSPW_HALO;
+    return col >= lo && col < lo + PSPW_BLOCK + 2 * PSPW_HALO && col < M;
 }
 
 // one lane per row: local entries first, remote ones after, each part in the original order
@@ -397,7 +399,7 @@ psp_window_build_kernel(const int *__restrict__ rowPtr, const int *__restrict__ 
     int w = lb;
     for (int p = lb; p < hb; p++) {
         const int c = colIdx[p];
-        if (pspw_is_local(r, c)) {
+        if (pspw_is_local(r, c, M)) {
             colIdx_w[w] = c;
             val_w[w] = val[p];
             w++;
@@ -407,7 +409,7 @@ psp_window_build_kernel(const int *__restrict__ rowPtr, const int *__restrict__ 
     rowPtr_w[2 * r + 1] = w;
     for (int p = lb; p < hb; p++) {
         const int c = colIdx[p];
-        if (!pspw_is_local(r, c)) {
+        if (!pspw_is_local(r, c, M)) {
             colIdx_w[w] = c;
             val_w[w] = val[p];
             w++;
@@ -426,14 +428,14 @@ PSP_EXPORT int psp_window_build(const int *rowPtr, const int *colIdx, const floa
         PSP_REQUIRE(lb >= 0 && hb >= lb && hb <= nnz, "window_build: rowPtr is not a monotone prefix at row %d", r);
         int w = lb;
         for (int p = lb; p < hb; p++)
-            if (pspw_is_local(r, colIdx[p])) {
+            if (pspw_is_local(r, colIdx[p], M)) {
                 colIdx_w[w] = colIdx[p];
                 val_w[w++] = val[p];
             }
         rowPtr_w[2 * r] = lb;
         rowPtr_w[2 * r + 1] = w;
         for (int p = lb; p < hb; p++)
-            if (!pspw_is_local(r, colIdx[p])) {
+            if (!pspw_is_local(r, colIdx[p], M)) {
                 colIdx_w[w] = colIdx[p];
                 val_w[w++] = val[p];
             }

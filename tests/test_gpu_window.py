@@ -40,7 +40,7 @@ def window_reference(rowPtr, colIdx, val):
     M = rowPtr.size - 1
     rows = np.repeat(np.arange(M, dtype=np.int64), np.diff(rowPtr))
     lo = rows // BLOCK * BLOCK - HALO
-    local = (colIdx >= lo) & (colIdx < lo + BLOCK + 2 * HALO)
+    local = (colIdx >= lo) & (colIdx < lo + BLOCK + 2 * HALO) & (colIdx < M)  # columns past the last row are never local
     order = np.lexsort((np.arange(colIdx.size), ~local, rows))  # stable: row, then local first, then position
     rp = np.empty(2 * M + 2, np.int32)
     rp[0:2 * M:2] = rowPtr[:-1]
@@ -143,6 +143,43 @@ def test_device_builder_and_spmm_against_the_oracle(oracle, name):
     assert torch.equal(_spmm_window(F, X, relu=True), _spmm_window(F, torch.relu(X)))
     got = _spmm_window(F, X, mask=mask)
     assert torch.equal(got, torch.where(mask > 0, plain, torch.zeros_like(plain)))
+
+
+@pytest.mark.gpu
+def test_a_matrix_with_more_columns_than_rows(oracle):
+    """The first 1200 rows of a 1300-column banded matrix: columns past the last row are never local (the kernels stage
+    rows 0 .. M - 1 of the dense operand), so the SpMM and the SDDMM reach them through the gathers; X and B have a row
+    for every column."""
+    from gpu_util import assert_close, dev
+    from paramspmm_ae_amd import _capi
+    import ParamSpMM
+
+    rowPtr, colIdx, val = banded_csr(1300, 8, 40, 7, far=0.1)
+    M, ncols = 1200, 1300
+    rowPtr, colIdx, val = rowPtr[:M + 1].copy(), colIdx[:rowPtr[M]].copy(), val[:rowPtr[M]].copy()
+    assert colIdx.max() >= M
+    want_fmt = window_reference(rowPtr, colIdx, val)
+    rp, ci, v = ParamSpMM.window_build(dev(rowPtr), dev(colIdx), dev(val))
+    assert np.array_equal(rp.cpu().numpy(), want_fmt[0]) and np.array_equal(ci.cpu().numpy(), want_fmt[1])
+    ci_w = ci.cpu().numpy()
+    rows = np.repeat(np.arange(M), np.diff(rowPtr))
+    p, L = _capi.ptr, _capi.lib
+    st = torch.cuda.current_stream().cuda_stream
+    for N in (16, 32, 64, 128):
+        rng = np.random.default_rng(N)
+        X = rng.standard_normal((ncols, N)).astype(np.float32)
+        Xd = torch.from_numpy(X).cuda()
+        Y = torch.full((M, N), float("nan"), device="cuda")
+        _capi.check(L.psp_spmm_window_f32(p(rp), p(ci), p(v), p(Xd), p(Y), M, int(ci.numel()), N, M, 0, 0, None, st))
+        want = oracle.spmm_csr(rowPtr, colIdx, val, X, rows_out=M)
+        scale = oracle.spmm_csr(rowPtr, colIdx, np.abs(val), np.abs(X), rows_out=M)
+        assert_close(Y, want, what="rectangular spmm N=%d" % N, scale=scale)
+        A = rng.standard_normal((M, N)).astype(np.float32)
+        Ad = torch.from_numpy(A).cuda()
+        out = torch.full((colIdx.size,), float("nan"), device="cuda")
+        _capi.check(L.psp_sddmm_window_f32(p(rp), p(ci), p(Ad), p(Xd), None, p(out), M, int(ci.numel()), N, ncols, st))
+        assert_close(out, oracle.sddmm_csr(rowPtr, ci_w, A, X), what="rectangular sddmm K=%d" % N,
+                     scale=(np.abs(A[rows]) * np.abs(X[ci_w])).sum(1))
 
 
 @pytest.mark.gpu
