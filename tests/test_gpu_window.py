@@ -145,6 +145,84 @@ def test_device_builder_and_spmm_against_the_oracle(oracle, name):
     assert torch.equal(got, torch.where(mask > 0, plain, torch.zeros_like(plain)))
 
 
+def shaped_csr(M, seed):
+    """Rows whose numbers of local and remote entries run through every count the kernels treat differently: 0 .. 40
+    local entries (32 are fetched up front, the rest in a loop) and 0 .. 10 remote ones (4 prefetched, 4 more in a
+    second round for lane groups of 8, the rest in a loop), in all combinations that fit the row count."""
+    rng = np.random.default_rng(seed)
+    cols = []
+    for r in range(M):
+        n_local, n_remote = r % 41, (r // 3) % 11
+        lo = r // BLOCK * BLOCK - HALO
+        window = np.arange(max(lo, 0), min(lo + BLOCK + 2 * HALO, M))
+        outside = np.setdiff1d(np.arange(M), window)
+        c = np.concatenate([rng.choice(window, min(n_local, window.size), replace=False),
+                            rng.choice(outside, min(n_remote, outside.size), replace=False)])
+        cols.append(np.sort(c))
+    rowPtr = np.zeros(M + 1, np.int32)
+    rowPtr[1:] = np.cumsum([c.size for c in cols])
+    colIdx = (np.concatenate(cols) if rowPtr[-1] else np.zeros(0)).astype(np.int32)
+    val = rng.uniform(-1.0, 1.0, colIdx.size).astype(np.float32)
+    return rowPtr, colIdx, val
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("M", [1, 63, 64, 65, 129, 500, 1500])
+def test_every_row_shape_through_every_windowed_kernel(oracle, M):
+    """SpMM (three variants, with the dense product folded in where it exists), SDDMM and the attention passes on rows
+    of every local / remote count (shaped_csr), at row counts around the 64-row blocks, against the oracle."""
+    from gpu_util import assert_close, dev
+    from paramspmm_ae_amd import _capi
+    import ParamSpMM
+
+    rowPtr, colIdx, val = shaped_csr(M, M)
+    nnz = colIdx.size
+    rp, ci, v = ParamSpMM.window_build(dev(rowPtr), dev(colIdx), dev(val))
+    want_fmt = window_reference(rowPtr, colIdx, val)
+    assert np.array_equal(rp.cpu().numpy(), want_fmt[0]) and np.array_equal(ci.cpu().numpy(), want_fmt[1])
+    ci_w, v_w = ci.cpu().numpy(), v.cpu().numpy()
+    rows = np.repeat(np.arange(M), np.diff(rowPtr))
+    p, L = _capi.ptr, _capi.lib
+    st = torch.cuda.current_stream().cuda_stream
+    for N in (16, 32, 64, 128):
+        print("case shapes", M, N, flush=True)
+        rng = np.random.default_rng(N)
+        X = rng.standard_normal((M, N)).astype(np.float32)
+        Xd = torch.from_numpy(X).cuda()
+        want = oracle.spmm_csr(rowPtr, colIdx, val, X)
+        scale = oracle.spmm_csr(rowPtr, colIdx, np.abs(val), np.abs(X))
+        for variant in (0, 1, 2, 3):
+            assert_close(_spmm_window((rp, ci, v, M), Xd, variant), want, what="spmm N=%d variant %d" % (N, variant), scale=scale)
+        if N <= 32:
+            W = (rng.standard_normal((N, N)) / np.sqrt(N)).astype(np.float32)
+            Y, R = torch.empty(M, N, device="cuda"), torch.empty(M, N, device="cuda")
+            _capi.check(L.psp_spmm_window_xw_f32(p(rp), p(ci), p(v), p(Xd), p(torch.from_numpy(W).cuda()), 0, p(Y), p(R), M, nnz, N, M, 0,
+                                                 None, st))
+            assert_close(R, want, what="raw product beside the folded one", scale=scale)
+            assert_close(Y, want.astype(np.float64) @ W.astype(np.float64), what="folded dense product",
+                         scale=scale.astype(np.float64) @ np.abs(W).astype(np.float64))
+        out = torch.full((max(nnz, 1),), float("nan"), device="cuda")[:nnz]
+        _capi.check(L.psp_sddmm_window_f32(p(rp), p(ci), p(Xd), p(Xd), None, p(out), M, nnz, N, M, st))
+        e_scale = (np.abs(X[rows]) * np.abs(X[ci_w])).sum(1)
+        assert_close(out, oracle.sddmm_csr(rowPtr, ci_w, X, X), what="sddmm K=%d" % N, scale=e_scale)
+        if N <= 64:
+            att = torch.full((max(nnz, 1),), float("nan"), device="cuda")[:nnz]
+            Y = torch.full((M, N), float("nan"), device="cuda")
+            _capi.check(L.psp_attn_window_forward_f32(p(rp), p(ci), p(Xd), None, p(att), p(Y), M, nnz, N, M, st))
+            e = oracle.sddmm_csr(rowPtr, ci_w, X, X)
+            assert_close(att, e, what="attention scores K=%d" % N, scale=e_scale)
+            assert_close(Y, oracle.spmm_csr(rowPtr, ci_w, e, X), rtol=2e-5, what="attention aggregate K=%d" % N,
+                         scale=oracle.spmm_csr(rowPtr, ci_w, e_scale.astype(np.float32), np.abs(X)))
+            G = torch.full((M, N), float("nan"), device="cuda")
+            wsum = torch.full((1,), float("nan"), device="cuda")
+            _capi.check(L.psp_attn_window_backward_f32(p(rp), p(ci), p(v), p(Xd), p(G), p(wsum), M, nnz, N, M, st))
+            assert_close(G, oracle.spmm_csr(rowPtr, ci_w, v_w, X), what="attention backward aggregate K=%d" % N,
+                         scale=oracle.spmm_csr(rowPtr, ci_w, np.abs(v_w), np.abs(X)))
+            d = (X[rows].astype(np.float64) * X[ci_w].astype(np.float64)).sum(1)
+            w_scale = float((e_scale.astype(np.float64) * ci_w).sum())
+            assert abs(float(wsum.item()) - float((d * ci_w).sum())) <= 1e-6 + 2e-5 * w_scale
+
+
 @pytest.mark.gpu
 def test_a_matrix_with_more_columns_than_rows(oracle):
     """The first 1200 rows of a 1300-column banded matrix: columns past the last row are never local (the kernels stage
