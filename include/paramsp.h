@@ -100,8 +100,8 @@ int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan);
  *   "dense_split"      1 (default): the dense layer products (the gemm_xw and gemm_atb entry points) at 128 x 128 form
  *                      every fp32 product from the three bf16 terms of each operand (six bf16 matrix-core products,
  *                      fp32 accumulation: error 2^-23 of |x||w| per product, the rounding level of fp32) and are
- *                      bound by their memory traffic; an infinite input turns its row into NaN.  0: the fp32
- *                      matrix-core instruction, 25-40 % slower at that shape.
+ *                      bound by their memory traffic; an infinite input (or one within a bf16 rounding step of
+ *                      FLT_MAX) turns its row into NaN.  0: the fp32 matrix-core instruction, 25-40 % slower at that shape.
  * The environment (PSP_XCD_STRIPE_ROWS, PSP_ALIGN_PCT, PSP_SPLIT_CLEAR_MIN, PSP_WHOLE_ROWS, PSP_DENSE_SPLIT) sets the
  * initial values, once.
  * psp_get_option returns the value, or a negative psp_status for an unknown name.  Not synchronised with running
