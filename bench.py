@@ -810,9 +810,11 @@ def main():
             by_symbol.setdefault(sym, []).append(r)
             continue
         plan = _capi.spmm_plan(r["dim"], r["CF"], r["blkWarpNum"])
-        sym = "psp_spmm_kernel<%d, %d, %d, %d, %s, false, false>" % (plan["coarsen"], plan["vec"], plan["unroll"],
-                                                       2 if r["format"].startswith("bcsr") else 1,
-                                                       "true" if "split" in r["format"] else "false")
+        one_set = _capi.lib.psp_spmm_register_sets(plan["unroll"], plan["lanes_per_row"]) == 1
+        sym = "psp_spmm_kernel<%d, %d, %d, %d, %s, false, false, %s>" % (plan["coarsen"], plan["vec"], plan["unroll"],
+                                                           2 if r["format"].startswith("bcsr") else 1,
+                                                           "true" if "split" in r["format"] else "false",
+                                                           "true" if one_set else "false")
         r["kernel"] = sym
         by_symbol.setdefault(sym, []).append(r)
     sym, rows_of = max(by_symbol.items(), key=lambda kv: sum(r["ms"] for r in kv[1]))

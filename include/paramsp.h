@@ -40,9 +40,10 @@ const char *psp_last_error(void);
  *   300: option "whole_rows"; the windowed-CSR entry points;
  *   310: PSP_WINDOW_HALO is 88 (64 before: windowed arrays built by a 300 library do not match these kernels -- build
  *        them again); psp_sddmm_window_f32, psp_attn_window_forward_f32 / _backward_f32, psp_softmax_nll_mean_f32 (+ backward);
- *        option "dense_split".
+ *        option "dense_split";
+ *   311: psp_spmm_register_sets (no buffer changed).
  * The extension modules and the ctypes loader of this package check it when they are imported. */
-#define PSP_ABI_VERSION 310
+#define PSP_ABI_VERSION 311
 int psp_version(void);
 
 /* How a (N, CF, blkWarpNum) request of the Python layer maps onto the wave64 kernels.
@@ -75,6 +76,11 @@ typedef struct psp_spmm_plan {
     int xcd_stripe_rows;   /* rows (segments) dealt to one XCD at a time; 0: the library option "xcd_stripe_rows" */
 } psp_spmm_plan;
 int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *plan);
+/* Register sets of the SpMM kernel a plan runs (the last argument of the kernel's symbol as a profiler prints it: true
+ * for 1).  2: the feature loads of a batch of `unroll` entries are issued while the batch before is added.  1: a batch
+ * is gathered, added, and the next one gathered -- fewer registers, more wavefronts per SIMD; faster wherever at least
+ * four entries are in flight, or two with 8 or more lanes per row.  No counterpart in the reference. */
+int psp_spmm_register_sets(int unroll, int lanes_per_row);
 
 /* SpMM and SDDMM entry points (row-wise walks), blkWarpNum | PSP_BW_STRIPE(rows): this launch deals `rows`
  * consecutive rows (segments, block-rows) to one XCD at a time instead of the library option "xcd_stripe_rows".

@@ -45,6 +45,7 @@ SIGNATURES = {
     "psp_set_option": [ctypes.c_char_p, ctypes.c_longlong],
     "psp_get_option": [ctypes.c_char_p],
     "psp_spmm_plan_for": [_i, _i, _i, ctypes.POINTER(SpmmPlan)],
+    "psp_spmm_register_sets": [_i, _i],
     "psp_split_csr_count": [_vp, _i, _i],
     "psp_split_csr": [_vp, _i, _i, _vp, _vp],
     "psp_split_csr_par": [_vp, _vp, _i, _i, _vp, _vp],
@@ -118,7 +119,7 @@ for _name, _args in SIGNATURES.items():
 lib.psp_last_error.argtypes = []
 lib.psp_last_error.restype = ctypes.c_char_p
 
-ABI_VERSION = 310  # PSP_ABI_VERSION of include/paramsp.h: the struct layouts and buffer sizes this module assumes
+ABI_VERSION = 311  # PSP_ABI_VERSION of include/paramsp.h: the struct layouts and buffer sizes this module assumes
 if lib.psp_version() < ABI_VERSION:
     raise ImportError("%s is version %d, this package needs %d: rebuild it (paramspmm_ae_amd/build_param.sh)"
                       % (LIB_PATH, lib.psp_version(), ABI_VERSION))

@@ -151,6 +151,8 @@ PSP_EXPORT int psp_spmm_plan_for(int N, int CF, int blkWarpNum, psp_spmm_plan *p
     return PSP_OK;
 }
 
+PSP_EXPORT int psp_spmm_register_sets(int unroll, int lanes_per_row) { return psp_spmm_single_set(unroll, lanes_per_row) ? 1 : 2; }
+
 // ------------------------------------------------------------------------------------------------
 // zero fill
 // ------------------------------------------------------------------------------------------------

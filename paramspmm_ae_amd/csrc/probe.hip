@@ -2,8 +2,8 @@
 // an SpMM and loads the same X row tiles (lane groups of 2^logL lanes, one float4 per lane, column tiles in
 // grid.y), but has no rows: no row pointer, no multiplications, no row stores -- every lane only adds what it
 // loads and stores one float4 when its wavefront is done.  Its time is what the memory system needs for the
-// gathers alone, with the loads of the next batch in flight while a batch is added; an SpMM on the same pattern
-// cannot be faster.
+// gathers alone, U loads in flight per lane (bench.py tries U = 4 and 8 with several wavefront shares and keeps the
+// fastest); an SpMM that walks the same pattern the same way cannot be faster.
 #include "psp_common.h"
 
 typedef float psp_f32x4 __attribute__((ext_vector_type(4)));

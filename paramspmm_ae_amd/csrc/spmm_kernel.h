@@ -104,7 +104,8 @@ __device__ __forceinline__ float psp_bperm_f(int src_lane, float v)
 // most registers and where every lane group of the wavefront waits for the slowest -- the mask took the most used
 // configuration from five to four wavefronts per SIMD and made the product 25-45 % slower on the community-ordered
 // graph (341 against 243 us at N = 32, 1018 against 703 at N = 128; the separate pass costs 66 and 256 us).
-template <int C, int V, int U, int NR, bool SPLIT, bool SM, bool ACT = false>
+// SINGLE: one register set instead of two (the walk below).
+template <int C, int V, int U, int NR, bool SPLIT, bool SM, bool ACT = false, bool SINGLE = false>
 __global__ void __launch_bounds__(512)
 psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
                 const int *__restrict__ target_row, const float *__restrict__ X, float *__restrict__ Y,
@@ -369,6 +370,13 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     // loads at the same time (nothing before them depends on the row lengths), and only the short row-closing
     // part diverges between groups.  Entries past the group's range (last, partial batch) are loaded from a valid
     // address but never added, so values of other rows cannot leak in.
+    // SINGLE: one register set -- gather a batch, add it, gather the next.  What the second set buys is small: the
+    // wait in front of a batch's additions is placed for the path on which the next gather was skipped, so behind a
+    // gather that was issued it also covers that gather's loads, and a wavefront has one batch in flight beyond the one
+    // it waits for only while it issues.  The registers of the second set cost more: without it the kernel with four
+    // entries in flight keeps 7 wavefronts per SIMD instead of 5, and is 15-20 % faster on graphs whose gathers mostly
+    // hit (block model, stencil), 2-8 % on the R-MAT graph.  With one entry in flight, or lane groups of 2 or 4 lanes
+    // with two, the second set still pays (psp_spmm_single_set).
     int pos = a;      // first entry of the next batch to gather
     int cbase = a;    // first entry of the chunk c_cur / v_cur hold (lane `sub` holds entries cbase + sub*U ..)
     int jb = 0;       // batch of that chunk the next gather takes: the one lane `jb` of the group holds
@@ -434,7 +442,15 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         }                                                                                              \
     }
 
-    if (busy) {
+    if constexpr (SINGLE) {
+        if (busy) {
+            PSP_DECLARE(A)
+            do {
+                PSP_GATHER(A)
+                PSP_CONSUME(A)
+            } while (pos < b);
+        }
+    } else if (busy) {
         PSP_DECLARE(A)
         PSP_DECLARE(B)
         PSP_GATHER(A)
@@ -529,29 +545,46 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
 typedef void (*psp_spmm_kernel_t)(const int *, const int *, const float *, const int *, const float *, float *,
                                   int, int, int, int, int, int, int, const float *, float *, int);
 
+// One register set or two (template parameter SINGLE)?  Measured on the block model, the stencil and the R-MAT graph at
+// N = 16 ... 256, all layouts: four or more entries in flight -- one set, everywhere (-8 ... -25 %; these kernels always
+// have lane groups of at least four lanes); two entries -- one set from 8 lanes per row on (-0 ... -13 %; +2 ... +20 %
+// with 2 or 4 lanes); one entry in flight -- two sets (one set: +2 ... +31 %).
+static inline bool psp_spmm_single_set(int U, int lanes_per_row) { return U >= 4 || (U == 2 && lanes_per_row >= 8); }
+
+// only the variants psp_spmm_single_set can ask for are instantiated
+template <int C, int V, int U, int NR, bool SPLIT, bool SM, bool ACT>
+static psp_spmm_kernel_t psp_spmm_pick(bool single)
+{
+    if constexpr (U >= 4) return psp_spmm_kernel<C, V, U, NR, SPLIT, SM, ACT, true>;
+    else if constexpr (U == 2)
+        return single ? psp_spmm_kernel<C, V, U, NR, SPLIT, SM, ACT, true> : psp_spmm_kernel<C, V, U, NR, SPLIT, SM, ACT, false>;
+    else return psp_spmm_kernel<C, V, U, NR, SPLIT, SM, ACT, false>;
+}
+
 // softmax-weighted variants exist for CSR layouts, float4 columns and up to 4 vectors per lane
 template <int NR, bool SPLIT>
-static psp_spmm_kernel_t psp_spmm_lookup(int C, int V, int U, bool softmax, bool act = false)
+static psp_spmm_kernel_t psp_spmm_lookup(int C, int V, int U, int lanes_per_row, bool softmax, bool act = false)
 {
+    const bool single = psp_spmm_single_set(U, lanes_per_row);
 #define PSP_CASE(C_, U_)                                                        \
     if (C == C_ && U == U_) {                                                   \
         if (act) {                                                              \
             if constexpr (NR <= 2) {                                            \
-                if (V == 4) return psp_spmm_kernel<C_, 4, U_, NR, SPLIT, false, true>; \
-                if (V == 2) return psp_spmm_kernel<C_, 2, U_, NR, SPLIT, false, true>; \
-                return psp_spmm_kernel<C_, 1, U_, NR, SPLIT, false, true>;      \
+                if (V == 4) return psp_spmm_pick<C_, 4, U_, NR, SPLIT, false, true>(single); \
+                if (V == 2) return psp_spmm_pick<C_, 2, U_, NR, SPLIT, false, true>(single); \
+                return psp_spmm_pick<C_, 1, U_, NR, SPLIT, false, true>(single); \
             }                                                                   \
             return nullptr;                                                     \
         }                                                                       \
         if (softmax) {                                                          \
             if constexpr (NR == 1 && C_ <= 4) {                                 \
-                if (V == 4) return psp_spmm_kernel<C_, 4, U_, 1, SPLIT, true>;  \
+                if (V == 4) return psp_spmm_pick<C_, 4, U_, 1, SPLIT, true, false>(single); \
             }                                                                   \
             return nullptr;                                                     \
         }                                                                       \
-        if (V == 4) return psp_spmm_kernel<C_, 4, U_, NR, SPLIT, false>;        \
-        if (V == 2) return psp_spmm_kernel<C_, 2, U_, NR, SPLIT, false>;        \
-        return psp_spmm_kernel<C_, 1, U_, NR, SPLIT, false>;                    \
+        if (V == 4) return psp_spmm_pick<C_, 4, U_, NR, SPLIT, false, false>(single); \
+        if (V == 2) return psp_spmm_pick<C_, 2, U_, NR, SPLIT, false, false>(single); \
+        return psp_spmm_pick<C_, 1, U_, NR, SPLIT, false, false>(single);       \
     }
     PSP_SPMM_FOR_EACH_CU(PSP_CASE)
 #undef PSP_CASE

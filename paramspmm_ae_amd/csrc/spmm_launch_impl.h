@@ -67,7 +67,7 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     }
 
     const int segs_per_block = plan.waves_per_block << logW;
-    psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll, softmax, relu_x != 0);
+    psp_spmm_kernel_t k = psp_spmm_lookup<NR, SPLIT>(plan.coarsen, plan.vec, plan.unroll, plan.lanes_per_row, softmax, relu_x != 0);
     if (!k)
         return psp_fail(PSP_ERR_ARG, "spmm%s: no kernel for coarsen %d vec %d unroll %d%s", softmax ? " softmax" : "", plan.coarsen,
                         plan.vec, plan.unroll, softmax ? " (needs N % 4 == 0 and CF <= 4)" : "");

@@ -52,6 +52,10 @@ def test_spmm_plan_mapping():
             p["even_split"]) == (2, 16, 4, 2, 1, 5, 1)
     assert _capi.spmm_plan(16, _capi.pack_cf(4, 8, 2), 4)["coarsen"] == 4
     assert _capi.spmm_plan(8, _capi.pack_cf(4, 8, 2), 4)["coarsen"] == 2
+    # one register set from four entries in flight on, or two entries with 8 lanes per row or more; two sets otherwise
+    sets = _capi.lib.psp_spmm_register_sets
+    assert [sets(u, l) for u, l in ((4, 4), (4, 8), (8, 8), (2, 8), (2, 64))] == [1] * 5
+    assert [sets(u, l) for u, l in ((2, 2), (2, 4), (1, 1), (1, 8), (1, 64))] == [2] * 5
     # per-launch XCD stripe in the flag bits of blkWarpNum
     assert _capi.spmm_plan(64, 1, 4)["xcd_stripe_rows"] == 0
     for rows in (256, 768, 6144, 65280):
