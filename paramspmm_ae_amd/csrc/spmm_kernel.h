@@ -15,10 +15,11 @@
 //   * colIdx / values are read once per L*U entries: lane s of a group takes the U consecutive entries
 //     base + s*U .. in one 4U-byte load per array (a group reads whole 128-byte lines), the pairs are handed
 //     round the group with ds_bpermute, and the next L*U are prefetched while the current ones are consumed;
-//   * the walk is software-pipelined over batches of U entries, whatever rows they belong to: the U*C
-//     feature loads of batch t+1 are issued before batch t is added (two register sets alternate), so every
-//     lane group issues the same loads at the same time and only the closing of a row -- a store where a row
-//     ends -- diverges between groups;
+//   * the walk goes over batches of U entries, whatever rows they belong to, so every lane group issues the
+//     same U*C feature loads at the same time and only the closing of a row -- a store where a row ends --
+//     diverges between groups.  With two register sets (SINGLE = false) the loads of batch t+1 are issued
+//     before batch t is added; with one set (SINGLE = true) a batch is gathered, added, and the next one
+//     gathered, which frees registers for more wavefronts per SIMD (psp_spmm_single_set picks);
 //   * a row cut by a group boundary is summed across the groups in registers (ds_bpermute), in group order,
 //     so plain CSR needs neither atomics nor a cleared Y.  Only a row whose segments lie in several
 //     wavefronts (row-split formats) is accumulated with fp32 atomics, once per wavefront.
