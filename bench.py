@@ -810,7 +810,7 @@ def main():
             by_symbol.setdefault(sym, []).append(r)
             continue
         plan = _capi.spmm_plan(r["dim"], r["CF"], r["blkWarpNum"])
-        one_set = _capi.lib.psp_spmm_register_sets(plan["unroll"], plan["lanes_per_row"]) == 1
+        one_set = plan["register_sets"] == 1
         sym = "psp_spmm_kernel<%d, %d, %d, %d, %s, false, false, %s>" % (plan["coarsen"], plan["vec"], plan["unroll"],
                                                            2 if r["format"].startswith("bcsr") else 1,
                                                            "true" if "split" in r["format"] else "false",

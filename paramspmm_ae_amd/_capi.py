@@ -185,7 +185,9 @@ def get_option(name):
 def spmm_plan(N, CF, blkWarpNum):
     p = SpmmPlan()
     check(lib.psp_spmm_plan_for(N, CF, blkWarpNum, ctypes.byref(p)))
-    return p.as_dict()
+    d = p.as_dict()
+    d["register_sets"] = lib.psp_spmm_register_sets(p.unroll, p.lanes_per_row)  # which kernel variant the plan launches
+    return d
 
 
 def ptr(t):

@@ -331,6 +331,7 @@ static py::dict spmm_plan(int N, int CF, int blkWarpNum)
     d["log_segs_per_wave"] = p.log_segs_per_wave;
     d["even_split"] = p.even_split;
     d["xcd_stripe_rows"] = p.xcd_stripe_rows;
+    d["register_sets"] = psp_spmm_register_sets(p.unroll, p.lanes_per_row);  // which kernel variant the plan launches
     return d;
 }
 

@@ -56,6 +56,7 @@ def test_spmm_plan_mapping():
     sets = _capi.lib.psp_spmm_register_sets
     assert [sets(u, l) for u, l in ((4, 4), (4, 8), (8, 8), (2, 8), (2, 64))] == [1] * 5
     assert [sets(u, l) for u, l in ((2, 2), (2, 4), (1, 1), (1, 8), (1, 64))] == [2] * 5
+    assert _capi.spmm_plan(16, 1, 4)["register_sets"] == 1 and _capi.spmm_plan(256, 8, 4)["register_sets"] == 2
     # per-launch XCD stripe in the flag bits of blkWarpNum
     assert _capi.spmm_plan(64, 1, 4)["xcd_stripe_rows"] == 0
     for rows in (256, 768, 6144, 65280):
@@ -321,6 +322,11 @@ def test_extension_modules_export_the_reference_binding_names():
     for mod, names in ((ParamSpMM, spmm), (ParamSDDMM, sddmm), (ParamSpCONV, conv)):
         for n in names:
             assert callable(getattr(mod, n)), (mod.__name__, n)
+    # the module reports a launch plan as the C ABI does
+    from paramspmm_ae_amd import _capi
+
+    for args in ((16, 1, 4), (128, 4, 8), (256, 8, 4), (96, _capi.pack_cf(2, 8, 2), 4)):
+        assert dict(ParamSpMM.spmm_plan(*args)) == _capi.spmm_plan(*args)
     # device entry points refuse CPU tensors instead of falling back
     x = torch.zeros(4, 16)
     rp = torch.zeros(5, dtype=torch.int32)
