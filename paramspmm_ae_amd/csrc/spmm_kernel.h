@@ -111,13 +111,24 @@ __global__ void __launch_bounds__(512)
 psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, const float *__restrict__ val,
                 const int *__restrict__ target_row, const float *__restrict__ X, float *__restrict__ Y,
                 int nseg, int N, int logL, int logW, int tiles, int stripe, int align_pct,
-                const float *__restrict__ row_max, float *__restrict__ row_sum, int relu_x)
+                const float *__restrict__ row_max, float *__restrict__ row_sum, int relu_x, int tail_rows)
 {
     static_assert(!SM || NR == 1, "softmax weights exist for the CSR layouts only");
     static_assert(!(SM && ACT), "the softmax-weighted product takes no activation argument");
     typedef typename psp_vec<V>::type vec_t;
     __shared__ int2 s_seg[PSP_MAX_WAVES][PSP_WAVE];  // (end offset, output row) of the wavefront's segments
     __shared__ float s_m[SM ? PSP_MAX_WAVES : 1][SM ? PSP_WAVE : 1];  // SM: reference maximum of each segment's row
+
+    // tail_rows: the few rows Y has past the matrix's own (a feature matrix padded to an even row count): the first
+    // wavefront of the launch writes their zeros, one column tile per blockIdx.y, instead of a launch of its own -- on
+    // a matrix of 10^5 entries that launch and the gap behind it took as long as the product
+    if (!SPLIT && tail_rows > 0 && blockIdx.x == 0 && threadIdx.x < PSP_WAVE) {
+        const int tile_w = (C * V) << logL;
+        const int col0 = blockIdx.y * tile_w;
+        const int w = min(tile_w, N - col0);
+        float *yt = Y + (size_t)nseg * NR * (size_t)N + col0;
+        for (int i = threadIdx.x; i < tail_rows * w; i += PSP_WAVE) yt[(size_t)(i / w) * (size_t)N + i % w] = 0.0f;
+    }
 
     const int tile = psp_xcd_tile(stripe);
     if (tile >= tiles) return;
@@ -544,7 +555,8 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
     M_(5, 1) M_(6, 1) M_(7, 1) M_(8, 1)
 
 typedef void (*psp_spmm_kernel_t)(const int *, const int *, const float *, const int *, const float *, float *,
-                                  int, int, int, int, int, int, int, const float *, float *, int);
+                                  int, int, int, int, int, int, int, const float *, float *, int, int);
+#define PSP_SPMM_TAIL_ROWS_MAX 16  // more rows than this past the matrix are cleared by a fill launch
 
 // One register set or two (template parameter SINGLE)?  Measured on the block model, the stencil and the R-MAT graph at
 // N = 16 ... 256, all layouts: four or more entries in flight -- one set, everywhere (-8 ... -25 %; these kernels always

@@ -44,6 +44,7 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     if (opt.whole_rows && logW < logR) logW = logR;
 
     // rows the kernel does not store to must read as zero
+    int tail_rows = 0;
     if (SPLIT) {
         // The kernel stores rows that one wavefront holds alone and adds (atomics) to rows shared by several
         // wavefronts.  Large outputs are therefore not cleared as a whole: a pass over the segments clears only
@@ -53,8 +54,13 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
         else
             rc = psp_zero_f32(Y, (size_t)rows_out * N, stream);
     } else {
+        // rows past the matrix's own: up to PSP_SPMM_TAIL_ROWS_MAX are zeroed by the kernel itself (tail_rows)
         const size_t covered = (size_t)nrows * NR;
-        rc = psp_zero_f32(Y + covered * N, ((size_t)rows_out - covered) * N, stream);
+        tail_rows = (int)std::min<size_t>((size_t)rows_out - covered, (size_t)PSP_SPMM_TAIL_ROWS_MAX + 1);
+        if (tail_rows > PSP_SPMM_TAIL_ROWS_MAX || nrows == 0) {
+            tail_rows = 0;
+            rc = psp_zero_f32(Y + covered * N, ((size_t)rows_out - covered) * N, stream);
+        }
     }
     if (rc != PSP_OK) return rc;
     if (nrows == 0) return PSP_OK;
@@ -76,7 +82,7 @@ int psp_spmm_launch(const int *rowPtr, const int *colIdx, const float *val, cons
     const psp_grid1d g = psp_xcd_grid(psp_ceil_div(nrows, segs_per_block),
                                       (plan.xcd_stripe_rows ? plan.xcd_stripe_rows : opt.stripe_rows) / segs_per_block);
     dim3 grid(g.launch, plan.col_tiles, 1), block(plan.waves_per_block * PSP_WAVE, 1, 1);
-    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.stripe, align_pct, row_max, row_sum, relu_x);
+    hipLaunchKernelGGL(k, grid, block, 0, stream, rowPtr, colIdx, val, target_row, X, Y, nrows, N, logL, logW, g.real, g.stripe, align_pct, row_max, row_sum, relu_x, tail_rows);
     rc = psp_check_launch("spmm kernel");
     if (rc != PSP_OK || !(softmax && SPLIT)) return rc;
     return psp_row_scale(Y, row_sum, rows_out, N, stream);  // rows that several wavefronts added to

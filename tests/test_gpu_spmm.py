@@ -55,6 +55,36 @@ def test_spmm_odd_widths(oracle, small, fmt, N):
         assert_close(got, want, what="%s N=%d CF=%d" % (fmt, N, CF), scale=scale)
 
 
+@pytest.mark.parametrize("fmt", ["csr", "bcsr"])
+@pytest.mark.parametrize("N", [16, 48, 160, 513])
+def test_spmm_rows_past_the_matrix_read_zero(oracle, small, fmt, N):
+    """Y may have more rows than the matrix (a padded feature matrix): they come back as zeros whether the kernel
+    writes them itself (up to 16 rows) or a fill launch does, and the matrix's own rows are what they are without."""
+    from gpu_util import spmm_oracle, spmm_abs_scale, assert_close, stream
+    from paramspmm_ae_amd import _capi
+
+    F = small
+    L, p, d = _capi.lib, _capi.ptr, F.d
+    X = np.random.default_rng(N).standard_normal((F.n + (F.n & 1), N)).astype(np.float32)
+    want = spmm_oracle(oracle, fmt, F, X)
+    covered = F.n if fmt == "csr" else 2 * (F.rpb.size - 1)
+    scale = spmm_abs_scale(oracle, F, X, want.shape[0])
+    Xd = torch.from_numpy(X).cuda()
+    for tail in (0, 1, 3, 16, 17, 40):
+        for CF, bw in ((1, 4), (2, 8), (8, 4)):
+            print("case", fmt, N, tail, CF, bw, flush=True)
+            Y = torch.full((covered + tail + 2, N), float("nan"), device="cuda")  # two guard rows behind rows_out
+            if fmt == "csr":
+                rc = L.psp_spmm_csr_f32(p(d["rowPtr"]), p(d["colIdx"]), p(d["val"]), p(Xd), p(Y), F.n, N, covered + tail, CF, bw, stream())
+            else:
+                rc = L.psp_spmm_bcsr_f32(p(d["rpb"]), p(d["cib"]), p(d["vb"]), p(Xd), p(Y), F.rpb.size - 1, N, covered + tail, CF, bw, stream())
+            _capi.check(rc)
+            torch.cuda.synchronize()
+            assert_close(Y[:covered], want[:covered], what="%s N=%d tail=%d CF=%d" % (fmt, N, tail, CF), scale=scale[:covered])
+            assert torch.count_nonzero(Y[covered:covered + tail]).item() == 0 and not torch.isnan(Y[covered:covered + tail]).any()
+            assert torch.isnan(Y[covered + tail:]).all(), "rows behind rows_out were touched"
+
+
 @pytest.mark.parametrize("fmt", FMTS)
 def test_spmm_ones_gives_row_sums(oracle, small, fmt):
     """The reference's own known answer: X = ones -> every column holds the row sums (verification.py:26,43)."""
