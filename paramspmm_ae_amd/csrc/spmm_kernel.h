@@ -375,13 +375,13 @@ psp_spmm_kernel(const int *__restrict__ rowPtr, const int *__restrict__ colIdx, 
         }
     };
 
-    // The walk is software-pipelined over batches of U entries, whatever rows they belong to.  GATHER takes the
-    // next U (column, value) pairs of the group from the lanes that hold them and issues the feature loads;
-    // CONSUME adds a batch entry by entry and closes a row where one ends.  Two register sets alternate, so the
-    // loads of batch t+1 are in flight while batch t is added: every lane group of the wavefront issues the same
-    // loads at the same time (nothing before them depends on the row lengths), and only the short row-closing
-    // part diverges between groups.  Entries past the group's range (last, partial batch) are loaded from a valid
-    // address but never added, so values of other rows cannot leak in.
+    // The walk goes over batches of U entries, whatever rows they belong to.  GATHER takes the next U (column, value)
+    // pairs of the group from the lanes that hold them and issues the feature loads; CONSUME adds a batch entry by
+    // entry and closes a row where one ends.  Every lane group of the wavefront issues the same loads at the same time
+    // (nothing before them depends on the row lengths), and only the short row-closing part diverges between groups.
+    // Entries past the group's range (last, partial batch) are loaded from a valid address but never added, so values
+    // of other rows cannot leak in.
+    // !SINGLE: two register sets alternate, the loads of batch t+1 are issued before batch t is added.
     // SINGLE: one register set -- gather a batch, add it, gather the next.  What the second set buys is small: the
     // wait in front of a batch's additions is placed for the path on which the next gather was skipped, so behind a
     // gather that was issued it also covers that gather's loads, and a wavefront has one batch in flight beyond the one
